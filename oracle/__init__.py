@@ -1,0 +1,1 @@
+"""CPU oracles (test infrastructure only; the product never imports this package)."""

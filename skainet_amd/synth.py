@@ -1,0 +1,104 @@
+"""Seeded synthetic GGUF block data of the benchmark shapes (NumPy, host side).
+
+Every harness (tests, smoke, bench) draws its inputs from here so that the CPU oracle and the
+GPU library always see identical bytes.  Layouts follow the ggml block definitions whose sizes
+the reference tabulates in gguf/src/commonMain/kotlin/sk/ai/net/gguf/Constants.kt:58-90.
+
+  Q8_0  34 B : f16 d = |N(0,1)|*0.02, 32 x int8 uniform in [-127, 127]
+  Q4_K 144 B : f16 d = |N(0,1)|*0.01, f16 dmin = |N(0,1)|*0.005,
+               12 bytes packing eight 6-bit scales and eight 6-bit mins (uniform 0..63),
+               128 bytes of 4-bit quants (uniform 0..15)
+  Q6_K 210 B : 128 B low nibbles + 64 B high 2-bit pairs (6-bit quants uniform 0..63),
+               16 x int8 scales uniform in [-32, 31], f16 d = |N(0,1)|*0.01
+"""
+from __future__ import annotations
+
+import numpy as np
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+
+
+def _f16_bytes(values):
+    return np.ascontiguousarray(values.astype(np.float16)).view(np.uint8).reshape(-1, 2)
+
+
+def pack_q4k_scales(sc, m):
+    """[nb,8] 6-bit scales and mins -> [nb,12] packed bytes (inverse of the ggml 6-bit unpack)."""
+    sc = sc.astype(np.uint8)
+    m = m.astype(np.uint8)
+    out = np.empty(sc.shape[:-1] + (12,), dtype=np.uint8)
+    out[..., 0:4] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
+    out[..., 4:8] = (m[..., 0:4] & 63) | ((m[..., 4:8] >> 4) << 6)
+    out[..., 8:12] = (sc[..., 4:8] & 0x0F) | ((m[..., 4:8] & 0x0F) << 4)
+    return out
+
+
+def q8_0_blocks(n_blocks, rng):
+    b = np.empty((n_blocks, 34), dtype=np.uint8)
+    b[:, 0:2] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.02)
+    b[:, 2:34] = rng.integers(-127, 128, size=(n_blocks, 32), dtype=np.int8).view(np.uint8)
+    return b.reshape(-1)
+
+
+def q4_k_blocks(n_blocks, rng):
+    b = np.empty((n_blocks, 144), dtype=np.uint8)
+    b[:, 0:2] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.01)
+    b[:, 2:4] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.005)
+    sc = rng.integers(0, 64, size=(n_blocks, 8), dtype=np.uint8)
+    m = rng.integers(0, 64, size=(n_blocks, 8), dtype=np.uint8)
+    b[:, 4:16] = pack_q4k_scales(sc, m)
+    # two independent uniform nibbles per byte == one uniform byte
+    b[:, 16:144] = rng.integers(0, 256, size=(n_blocks, 128), dtype=np.uint8)
+    return b.reshape(-1)
+
+
+def q6_k_blocks(n_blocks, rng):
+    b = np.empty((n_blocks, 210), dtype=np.uint8)
+    # 6-bit quants uniform 0..63 == uniform low nibble and uniform high 2 bits == uniform bytes
+    b[:, 0:192] = rng.integers(0, 256, size=(n_blocks, 192), dtype=np.uint8)
+    b[:, 192:208] = rng.integers(-32, 32, size=(n_blocks, 16), dtype=np.int8).view(np.uint8)
+    b[:, 208:210] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.01)
+    return b.reshape(-1)
+
+
+_GEN = {Q8_0: q8_0_blocks, Q4_K: q4_k_blocks, Q6_K: q6_k_blocks}
+
+
+def weight(qtype, n_rows, k, seed):
+    """Raw block bytes of an [n_rows, k] weight ([out, in], rows contiguous), as uint8."""
+    elems, _ = BLOCK[qtype]
+    if k % elems:
+        raise ValueError(f"row size {k} is not a multiple of the block size {elems}")
+    rng = np.random.default_rng(seed)
+    return _GEN[qtype](n_rows * (k // elems), rng)
+
+
+def activation_f32(n, seed):
+    return np.random.default_rng(seed).standard_normal(n, dtype=np.float32)
+
+
+def f32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def activation_bf16(shape, seed):
+    x = np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+    return f32_to_bf16_bits(x)
+
+
+def kv_f16(shape, seed):
+    """fp16 bit patterns of N(0,1) draws."""
+    x = np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+    return x.astype(np.float16).view(np.uint16)
+
+
+def checksum(arr):
+    """FNV-1a 64 over a strided sample of the bytes plus the length: recorded beside bench results."""
+    a = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+    step = max(1, a.size // 65536)
+    h = 0xCBF29CE484222325
+    for byte in a[::step].tolist():
+        h = ((h ^ byte) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return f"{h:016x}:{a.size}"
