@@ -1,0 +1,245 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Q4_K batch-1 matvec 4096 x 11008 on one MI355X, effective HBM GB/s.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A step is one matvec  y = deq(W) . x  through the C ABI (skn_matvec_q) on device-resident inputs.  The
+weight of step i is copy i mod 24 of 24 distinct seeded 25.4 MB tensors (609 MB in all), so that no step
+finds its weights in the 256 MB last-level cache: the figure is an HBM figure.
+
+Output: ONE JSON line.
+  value            algorithmic bytes of K steps / wall time of K steps (launch gaps included), GB/s
+  roofline         algorithmic bytes of one launch / mean kernel duration (per-launch HIP events on the
+                   stream the kernel runs on), against the 8 TB/s HBM peak
+  cpu_baseline     the CPU oracle (C, OpenMP) on the same workload, timed on this box's host cores
+  extra            the other benchmark shapes, cache-hot figures, attention and decode throughput
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from skainet_amd import runtime, synth  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+N_COPIES = 24
+
+
+def matvec_bytes(qtype, n, k):
+    be, bb = synth.BLOCK[qtype]
+    return n * (k // be) * bb + 4 * k + 4 * n
+
+
+def bench_matvec(ctx, qtype, n, k, steps, warmup, copies=N_COPIES, seed=1234):
+    """-> dict with wall and per-kernel timing of `steps` matvecs rotating over `copies` weight tensors."""
+    be, bb = synth.BLOCK[qtype]
+    w_bytes = n * (k // be) * bb
+    weights = []
+    sums = []
+    for c in range(copies):
+        raw = synth.weight(qtype, n, k, seed=seed + c)
+        if c == 0:
+            sums.append(synth.checksum(raw))
+        weights.append(ctx.to_device(raw))
+    x = ctx.to_device(synth.activation_f32(k, seed=seed + 999))
+    y = ctx.alloc(4 * n)
+    for i in range(warmup):
+        ctx.matvec_q(qtype, weights[i % copies], n, k, x, y)
+    ctx.sync()
+    # (1) wall clock over exactly `steps` steps, synchronised on both sides
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ctx.matvec_q(qtype, weights[i % copies], n, k, x, y)
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    # (2) the same steps again with per-launch start/stop events: kernel durations without launch gaps
+    ctx.prof_start(steps)
+    for i in range(steps):
+        ctx.matvec_q(qtype, weights[i % copies], n, k, x, y)
+    kernel_ms, launches = ctx.prof_stop()
+    # (3) cache-hot: one weight copy only
+    hot_steps = min(steps, 200)
+    ctx.prof_start(hot_steps)
+    for i in range(hot_steps):
+        ctx.matvec_q(qtype, weights[0], n, k, x, y)
+    hot_ms, hot_n = ctx.prof_stop()
+    nbytes = matvec_bytes(qtype, n, k)
+    res = {
+        "bytes_per_launch": nbytes,
+        "wall_s": wall,
+        "ms_per_step": wall / steps * 1e3,
+        "wall_gbs": nbytes * steps / wall / 1e9,
+        "kernel_us": kernel_ms / launches * 1e3,
+        "kernel_gbs": nbytes / (kernel_ms / launches * 1e-3) / 1e9,
+        "hot_kernel_us": hot_ms / hot_n * 1e3,
+        "hot_kernel_gbs": nbytes / (hot_ms / hot_n * 1e-3) / 1e9,
+        "weight_bytes": w_bytes,
+        "copies": copies,
+        "checksum_copy0": sums[0],
+    }
+    for wbuf in weights:
+        wbuf.free()
+    x.free()
+    y.free()
+    return res
+
+
+def bench_attention(ctx, steps, warmup):
+    """8 sequences x 32 heads x 128 dims, 256-token pages: append one token per sequence, attend over 4096."""
+    n_seq, n_head, dim, n_ctx = 8, 32, 128, 4096
+    kv = ctx.kv_cache(n_seq, n_head, dim, 256, 8192)
+    for s in range(n_seq):
+        k = ctx.to_device(synth.kv_f16((n_ctx - 1, n_head, dim), seed=50 + s))
+        v = ctx.to_device(synth.kv_f16((n_ctx - 1, n_head, dim), seed=70 + s))
+        kv.append_run(s, k, v, n_ctx - 1)
+        k.free()
+        v.free()
+    k1 = ctx.to_device(synth.kv_f16((n_seq, n_head, dim), seed=90))
+    v1 = ctx.to_device(synth.kv_f16((n_seq, n_head, dim), seed=91))
+    q = ctx.to_device(np.random.default_rng(92).standard_normal((n_seq, n_head, dim)).astype(np.float32))
+    out = ctx.alloc(4 * n_seq * n_head * dim)
+    kv.append(k1, v1, list(range(n_seq)))
+    scale = 1.0 / np.sqrt(dim)
+    lens = [n_ctx] * n_seq
+    for _ in range(warmup):
+        kv.attn_decode(q, out, scale, n_ctx=lens)
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        kv.attn_decode(q, out, scale, n_ctx=lens)
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    ctx.prof_start(4 * steps)
+    for _ in range(steps):
+        kv.attn_decode(q, out, scale, n_ctx=lens)
+    kernel_ms, launches = ctx.prof_stop()
+    nbytes = n_seq * n_head * n_ctx * dim * 2 * 2 + 2 * 4 * n_seq * n_head * dim
+    kv.free()
+    per_step_us = kernel_ms / steps * 1e3
+    return {
+        "bytes_per_step": nbytes,
+        "kernel_us_per_step": per_step_us,
+        "kernel_gbs": nbytes / (per_step_us * 1e-6) / 1e9,
+        "frac_hbm_peak": nbytes / (per_step_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+        "wall_us_per_step": wall / steps * 1e6,
+        "launches_per_step": launches / steps,
+    }
+
+
+def cpu_baseline(qtype, n, k, budget_s=12.0):
+    """The CPU oracle (C, OpenMP over rows) on the headline workload; a bounded number of repetitions."""
+    from oracle import oracle_c  # the checker, timed as the "port" CPU baseline -- never the product path
+
+    raw = synth.weight(qtype, n, k, seed=1234)
+    x = synth.activation_f32(k, seed=2233)
+    cores = oracle_c.num_threads()
+    oracle_c.matvec_q(qtype, raw, n, k, x)  # warm
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        oracle_c.matvec_q(qtype, raw, n, k, x)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or reps >= 400:
+            break
+    per = dt / reps
+    # the reference's own algorithm for such a weight (dequantize to fp64, transpose, i-outer loop), one thread
+    t1 = time.perf_counter()
+    oracle_c.matvec_q(qtype, raw, n, k, x, reference_algorithm=True)
+    ref_alg = time.perf_counter() - t1
+    nbytes = matvec_bytes(qtype, n, k)
+    return {
+        "value": nbytes / per / 1e9,
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{reps} repetitions of the full Q4_K {n}x{k} matvec ({dt:.1f} s), fp64 accumulation, OpenMP over rows",
+        "ms_per_matvec": per * 1e3,
+        "reference_algorithm_1thread_ms": ref_alg * 1e3,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    ctx = runtime.Context(0)
+    info = ctx.device_info()
+    n, k = 4096, 11008
+    head = bench_matvec(ctx, Q4_K, n, k, args.steps, args.warmup)
+
+    extra = {"device": info["name"], "compute_units": info["compute_units"]}
+    if not args.no_extra:
+        es, ew = min(args.steps, 600), min(args.warmup, 50)
+        shapes = [("q4_k_4096x4096", Q4_K, 4096, 4096, 64), ("q4_k_11008x4096", Q4_K, 11008, 4096, 24),
+                  ("q8_0_4096x4096", Q8_0, 4096, 4096, 32), ("q6_k_4096x4096", Q6_K, 4096, 4096, 40)]
+        for name, qt, nn, kk, copies in shapes:
+            r = bench_matvec(ctx, qt, nn, kk, es, ew, copies=copies, seed=4000 + nn + kk + qt)
+            extra[name] = {key: (round(r[key], 3) if isinstance(r[key], float) else r[key])
+                           for key in ("kernel_us", "kernel_gbs", "hot_kernel_us", "hot_kernel_gbs", "wall_gbs")}
+            extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
+        att = bench_attention(ctx, min(args.steps, 200), 10)
+        extra["attention_8x32x128_ctx4096"] = {key: round(val, 4) for key, val in att.items()}
+        try:
+            from skainet_amd import llama_bench
+            extra["decode_7b_q4_k"] = llama_bench.run(ctx)
+        except Exception as e:  # the decoder leg reports its own absence instead of failing the headline
+            extra["decode_7b_q4_k"] = {"error": f"{type(e).__name__}: {e}"}
+
+    out = {
+        "metric": "Q4_K matvec effective HBM GB/s (% peak); decode tok/s, 7B-shape Q4_K",
+        "value": round(head["wall_gbs"], 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "q4_k x f32 -> f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Q4_K matvec batch 1, N=4096 K=11008 (BASELINE configs[1])",
+            "weight_copies_rotated": head["copies"],
+            "weight_bytes": head["weight_bytes"],
+            "algorithmic_bytes_per_step": head["bytes_per_launch"],
+            "weight_checksum_copy0": head["checksum_copy0"],
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(head["kernel_gbs"], 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(head["kernel_gbs"] / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "matvec_q4k_kernel",
+            "kernel_us": round(head["kernel_us"], 3),
+            "cache_hot_gbs": round(head["hot_kernel_gbs"], 2),
+        },
+        "extra": extra,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(Q4_K, n, k)
+    ctx.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

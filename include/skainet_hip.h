@@ -1,0 +1,203 @@
+/*
+ * libskainet_hip -- C ABI of the MI355X (gfx950) quantized-inference hot path for sk-ai-net/skainet.
+ *
+ * The reference has no native boundary of its own (it is pure Kotlin); these entry points are what a
+ * Kotlin/Native cinterop .def or a JVM Panama FFM binding would bind so that a device-backed tensor can
+ * sit behind the reference's existing seams.  Each declaration cites the reference interface it serves.
+ *
+ * Conventions
+ *   - Every function returns SKN_OK (0) or a negative SKN_ERR_* code; nothing throws or aborts across the
+ *     boundary.  skn_last_error() gives the message of the last failure on that context.
+ *   - `dev` pointers are device addresses (from skn_malloc, or any HIP allocation of the same process);
+ *     `host` pointers are ordinary host memory borrowed for the duration of the call.
+ *   - ggml type ids are the reference's GGMLQuantizationType values
+ *     (gguf/src/commonMain/kotlin/sk/ai/net/gguf/Constants.kt:14-46): F32 0, F16 1, Q8_0 8, Q4_K 12, Q6_K 14.
+ *   - Weights are [n, k] = [out, in] as in the reference's Linear (core/.../nn/Linear.kt:26-28): n rows, each
+ *     k / block consecutive GGUF blocks, rows contiguous -- exactly the bytes GGUFReader hands out for a
+ *     quantized tensor (gguf/.../GGUFReader.kt:354-373).
+ *   - One HIP stream per context; compute calls are asynchronous on it; skn_sync / skn_download wait.
+ *     Calls on one context must be serialised by the caller (the reference is single-threaded throughout).
+ */
+#ifndef SKAINET_HIP_H
+#define SKAINET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SKN_ABI_VERSION 1
+
+#define SKN_OK 0
+#define SKN_ERR_ARG (-1)    /* null pointer, negative size, bad handle */
+#define SKN_ERR_TYPE (-2)   /* ggml type id not on this path */
+#define SKN_ERR_SHAPE (-3)  /* row not a block multiple / operands do not align */
+#define SKN_ERR_OOM (-4)    /* device or host allocation failed */
+#define SKN_ERR_HIP (-5)    /* a HIP runtime call failed */
+#define SKN_ERR_RANGE (-6)  /* sequence id / token range outside the cache */
+#define SKN_ERR_POOL (-7)   /* KV page pool exhausted or sequence full */
+#define SKN_ERR_STATE (-8)  /* call not valid in the current state */
+
+#define SKN_TYPE_F32 0
+#define SKN_TYPE_F16 1
+#define SKN_TYPE_Q8_0 8
+#define SKN_TYPE_Q4_K 12
+#define SKN_TYPE_Q6_K 14
+
+typedef struct skn_ctx skn_ctx;
+typedef struct skn_kv skn_kv;
+typedef struct skn_llama skn_llama;
+
+/* ---- lifetime, errors -------------------------------------------------------------------------- */
+
+int skn_abi_version(void);
+/* Creates a context on HIP device `device` with its own stream.  (No reference counterpart: reference
+ * tensors are garbage-collected host objects; a Kotlin wrapper would be AutoCloseable around this.) */
+int skn_init(int device, skn_ctx** out);
+void skn_shutdown(skn_ctx* ctx);
+/* Message of the last error on `ctx` (or of the last context-less failure when ctx is NULL). */
+const char* skn_last_error(skn_ctx* ctx);
+const char* skn_status_string(int code);
+/* Device facts for reports: name, compute units, total memory. */
+int skn_device_info(skn_ctx* ctx, char* name, size_t name_len, int* compute_units, size_t* total_bytes);
+
+/* ---- format table -------------------------------------------------------------------------------- */
+
+/* GGML_QUANT_SIZES lookup (gguf/.../Constants.kt:58-90): elements and bytes per block. */
+int skn_type_block(int ggml_type, int* block_elems, int* block_bytes);
+/* quantShapeToByteShape on the last axis (gguf/.../Quants.kt:10-20): bytes of a row of k elements, or
+ * SKN_ERR_SHAPE when k is not a block multiple, SKN_ERR_TYPE for an unknown type. */
+int64_t skn_row_bytes(int ggml_type, int64_t k);
+
+/* ---- device memory ------------------------------------------------------------------------------- */
+
+/* Where the bytes of ReaderTensor.data (gguf/.../GGUFReader.kt:35-44,370-395) go to live on the device. */
+int skn_malloc(skn_ctx* ctx, size_t bytes, void** dev);
+int skn_free(skn_ctx* ctx, void* dev);
+int skn_upload(skn_ctx* ctx, void* dev, const void* host, size_t bytes);
+int skn_download(skn_ctx* ctx, void* host, const void* dev, size_t bytes);
+int skn_memset(skn_ctx* ctx, void* dev, int byte_value, size_t bytes);
+int skn_sync(skn_ctx* ctx);
+/* Adopt a caller-owned hipStream_t (NULL restores the context's own stream). */
+int skn_set_stream(skn_ctx* ctx, void* hip_stream);
+/* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
+int skn_timer_start(skn_ctx* ctx);
+int skn_timer_stop(skn_ctx* ctx, float* elapsed_ms);
+/* Per-launch kernel timing: between start and stop each kernel launched on this context carries its own
+ * start/stop HIP events (dispatch begin/end timestamps); stop waits for the stream and returns the summed
+ * kernel durations and the number of launches timed (at most max_launches). */
+int skn_prof_start(skn_ctx* ctx, int max_launches);
+int skn_prof_stop(skn_ctx* ctx, double* kernel_ms_total, int* launches);
+
+/* ---- dequantization ------------------------------------------------------------------------------ */
+
+/* The dequantizer the reference leaves as a TODO (gguf/.../Quants.kt:8): n_elems consecutive elements
+ * (a block multiple) of `ggml_type` at `w_dev` -> fp32 at `out_dev`.  Bit-exact with the ggml formulas. */
+int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64_t n_elems, float* out_dev);
+
+/* ---- quantized matvec / GEMM ---------------------------------------------------------------------- */
+
+/* y[n] = sum_k deq(W)[n,k] * x[k]: Linear.forward's `input.matmul(weight.t())` for a rank-1 input
+ * (core/.../nn/Linear.kt:43-49 -> core/.../impl/DoublesTensor.kt:255-264), without materialising t().
+ * x fp32 [k], y fp32 [n]. */
+int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev, float* y_dev);
+/* C[m,n] = sum_k A[m,k] * deq(W)[n,k]: the rank-2 case (core/.../impl/DoublesTensor.kt:267-279).
+ * A bf16 bits [m,k] row-major, C fp32 [m,n] row-major. */
+int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const uint16_t* a_bf16_dev, int m,
+               float* c_dev);
+
+/* ---- paged KV cache -------------------------------------------------------------------------------- */
+
+/* No reference counterpart (the reference has no sequences or attention).  A cache holds fp16 K and V rows of
+ * n_head * head_dim values per token for n_seq sequences, in device pages of page_tokens tokens drawn on
+ * demand from a pool sized for n_seq * ceil(max_tokens / page_tokens) pages. */
+int skn_kv_create(skn_ctx* ctx, int n_seq, int n_head, int head_dim, int page_tokens, int max_tokens, skn_kv** out);
+int skn_kv_free(skn_ctx* ctx, skn_kv* kv);
+/* Forget the tokens of one sequence (seq >= 0) or of all (seq = -1); pages return to the pool. */
+int skn_kv_reset(skn_ctx* ctx, skn_kv* kv, int seq);
+/* Current token count of a sequence, or a negative error code. */
+int skn_kv_len(skn_ctx* ctx, skn_kv* kv, int seq);
+/* Append one token for each of n listed sequences: k/v fp16 bits [n][n_head][head_dim] on the device,
+ * seq_ids on the host (a sequence may be listed more than once; its tokens land in list order). */
+int skn_kv_append(skn_ctx* ctx, skn_kv* kv, const uint16_t* k_dev, const uint16_t* v_dev, const int32_t* seq_ids_host,
+                  int n);
+/* Append n_tokens consecutive tokens to one sequence: k/v fp16 bits [n_tokens][n_head][head_dim]. */
+int skn_kv_append_run(skn_ctx* ctx, skn_kv* kv, int seq, const uint16_t* k_dev, const uint16_t* v_dev, int n_tokens);
+/* Copy tokens [t0, t1) of a sequence out, token-major [t1-t0][n_head][head_dim] fp16 bits. */
+int skn_kv_gather(skn_ctx* ctx, skn_kv* kv, int seq, int t0, int t1, uint16_t* k_out_dev, uint16_t* v_out_dev);
+
+/* out[s,h,:] = softmax(q[s,h,:] . K[s,0:n,h,:]^T * scale) . V[s,0:n,h,:] for every sequence and head.
+ * q/out fp32 [n_seq][n_head][head_dim] on the device; n_ctx_host[s] = tokens to attend (NULL = all cached). */
+int skn_attn_decode(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* n_ctx_host, float scale,
+                    float* out_dev);
+
+/* ---- decoder glue (fp32, device pointers) ------------------------------------------------------------ */
+
+/* y = x / sqrt(mean(x^2) + eps) * w, row-wise over `rows` rows of n. */
+int skn_rmsnorm(skn_ctx* ctx, const float* x_dev, const float* w_dev, int rows, int n, float eps, float* y_dev);
+/* Rotary embedding in place on [rows][n_head][head_dim]; row r is at position pos0 + r; interleaved pairs
+ * (2i, 2i+1), angle = pos * base^(-2i/head_dim). */
+int skn_rope(skn_ctx* ctx, float* x_dev, int rows, int n_head, int head_dim, int pos0, float base);
+/* out = silu(gate) * up elementwise. */
+int skn_swiglu(skn_ctx* ctx, const float* gate_dev, const float* up_dev, int64_t n, float* out_dev);
+/* y += x elementwise. */
+int skn_add_inplace(skn_ctx* ctx, float* y_dev, const float* x_dev, int64_t n);
+/* Index of the first maximum of x[0:n] -> *index_dev (int32 on the device); the reference's inline scan
+ * (samples/mnist-mlp-cli/src/jvmMain/kotlin/sk/ai/net/samples/mnist/mlp/Main.kt:269-278) keeps the first too. */
+int skn_argmax(skn_ctx* ctx, const float* x_dev, int n, int32_t* index_dev);
+/* fp32 -> fp16 / bf16 bits and back, elementwise (round to nearest even). */
+int skn_f32_to_f16(skn_ctx* ctx, const float* x_dev, int64_t n, uint16_t* out_dev);
+int skn_f32_to_bf16(skn_ctx* ctx, const float* x_dev, int64_t n, uint16_t* out_dev);
+
+/* ---- Llama-style decoder (7B-shaped Q4_K decode) ------------------------------------------------------ */
+
+typedef struct skn_llama_config {
+    int32_t n_layer;     /* 32 */
+    int32_t hidden;      /* 4096 */
+    int32_t ffn;         /* 11008 */
+    int32_t n_head;      /* 32 */
+    int32_t head_dim;    /* 128 */
+    int32_t vocab;       /* 32000 */
+    int32_t max_tokens;  /* KV capacity of the single sequence */
+    int32_t page_tokens; /* 256 */
+    float rope_base;     /* 10000 */
+    float rms_eps;       /* 1e-5 */
+} skn_llama_config;
+
+/* Per-layer weights, all device pointers into GGUF block data ([out, in] rows) or fp32 norm vectors. */
+typedef struct skn_llama_layer {
+    const void* wq; const void* wk; const void* wv; const void* wo; /* [hidden, hidden] */
+    const void* w_gate; const void* w_up;                            /* [ffn, hidden] */
+    const void* w_down;                                              /* [hidden, ffn] */
+    const float* attn_norm; const float* ffn_norm;                   /* [hidden] */
+    int32_t type_attn; int32_t type_ffn;                             /* ggml type ids of the matrices */
+} skn_llama_layer;
+
+typedef struct skn_llama_weights {
+    const void* tok_embd;    /* [vocab, hidden], ggml type `type_embd` */
+    const float* out_norm;   /* [hidden] */
+    const void* out_head;    /* [vocab, hidden], ggml type `type_head` */
+    int32_t type_embd; int32_t type_head;
+    const skn_llama_layer* layers; /* host array of n_layer entries (copied) */
+} skn_llama_weights;
+
+/* The module graph the reference would express as nested Module.forward calls (core/.../nn/Module.kt:6-16,
+ * core/.../nn/topology/MLP.kt:13-19) for a Llama block stack; weights stay owned by the caller. */
+int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_weights* w, skn_llama** out);
+int skn_llama_free(skn_ctx* ctx, skn_llama* m);
+int skn_llama_reset(skn_ctx* ctx, skn_llama* m);
+/* Runs n_tokens prompt tokens (host ids) through the model with batched GEMMs, filling the KV cache;
+ * logits of the last token (fp32 [vocab]) stay on the device, *next_token_host receives their argmax. */
+int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, int n_tokens, int32_t* next_token_host);
+/* Greedy decode: feeds `first_token`, then its own argmax, for n_steps steps; tokens_out_host[i] is the token
+ * produced by step i.  One captured HIP graph per step shape is replayed. */
+int skn_llama_decode(skn_ctx* ctx, skn_llama* m, int32_t first_token, int n_steps, int32_t* tokens_out_host);
+/* Device pointer to the fp32 [vocab] logits of the last processed token. */
+int skn_llama_logits(skn_ctx* ctx, skn_llama* m, const float** logits_dev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKAINET_HIP_H */

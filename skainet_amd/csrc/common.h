@@ -1,0 +1,136 @@
+// Shared internals of libskainet_hip: context, error plumbing, wave-level helpers.  gfx950 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/skainet_hip.h"
+
+struct skn_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;      // stream in use
+    hipStream_t own_stream = nullptr;  // stream created by skn_init
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    bool timer_running = false;
+    int compute_units = 0;
+    size_t lds_per_block = 0;
+    std::string err;
+    // per-launch kernel timing (skn_prof_start / skn_prof_stop): one start/stop event pair per launch
+    bool prof_on = false;
+    size_t prof_used = 0;
+    std::vector<hipEvent_t> prof_events;
+    // scratch for split-context attention partials, grown on demand
+    void* attn_scratch = nullptr;
+    size_t attn_scratch_bytes = 0;
+};
+
+// Records a failure on the context (or on the context-less slot) and returns `code`.
+int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);
+
+#define SKN_REQUIRE(ctx, cond, code, ...)                         \
+    do {                                                          \
+        if (!(cond)) return skn_fail((ctx), (code), __VA_ARGS__); \
+    } while (0)
+
+#define SKN_HIP(ctx, expr)                                                                             \
+    do {                                                                                               \
+        hipError_t e_ = (expr);                                                                        \
+        if (e_ != hipSuccess)                                                                          \
+            return skn_fail((ctx), SKN_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), \
+                            __FILE__, __LINE__);                                                       \
+    } while (0)
+
+// Call after a kernel launch.
+#define SKN_LAUNCH_CHECK(ctx) SKN_HIP((ctx), hipGetLastError())
+
+// Every kernel launch of the library goes through here.  While per-launch timing is on, the launch carries
+// its own start/stop events, which read the dispatch's begin and end timestamps (the kernel's duration as a
+// profiler reports it, without launch gaps).
+template <typename F, typename... Args>
+inline void skn_launch(skn_ctx* ctx, F kernel, dim3 grid, dim3 block, size_t lds, Args... args) {
+    if (ctx->prof_on && 2 * ctx->prof_used + 1 < ctx->prof_events.size()) {
+        hipEvent_t e0 = ctx->prof_events[2 * ctx->prof_used], e1 = ctx->prof_events[2 * ctx->prof_used + 1];
+        ctx->prof_used++;
+        hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds, ctx->stream, e0, e1, 0, args...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, (unsigned)lds, ctx->stream, args...);
+    }
+}
+
+static inline bool skn_is_quant(int t) { return t == SKN_TYPE_Q8_0 || t == SKN_TYPE_Q4_K || t == SKN_TYPE_Q6_K; }
+
+// ---- device helpers --------------------------------------------------------------------------------
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float h2f_bits(uint32_t bits16) {
+    return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+// Sum over the 64 lanes of a wavefront; every lane returns the total.
+// Steps 1-4 stay inside a 16-lane row and use DPP lane permutations; the two cross-row steps read the
+// four row totals back through scalar registers.
+__device__ __forceinline__ float wave_sum(float v) {
+    int i;
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true);  // row_half_mirror
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true);  // row_mirror
+    v += __int_as_float(i);
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    int i;
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true);
+    v = fmaxf(v, __int_as_float(i));
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true);
+    v = fmaxf(v, __int_as_float(i));
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true);
+    v = fmaxf(v, __int_as_float(i));
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true);
+    v = fmaxf(v, __int_as_float(i));
+    float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// Sum over each aligned group of 16 lanes (one DPP row); every lane of the group returns its group's total.
+__device__ __forceinline__ float row16_sum(float v) {
+    int i;
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true);
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true);
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true);
+    v += __int_as_float(i);
+    i = __builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true);
+    v += __int_as_float(i);
+    return v;
+}
+
+// Little-endian loads from addresses that are only 2-byte (or 1-byte) aligned.
+__device__ __forceinline__ uint32_t load_u32_a2(const uint8_t* p) {
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(p);
+    return (uint32_t)q[0] | ((uint32_t)q[1] << 16);
+}
+__device__ __forceinline__ uint32_t load_u16_a2(const uint8_t* p) {
+    return *reinterpret_cast<const uint16_t*>(p);
+}

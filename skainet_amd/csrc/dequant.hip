@@ -1,0 +1,114 @@
+// GGUF block dequantization (Q8_0, Q4_K, Q6_K) -> fp32, bit-exact with the ggml block formulas.
+//
+// Every thread produces four consecutive fp32 outputs (one 16-byte store), so a wavefront writes 1 KiB
+// contiguous per store instruction; the kernels are bound by the fp32 write stream (4 B per element out
+// against 0.56-1.06 B per element in).  Products are formed with the explicitly rounded intrinsics so that
+// no contraction can change a bit: each value is the exact real d*sc*q (- dmin*m) rounded once.
+#include "common.h"
+
+namespace {
+
+// Q8_0: 34-byte block = f16 d @0, int8 qs[32] @2.
+__global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                           int64_t n_quads) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_quads) return;
+    int64_t blk = t >> 3;   // 8 quads of 4 elements per 32-element block
+    int quad = (int)(t & 7);
+    const uint8_t* b = w + blk * 34;
+    float d = h2f_bits(load_u16_a2(b));
+    uint32_t q = load_u32_a2(b + 2 + 4 * quad);
+    float4 y;
+    y.x = __fmul_rn(d, (float)(int8_t)(q & 0xFF));
+    y.y = __fmul_rn(d, (float)(int8_t)((q >> 8) & 0xFF));
+    y.z = __fmul_rn(d, (float)(int8_t)((q >> 16) & 0xFF));
+    y.w = __fmul_rn(d, (float)(int8_t)(q >> 24));
+    reinterpret_cast<float4*>(out)[t] = y;
+}
+
+// Q4_K: 144-byte superblock = f16 d @0, f16 dmin @2, 12 packed 6-bit scale/min bytes @4, 128 nibble bytes @16.
+__global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                           int64_t n_quads) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_quads) return;
+    int64_t blk = t >> 6;    // 64 quads per 256-element superblock
+    int e = (int)(t & 63) * 4;  // first element of this quad inside the superblock
+    const uint8_t* b = w + blk * 144;
+    const uint32_t* b32 = reinterpret_cast<const uint32_t*>(b);  // superblocks are 16-byte aligned
+    uint32_t dd = b32[0];
+    float d = h2f_bits(dd & 0xFFFF), dmin = h2f_bits(dd >> 16);
+    int c = e >> 6, r = e & 63;
+    int j = 2 * c + (r >= 32);
+    const uint8_t* s = b + 4;
+    int sc, m;
+    if (j < 4) {
+        sc = s[j] & 63;
+        m = s[j + 4] & 63;
+    } else {
+        sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    }
+    uint32_t q = b32[4 + 8 * c + ((r & 31) >> 2)];
+    if (r >= 32) q >>= 4;
+    float d1 = __fmul_rn(d, (float)sc);
+    float m1 = __fmul_rn(dmin, (float)m);
+    float4 y;
+    y.x = __fsub_rn(__fmul_rn(d1, (float)(q & 0xF)), m1);
+    y.y = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xF)), m1);
+    y.z = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xF)), m1);
+    y.w = __fsub_rn(__fmul_rn(d1, (float)((q >> 24) & 0xF)), m1);
+    reinterpret_cast<float4*>(out)[t] = y;
+}
+
+// Q6_K: 210-byte superblock = ql[128] @0 (low nibbles), qh[64] @128 (high bit pairs), int8 scales[16] @192, f16 d @208.
+__global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                           int64_t n_quads) {
+    int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_quads) return;
+    int64_t blk = t >> 6;
+    int e = (int)(t & 63) * 4;
+    const uint8_t* b = w + blk * 210;  // only 2-byte aligned
+    int n = e >> 7, r = e & 127;
+    int quarter = r >> 5, l = r & 31;  // l is a multiple of 4
+    uint32_t lo = load_u32_a2(b + 64 * n + l + 32 * (quarter & 1));
+    if (quarter >= 2) lo >>= 4;
+    uint32_t hi = load_u32_a2(b + 128 + 32 * n + l) >> (2 * quarter);
+    float sc = (float)(int8_t)b[192 + 8 * n + 2 * quarter + (l >> 4)];
+    float d = h2f_bits(load_u16_a2(b + 208));
+    float ds = __fmul_rn(d, sc);
+    float4 y;
+    y.x = __fmul_rn(ds, (float)((int)((lo & 0xF) | ((hi & 3) << 4)) - 32));
+    y.y = __fmul_rn(ds, (float)((int)(((lo >> 8) & 0xF) | (((hi >> 8) & 3) << 4)) - 32));
+    y.z = __fmul_rn(ds, (float)((int)(((lo >> 16) & 0xF) | (((hi >> 16) & 3) << 4)) - 32));
+    y.w = __fmul_rn(ds, (float)((int)(((lo >> 24) & 0xF) | (((hi >> 24) & 3) << 4)) - 32));
+    reinterpret_cast<float4*>(out)[t] = y;
+}
+
+}  // namespace
+
+extern "C" int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64_t n_elems, float* out_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_dequant: ctx is null");
+    SKN_REQUIRE(ctx, skn_is_quant(ggml_type), SKN_ERR_TYPE, "skn_dequant: ggml type %d is not supported", ggml_type);
+    int be, bb;
+    skn_type_block(ggml_type, &be, &bb);
+    SKN_REQUIRE(ctx, n_elems >= 0 && n_elems % be == 0, SKN_ERR_SHAPE,
+                "skn_dequant: element count (%lld) is not a multiple of block size (%d)", (long long)n_elems, be);
+    if (n_elems == 0) return SKN_OK;
+    SKN_REQUIRE(ctx, w_dev && out_dev, SKN_ERR_ARG, "skn_dequant: null pointer");
+    SKN_REQUIRE(ctx, ((uintptr_t)out_dev & 15) == 0, SKN_ERR_ARG, "skn_dequant: out must be 16-byte aligned");
+    SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : 1)) == 0, SKN_ERR_ARG,
+                "skn_dequant: weight pointer is misaligned for its block type");
+    int64_t n_quads = n_elems / 4;
+    int64_t blocks = (n_quads + 255) / 256;
+    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_dequant: too many elements for one launch");
+    const uint8_t* w = (const uint8_t*)w_dev;
+    dim3 grid((unsigned)blocks), block(256);
+    if (ggml_type == SKN_TYPE_Q8_0)
+        skn_launch(ctx, dequant_q8_0_kernel, grid, block, 0, w, out_dev, n_quads);
+    else if (ggml_type == SKN_TYPE_Q4_K)
+        skn_launch(ctx, dequant_q4_k_kernel, grid, block, 0, w, out_dev, n_quads);
+    else
+        skn_launch(ctx, dequant_q6_k_kernel, grid, block, 0, w, out_dev, n_quads);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}

@@ -1,0 +1,123 @@
+"""GPU parity: dequantization (bit-exact) and batch-1 matvec (rel. error <= 1e-3) through the C ABI vs the CPU oracle."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle_c, oracle_np
+from skainet_amd import runtime, synth
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TOL = 1e-3  # max_i |a_i - r_i| / max(|r_i|, 1e-3 * max|r|) against the fp64-accumulated oracle
+
+
+@pytest.mark.parametrize("qtype,name", [(Q8_0, "q8_0"), (Q4_K, "q4_k"), (Q6_K, "q6_k")])
+def test_dequant_golden_blocks_bit_exact(hip, golden_dir, qtype, name):
+    blocks = np.load(os.path.join(golden_dir, "quant_blocks.npz"))
+    got = hip.dequant_host(qtype, blocks[f"{name}_raw"])
+    assert np.array_equal(got.view(np.uint32), blocks[f"{name}_f32_bits"])
+
+
+@pytest.mark.parametrize("qtype", [Q8_0, Q4_K, Q6_K])
+def test_dequant_bit_exact_vs_oracle(hip, qtype):
+    be, bb = synth.BLOCK[qtype]
+    raw = synth.weight(qtype, 512, 4096, seed=100 + qtype)
+    got = hip.dequant_host(qtype, raw)
+    want = oracle_c.dequant(qtype, raw)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # arbitrary bytes (random f16 scales incl. subnormals and negatives; inf / nan scales excluded)
+    rng = np.random.default_rng(7 + qtype)
+    rnd = rng.integers(0, 256, size=(4096, bb), dtype=np.uint8)
+    for p in {Q8_0: [1], Q4_K: [1, 3], Q6_K: [209]}[qtype]:
+        rnd[:, p] &= 0xFB
+    got = hip.dequant_host(qtype, rnd.reshape(-1))
+    want = oracle_c.dequant(qtype, rnd.reshape(-1))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_full_size_checksum(hip):
+    # full benchmark tensor (Q4_K 4096 x 11008): compared through a 64-bit sum of the output words
+    raw = synth.weight(Q4_K, 4096, 11008, seed=42)
+    got = hip.dequant_host(Q4_K, raw)
+    want = oracle_c.dequant(Q4_K, raw)
+    assert int(got.view(np.uint32).astype(np.uint64).sum()) == int(want.view(np.uint32).astype(np.uint64).sum())
+    assert np.array_equal(got[:: 4099].view(np.uint32), want[:: 4099].view(np.uint32))
+
+
+def test_dequant_errors(hip):
+    buf = hip.alloc(1024)
+    with pytest.raises(runtime.SknError) as e:
+        hip.dequant(13, buf, 256, buf)
+    assert e.value.code == runtime.ERR_TYPE
+    with pytest.raises(runtime.SknError) as e:
+        hip.dequant(Q4_K, buf, 100, buf)
+    assert e.value.code == runtime.ERR_SHAPE
+    with pytest.raises(runtime.SknError) as e:
+        hip.dequant(Q4_K, None, 256, buf)
+    assert e.value.code == runtime.ERR_ARG
+    hip.dequant(Q4_K, buf, 0, buf)  # empty input is a no-op
+
+
+MATVEC_CASES = [
+    (Q8_0, 4096, 4096),
+    (Q4_K, 4096, 4096),
+    (Q4_K, 11008, 4096),
+    (Q4_K, 4096, 11008),
+    (Q6_K, 4096, 4096),
+    # ragged: rows not a multiple of the workgroup, K from one superblock up to a non-power-of-two count
+    (Q4_K, 37, 256),
+    (Q4_K, 5, 2304),
+    (Q4_K, 100, 13 * 256),
+    (Q4_K, 3, 57 * 256),
+    (Q8_0, 33, 96),
+    (Q8_0, 7, 32 * 131),
+    (Q6_K, 19, 768),
+]
+
+
+@pytest.mark.parametrize("qtype,n,k", MATVEC_CASES)
+def test_matvec_vs_oracle(hip, qtype, n, k):
+    raw = synth.weight(qtype, n, k, seed=n * 7 + k)
+    x = synth.activation_f32(k, seed=k + 1)
+    got = hip.matvec_q_host(qtype, raw, n, k, x)
+    want = oracle_c.matvec_q(qtype, raw, n, k, x)
+    err = oracle_np.rel_err(got, want)
+    assert err <= TOL, f"rel err {err}"
+
+
+@pytest.mark.parametrize("qtype", [Q8_0, Q4_K, Q6_K])
+def test_matvec_one_hot_and_linearity(hip, qtype):
+    n, k = 64, 2048
+    raw = synth.weight(qtype, n, k, seed=5)
+    w = oracle_c.dequant(qtype, raw).reshape(n, k)
+    for col in (0, 31, 32, 255, 256, 1029, k - 1):
+        e = np.zeros(k, dtype=np.float32)
+        e[col] = 1.0
+        got = hip.matvec_q_host(qtype, raw, n, k, e)
+        assert np.allclose(got, w[:, col], rtol=1e-6, atol=1e-7), col
+    x1 = synth.activation_f32(k, seed=1)
+    x2 = synth.activation_f32(k, seed=2)
+    y1 = hip.matvec_q_host(qtype, raw, n, k, x1).astype(np.float64)
+    y2 = hip.matvec_q_host(qtype, raw, n, k, x2).astype(np.float64)
+    y12 = hip.matvec_q_host(qtype, raw, n, k, 2.0 * x1 - x2).astype(np.float64)
+    assert oracle_np.rel_err(y12, 2.0 * y1 - y2) <= TOL
+
+
+def test_matvec_errors_and_empty(hip):
+    buf = hip.alloc(4096)
+    with pytest.raises(runtime.SknError) as e:
+        hip.matvec_q(Q4_K, buf, 4, 200, buf, buf)
+    assert e.value.code == runtime.ERR_SHAPE
+    assert "is not a multiple of block size (256)" in e.value.message
+    with pytest.raises(runtime.SknError) as e:
+        hip.matvec_q(2, buf, 4, 256, buf, buf)
+    assert e.value.code == runtime.ERR_TYPE
+    with pytest.raises(runtime.SknError) as e:
+        hip.matvec_q(Q4_K, buf, 4, 256, None, buf)
+    assert e.value.code == runtime.ERR_ARG
+    hip.matvec_q(Q4_K, buf, 0, 256, buf, buf)
+    y = hip.to_device(np.ones(4, dtype=np.float32))
+    hip.matvec_q(Q4_K, buf, 4, 0, buf, y)  # k = 0: the empty sum
+    assert np.all(y.download(np.float32, 4) == 0.0)
