@@ -82,6 +82,9 @@ int skn_memset(skn_ctx* ctx, void* dev, int byte_value, size_t bytes);
 int skn_sync(skn_ctx* ctx);
 /* Adopt a caller-owned hipStream_t (NULL restores the context's own stream). */
 int skn_set_stream(skn_ctx* ctx, void* hip_stream);
+/* Launch-shape tuning knobs, 0 = library default: "q4k.waves" (wavefronts per workgroup of the Q4_K matvec),
+ * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention). */
+int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
 int skn_timer_start(skn_ctx* ctx);
 int skn_timer_stop(skn_ctx* ctx, float* elapsed_ms);

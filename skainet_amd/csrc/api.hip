@@ -183,6 +183,16 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream) {
     return SKN_OK;
 }
 
+int skn_set_option(skn_ctx* ctx, const char* key, int value) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_set_option: ctx is null");
+    SKN_REQUIRE(ctx, key != nullptr, SKN_ERR_ARG, "skn_set_option: key is null");
+    if (!strcmp(key, "q4k.waves")) ctx->opt_q4k_waves = value;
+    else if (!strcmp(key, "q4k.rows")) ctx->opt_q4k_rows = value;
+    else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
+    else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
+    return SKN_OK;
+}
+
 int skn_timer_start(skn_ctx* ctx) {
     SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_timer_start: ctx is null");
     SKN_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));

@@ -27,6 +27,8 @@ struct skn_ctx {
     bool prof_on = false;
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
+    // tuning options (skn_set_option); 0 = library default
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0;
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;

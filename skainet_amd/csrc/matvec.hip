@@ -11,173 +11,225 @@ namespace {
 //
 // A row of k weights is k/256 superblocks of 144 bytes = 9 aligned 16-byte chunks each: one header chunk
 // (f16 d, f16 dmin, 12 bytes of 6-bit scales/mins) and eight chunks of nibbles.  Per step a wavefront takes
-// eight superblocks: lane (b, c) = (lane / 8, lane % 8) loads nibble chunk c of superblock b with one
-// 128-bit load (64 lanes x 16 B, eight 128-byte runs) and the superblock's header with a second 128-bit load
-// that its eight lanes share.  All loads of a row are issued before anything is consumed, so a row's whole
-// byte range is in flight at once.
+// sixteen superblocks of R consecutive rows: lane (b, p) = (lane / 4, lane % 4) owns the 64 weights of
+// sub-block pair p of superblock b -- nibble chunks 2p and 2p+1, two 128-bit loads -- plus the header chunk
+// that its four lanes share.  Every load of the wavefront's rows is issued before anything is consumed.
 //
-// Nibble chunk c holds bytes 16c..16c+15 of qs: low nibbles are elements 64*(c/2) + 16*(c%2) + 0..15 (sub-block
-// 2*(c/2)), high nibbles the same positions + 32 (sub-block 2*(c/2)+1).  The activation is staged in LDS in
-// exactly that lane order -- slot [(step*8 + i)*64 + lane] holds the i-th float4 the lane needs -- so the
-// eight 128-bit LDS reads of a step are conflict-free, together with the two 16-element partial sums of x
-// that the "- dmin * m" term needs.
+// Nibble bytes 32p..32p+31 of qs: low nibbles are elements 64p + 0..31 (sub-block 2p), high nibbles elements
+// 64p + 32..63 (sub-block 2p+1).  The activation is staged in LDS in lane order -- slot [(step*16 + i)*64 + lane]
+// is the i-th float4 of the lane's 64 activations -- so the 128-bit LDS reads are conflict-free, and one read
+// of x serves the R rows.  Two tricks keep the VALU work per weight low:
+//   * a nibble masked in place (q & 0x000F000F, q & 0x00F000F0) is read as a pair of fp16 subnormals
+//     n * 2^-24 (or 16n * 2^-24), which v_fma_mix_f32 multiplies with the fp32 activation directly: no
+//     integer-to-float conversion, one mask per two weights, one fused multiply-add per weight;
+//   * the powers of two are folded into the staged data: the activations that meet high nibbles are stored
+//     divided by 16, the per-sub-block sums of x (for the "- dmin * m" term) multiplied by 2^-24, and the row
+//     total is multiplied by 2^24 once.
 //
-//   y += d * (sc_lo * sum(q_lo * x_lo) + sc_hi * sum(q_hi * x_hi)) - dmin * (m_lo * sum(x_lo) + m_hi * sum(x_hi))
+//   y = 2^24 * sum_blocks [ d * (sc_lo * A_lo + sc_hi * A_hi) - dmin * (m_lo * S_lo + m_hi * S_hi) ]
 
 constexpr int kQ4kBlockBytes = 144;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
+// 6-bit scales / mins of sub-blocks 2p and 2p+1 out of the header chunk h = (d|dmin, scales[0..3], [4..7], [8..11]).
+// Branch-free and two values at a time: both packings are formed as byte pairs and the lane's pair index
+// selects one, so the header registers are only ever read by straight-line code.
 __device__ __forceinline__ void q4k_pair_scales(const uint4& h, int pair, float& sc0, float& sc1, float& m0,
                                                 float& m1) {
-    // pair p covers sub-blocks 2p and 2p+1; scales[] = bytes of (h.y, h.z, h.w)
     const int sh = 16 * (pair & 1);
-    const uint32_t a = (h.y >> sh) & 0xFFFF;  // scales[j], scales[j+1] of the low group (j = 2p or 2p-4)
-    const uint32_t b = (h.z >> sh) & 0xFFFF;  // scales[4+..]
-    const uint32_t c = (h.w >> sh) & 0xFFFF;  // scales[8+..]
-    uint32_t s0, s1, n0, n1;
-    if (pair < 2) {
-        s0 = a & 63;
-        s1 = (a >> 8) & 63;
-        n0 = b & 63;
-        n1 = (b >> 8) & 63;
-    } else {
-        s0 = (c & 0xF) | (((a >> 6) & 3) << 4);
-        s1 = ((c >> 8) & 0xF) | (((a >> 14) & 3) << 4);
-        n0 = ((c >> 4) & 0xF) | (((b >> 6) & 3) << 4);
-        n1 = ((c >> 12) & 0xF) | (((b >> 14) & 3) << 4);
-    }
-    sc0 = (float)s0;
-    sc1 = (float)s1;
-    m0 = (float)n0;
-    m1 = (float)n1;
+    const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
+    const uint32_t s_lo = a & 0x3F3Fu, n_lo = b & 0x3F3Fu;                        // sub-blocks 0..3: plain 6-bit fields
+    const uint32_t s_hi = (c & 0x0F0Fu) | ((a >> 2) & 0x3030u);                    // sub-blocks 4..7: 4 low bits in
+    const uint32_t n_hi = ((c >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u);             // scales[8..11], 2 high bits parked
+    const uint32_t sp = pair < 2 ? s_lo : s_hi;                                    // in the tops of scales[0..7]
+    const uint32_t np = pair < 2 ? n_lo : n_hi;
+    sc0 = (float)(sp & 0xFF);
+    sc1 = (float)((sp >> 8) & 0xFF);
+    m0 = (float)(np & 0xFF);
+    m1 = (float)((np >> 8) & 0xFF);
 }
 
-// sum over the 4 bytes of q of nibble * x: low nibbles against xl, high nibbles against xh
+// One dword of nibbles: low nibbles of bytes 0..3 against xl.{x,y,z,w}, high nibbles against xh (pre-divided by 16).
 __device__ __forceinline__ void q4k_dot_dword(uint32_t q, const float4& xl, const float4& xh, float& alo, float& ahi) {
-    const uint32_t lo = q & 0x0F0F0F0Fu;
-    const uint32_t hi = (q >> 4) & 0x0F0F0F0Fu;
-    alo = fmaf((float)(lo & 0xFF), xl.x, alo);
-    alo = fmaf((float)((lo >> 8) & 0xFF), xl.y, alo);
-    alo = fmaf((float)((lo >> 16) & 0xFF), xl.z, alo);
-    alo = fmaf((float)(lo >> 24), xl.w, alo);
-    ahi = fmaf((float)(hi & 0xFF), xh.x, ahi);
-    ahi = fmaf((float)((hi >> 8) & 0xFF), xh.y, ahi);
-    ahi = fmaf((float)((hi >> 16) & 0xFF), xh.z, ahi);
-    ahi = fmaf((float)(hi >> 24), xh.w, ahi);
+    const uint32_t q8 = q >> 8;
+    const half2_t l02 = __builtin_bit_cast(half2_t, q & 0x000F000Fu);
+    const half2_t h02 = __builtin_bit_cast(half2_t, q & 0x00F000F0u);
+    const half2_t l13 = __builtin_bit_cast(half2_t, q8 & 0x000F000Fu);
+    const half2_t h13 = __builtin_bit_cast(half2_t, q8 & 0x00F000F0u);
+    alo = fmaf((float)l02.x, xl.x, alo);
+    ahi = fmaf((float)h02.x, xh.x, ahi);
+    alo = fmaf((float)l13.x, xl.y, alo);
+    ahi = fmaf((float)h13.x, xh.y, ahi);
+    alo = fmaf((float)l02.y, xl.z, alo);
+    ahi = fmaf((float)h02.y, xh.z, ahi);
+    alo = fmaf((float)l13.y, xl.w, alo);
+    ahi = fmaf((float)h13.y, xh.w, ahi);
 }
 
-// Stage x for Q4_K rows of nb superblocks into LDS in lane order; see the layout note above.
-__device__ __forceinline__ void q4k_stage_x(const float* __restrict__ x, int nb, float4* xs, float2* ss, int tid,
-                                            int nthreads) {
-    const int ncols = nb * 8;  // one column of 32 activations per (superblock, nibble chunk)
-    const int steps = (nb + 7) >> 3;
-    for (int cc = tid; cc < steps * 64; cc += nthreads) {
-        const int step = cc >> 6, lane = cc & 63;
-        float4 v[8];
-        if (cc < ncols) {
-            const int blk = cc >> 3, c = cc & 7;
-            const float4* src = reinterpret_cast<const float4*>(x + 256 * blk + 64 * (c >> 1) + 16 * (c & 1));
+// Staging of x, split in two so that the weight loads can be issued in between: the global loads of one
+// half column (32 activations of one (superblock, pair) column) into registers, and later their LDS stores.
+struct Q4kStage {
+    float4 v[8];
+};
+
+__device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int hc, Q4kStage& st) {
+    const float4* src = reinterpret_cast<const float4*>(x + 32 * hc);
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                v[i] = src[i];
-                v[4 + i] = src[8 + i];
-            }
-        } else {
+    for (int i = 0; i < 8; i++) st.v[i] = src[i];
+}
+
+__device__ __forceinline__ void q4k_stage_store(const Q4kStage& st, int hc, float4* xs, float* ss) {
+    const int cc = hc >> 1, half = hc & 1;
+    const int step = cc >> 6, lane = cc & 63;
+    const float mul = half ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
+    float sum = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = 0; i < 8; i++) {
+        const float4 v = st.v[i];
+        sum += (v.x + v.y) + (v.z + v.w);
+        xs[(step * 16 + 8 * half + i) * 64 + lane] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
+    }
+    ss[2 * cc + half] = sum * 5.9604644775390625e-08f;  // 2^-24, see the scaling note above
+}
+
+struct Q4kLoads {
+    uint4 h, qa, qb;
+    bool ok;  // false: the slot lies past the row end / past the last row and must contribute nothing
+};
+
+// One step for R rows: the lane's 64 activations are read from LDS in two halves of 32 (8 float4 live at a
+// time) and each half meets the matching nibble chunk of every row.
+template <int R>
+__device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, int pair, float (&acc)[R]) {
+    float alo[R], ahi[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) alo[r] = ahi[r] = 0.f;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        float4 xl[4], xh[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xl[j] = xs[(s * 16 + 4 * half + j) * 64 + lane];
+            xh[j] = xs[(s * 16 + 8 + 4 * half + j) * 64 + lane];
         }
-        float slo = 0.f, shi = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            slo += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            shi += (v[4 + i].x + v[4 + i].y) + (v[4 + i].z + v[4 + i].w);
+        for (int r = 0; r < R; r++) {
+            const uint4 qq = half == 0 ? L[r].qa : L[r].qb;
+            q4k_dot_dword(qq.x, xl[0], xh[0], alo[r], ahi[r]);
+            q4k_dot_dword(qq.y, xl[1], xh[1], alo[r], ahi[r]);
+            q4k_dot_dword(qq.z, xl[2], xh[2], alo[r], ahi[r]);
+            q4k_dot_dword(qq.w, xl[3], xh[3], alo[r], ahi[r]);
         }
+    }
+    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];
 #pragma unroll
-        for (int i = 0; i < 8; i++) xs[(step * 8 + i) * 64 + lane] = v[i];
-        ss[cc] = make_float2(slo, shi);
+    for (int r = 0; r < R; r++) {
+        float sc0, sc1, m0, m1;
+        q4k_pair_scales(L[r].h, pair, sc0, sc1, m0, m1);
+        const half2_t dd = __builtin_bit_cast(half2_t, L[r].h.x);
+        const float t1 = fmaf(sc1, ahi[r], sc0 * alo[r]);
+        const float t2 = fmaf(m1, sx.y, m0 * sx.x);
+        const float v = fmaf((float)dd.x, t1, -((float)dd.y * t2));
+        acc[r] += L[r].ok ? v : 0.f;
     }
 }
 
-// STEPS > 0: the row is covered by exactly STEPS fully unrolled steps with every load hoisted.
-// STEPS == 0: generic rolled loop for any k.
-template <int STEPS>
-__global__ __launch_bounds__(1024) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                                          float* __restrict__ y, int n_rows, int nb) {
+// R = consecutive rows per wavefront (x is read from LDS once for the R rows).
+// STEPS > 0: the row takes exactly STEPS steps, fully unrolled.  STEPS == 0: rolled loop for any k.
+//
+// Order of events in a wavefront: issue the x loads, issue the weight loads of step 0, wait for x only (its
+// loads are the oldest in flight), store it to LDS, barrier; then per step: issue the weight loads of the
+// next step, consume the current one.  A compute unit's memory pipeline accepts only so many requests before
+// a wavefront stalls at issue, so the loads are kept one step ahead instead of all up front -- otherwise the
+// x stores (and with them every wavefront at the barrier) would sit behind the issue of a whole row.
+template <int STEPS, int R>
+__global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ y, int n_rows, int nb) {
     extern __shared__ float4 lds4[];
-    const int steps = STEPS > 0 ? STEPS : (nb + 7) >> 3;
+    const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
-    float2* ss = reinterpret_cast<float2*>(lds4 + steps * 8 * 64);
+    float* ss = reinterpret_cast<float*>(lds4 + steps * 16 * 64);
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
     const int waves = blockDim.x >> 6;
-    const int row = blockIdx.x * waves + wave;
-    const bool row_ok = row < n_rows;
-    const int sub = lane >> 3;  // superblock within the step
-    const int c = lane & 7;     // nibble chunk within the superblock
-    const uint4* rowp = reinterpret_cast<const uint4*>(w + (size_t)(row_ok ? row : 0) * nb * kQ4kBlockBytes);
+    const int row0 = (blockIdx.x * waves + wave) * R;
+    const int sub = lane >> 2;  // superblock within the step
+    const int p = lane & 3;     // sub-block pair within the superblock
+    const size_t row_chunks = (size_t)nb * 9;
+    const int n_half_cols = nb * 8;
+
+    // this thread's first half column of x goes into registers (threads past the last half column repeat the
+    // last one: same data to the same slot, no branch)
+    Q4kStage st;
+    const int hc0 = min(tid, n_half_cols - 1);
+    q4k_stage_load(x, hc0, st);
+
+    float acc[R];
+    const uint4* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
+        rp[r] = reinterpret_cast<const uint4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + 1 + 2 * p;
+    }
+    auto issue = [&](int s, int tie, Q4kLoads (&L)[R]) {
+        const int blk = s * 16 + sub;
+        const int off = min(blk, nb - 1) * 9 + tie;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint4* bp = rp[r] + off;
+            L[r].qa = bp[0];
+            L[r].qb = bp[1];
+            L[r].h = bp[-1 - 2 * p];
+            L[r].ok = row_ok[r] && blk < nb;
+        }
+    };
 
     if constexpr (STEPS > 0) {
-        uint4 qv[STEPS], hv[STEPS];
-#pragma unroll
-        for (int s = 0; s < STEPS; s++) {
-            const int blk = s * 8 + sub;
-            const bool ok = row_ok && blk < nb;
-            const uint4* bp = rowp + (ok ? blk : 0) * 9;
-            qv[s] = bp[1 + c];
-            hv[s] = bp[0];
-            if (!ok) {
-                qv[s] = make_uint4(0, 0, 0, 0);
-                hv[s] = make_uint4(0, 0, 0, 0);
-            }
-        }
-        q4k_stage_x(x, nb, xs, ss, threadIdx.x, blockDim.x);
+        Q4kLoads L[STEPS][R];
+        issue(0, 0, L[0]);
+        // the launcher guarantees blockDim.x >= nb * 8 here: one half column per thread covers x, no loop
+        q4k_stage_store(st, hc0, xs, ss);
         __syncthreads();
-        float acc = 0.f;
+        // `tie` is always 0; an empty asm after each step makes it look rewritten from the finished accumulator,
+        // which pins the loads of step s+1 between the arithmetic of steps s-1 and s (one step of lookahead) and
+        // the LDS reads of step s below the arithmetic of step s-1 (bounded registers)
+        int tie = 0;
+        asm volatile("" : "+v"(tie));
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
-            float alo = 0.f, ahi = 0.f;
-            const uint32_t q[4] = {qv[s].x, qv[s].y, qv[s].z, qv[s].w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float4 xl = xs[(s * 8 + i) * 64 + lane];
-                const float4 xh = xs[(s * 8 + 4 + i) * 64 + lane];
-                q4k_dot_dword(q[i], xl, xh, alo, ahi);
-            }
-            const float2 sx = ss[s * 64 + lane];
-            float sc0, sc1, m0, m1;
-            q4k_pair_scales(hv[s], c >> 1, sc0, sc1, m0, m1);
-            const float d = h2f_bits(hv[s].x & 0xFFFF), dmin = h2f_bits(hv[s].x >> 16);
-            acc += d * (sc0 * alo + sc1 * ahi) - dmin * (m0 * sx.x + m1 * sx.y);
+            if (s + 1 < STEPS) issue(s + 1, tie, L[s + 1]);
+            asm volatile("" ::: "memory");  // the loads above stay above the LDS reads below
+            q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
+            asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
         }
-        acc = wave_sum(acc);
-        if (row_ok && lane == 0) y[row] = acc;
     } else {
-        q4k_stage_x(x, nb, xs, ss, threadIdx.x, blockDim.x);
+        Q4kLoads bufa[R], bufb[R];
+        issue(0, 0, bufa);
+        q4k_stage_store(st, hc0, xs, ss);
+        for (int hc = tid + blockDim.x; hc < n_half_cols; hc += blockDim.x) {
+            q4k_stage_load(x, hc, st);
+            q4k_stage_store(st, hc, xs, ss);
+        }
         __syncthreads();
-        float acc = 0.f;
-        for (int s = 0; s < steps; s++) {
-            const int blk = s * 8 + sub;
-            if (row_ok && blk < nb) {
-                const uint4* bp = rowp + blk * 9;
-                const uint4 qq = bp[1 + c];
-                const uint4 hh = bp[0];
-                float alo = 0.f, ahi = 0.f;
-                const uint32_t q[4] = {qq.x, qq.y, qq.z, qq.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float4 xl = xs[(s * 8 + i) * 64 + lane];
-                    const float4 xh = xs[(s * 8 + 4 + i) * 64 + lane];
-                    q4k_dot_dword(q[i], xl, xh, alo, ahi);
-                }
-                const float2 sx = ss[s * 64 + lane];
-                float sc0, sc1, m0, m1;
-                q4k_pair_scales(hh, c >> 1, sc0, sc1, m0, m1);
-                const float d = h2f_bits(hh.x & 0xFFFF), dmin = h2f_bits(hh.x >> 16);
-                acc += d * (sc0 * alo + sc1 * ahi) - dmin * (m0 * sx.x + m1 * sx.y);
+        for (int s = 0; s < steps; s += 2) {
+            if (s + 1 < steps) issue(s + 1, 0, bufb);
+            q4k_step<R>(bufa, xs, ss, s, lane, p, acc);
+            if (s + 1 < steps) {
+                if (s + 2 < steps) issue(s + 2, 0, bufa);
+                q4k_step<R>(bufb, xs, ss, s + 1, lane, p, acc);
             }
         }
-        acc = wave_sum(acc);
-        if (row_ok && lane == 0) y[row] = acc;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]) * 16777216.0f;
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
     }
 }
 
@@ -246,20 +298,33 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
     if (lane == 0) y[row] = acc;
 }
 
-template <int STEPS>
+template <int STEPS, int R>
 int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
-    const int steps = STEPS > 0 ? STEPS : (nb + 7) / 8;
-    const size_t lds = (size_t)steps * 64 * (8 * sizeof(float4) + sizeof(float2));
+    if (STEPS > 0 && waves * 64 < nb * 8) return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
+    const int steps = (nb + 15) / 16;
+    const size_t lds = (size_t)steps * 64 * (16 * sizeof(float4) + sizeof(float2));
     SKN_REQUIRE(ctx, lds <= 160 * 1024, SKN_ERR_SHAPE, "skn_matvec_q: k = %d needs %zu bytes of LDS (limit 163840)",
                 nb * 256, lds);
-    auto kern = matvec_q4k_kernel<STEPS>;
+    auto kern = matvec_q4k_kernel<STEPS, R>;
     if (lds > 48 * 1024)
         SKN_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)lds));
-    dim3 grid((unsigned)((n + waves - 1) / waves)), block((unsigned)(waves * 64));
+    const int rows_per_wg = waves * R;
+    dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block((unsigned)(waves * 64));
     skn_launch(ctx, kern, grid, block, lds, w, x, y, n, nb);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
+}
+
+template <int R>
+int dispatch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
+    switch ((nb + 15) / 16) {
+        case 1: return launch_q4k<1, R>(ctx, w, n, nb, x, y, waves);
+        case 2: return launch_q4k<2, R>(ctx, w, n, nb, x, y, waves);
+        case 3: return launch_q4k<3, R>(ctx, w, n, nb, x, y, waves);
+        case 4: return launch_q4k<4, R>(ctx, w, n, nb, x, y, waves);
+        default: return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
+    }
 }
 
 }  // namespace
@@ -283,17 +348,13 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     const uint8_t* w = (const uint8_t*)w_dev;
     const int nb = k / be;
     if (ggml_type == SKN_TYPE_Q4_K) {
-        const int steps = (nb + 7) / 8;
-        const int waves = 16;
-        switch (steps) {
-            case 1: return launch_q4k<1>(ctx, w, n, nb, x_dev, y_dev, waves);
-            case 2: return launch_q4k<2>(ctx, w, n, nb, x_dev, y_dev, waves);
-            case 3: return launch_q4k<3>(ctx, w, n, nb, x_dev, y_dev, waves);
-            case 4: return launch_q4k<4>(ctx, w, n, nb, x_dev, y_dev, waves);
-            case 6: return launch_q4k<6>(ctx, w, n, nb, x_dev, y_dev, waves);
-            case 7: return launch_q4k<7>(ctx, w, n, nb, x_dev, y_dev, waves);
-            default: return launch_q4k<0>(ctx, w, n, nb, x_dev, y_dev, waves);
-        }
+        int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;
+        if (waves <= 0) waves = 8;
+        if (rows <= 0) rows = 2;
+        if (waves > 8) waves = 8;
+        return rows >= 4   ? dispatch_q4k<4>(ctx, w, n, nb, x_dev, y_dev, waves)
+               : rows >= 2 ? dispatch_q4k<2>(ctx, w, n, nb, x_dev, y_dev, waves)
+                           : dispatch_q4k<1>(ctx, w, n, nb, x_dev, y_dev, waves);
     }
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
     if (ggml_type == SKN_TYPE_Q8_0)

@@ -67,6 +67,7 @@ _SIGNATURES = {
     "skn_memset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t]),
     "skn_sync": (C.c_int, [C.c_void_p]),
     "skn_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "skn_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
     "skn_timer_start": (C.c_int, [C.c_void_p]),
     "skn_timer_stop": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "skn_prof_start": (C.c_int, [C.c_void_p, C.c_int]),
@@ -287,6 +288,9 @@ class Context:
         ms = C.c_float()
         self._check(self.lib.skn_timer_stop(self.handle, C.byref(ms)))
         return ms.value
+
+    def set_option(self, key, value):
+        self._check(self.lib.skn_set_option(self.handle, key.encode(), int(value)))
 
     def prof_start(self, max_launches):
         self._check(self.lib.skn_prof_start(self.handle, max_launches))
