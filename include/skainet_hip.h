@@ -83,7 +83,8 @@ int skn_sync(skn_ctx* ctx);
 /* Adopt a caller-owned hipStream_t (NULL restores the context's own stream). */
 int skn_set_stream(skn_ctx* ctx, void* hip_stream);
 /* Launch-shape tuning knobs, 0 = library default: "q4k.waves" (wavefronts per workgroup of the Q4_K matvec),
- * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention). */
+ * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention),
+ * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel). */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
 int skn_timer_start(skn_ctx* ctx);

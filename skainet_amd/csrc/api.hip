@@ -62,6 +62,12 @@ int skn_init(int device, skn_ctx** out) {
         return rc;
     }
     ctx->stream = ctx->own_stream;
+    int rc = skn_matvec_init(ctx);
+    if (rc != SKN_OK) {
+        g_ctxless_error = ctx->err;
+        skn_shutdown(ctx);
+        return rc;
+    }
     *out = ctx;
     return SKN_OK;
 }
@@ -70,6 +76,7 @@ void skn_shutdown(skn_ctx* ctx) {
     if (!ctx) return;
     if (ctx->own_stream) (void)hipStreamSynchronize(ctx->own_stream);
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
+    if (ctx->gemm_ws) (void)hipFree(ctx->gemm_ws);
     for (hipEvent_t e : ctx->prof_events) (void)hipEventDestroy(e);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
@@ -189,6 +196,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     if (!strcmp(key, "q4k.waves")) ctx->opt_q4k_waves = value;
     else if (!strcmp(key, "q4k.rows")) ctx->opt_q4k_rows = value;
     else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
+    else if (!strcmp(key, "llama.graph")) ctx->opt_llama_graph = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
     return SKN_OK;
 }

@@ -15,7 +15,7 @@ template <int D>
 __global__ __launch_bounds__(256) void attn_decode_split_kernel(
     const uint16_t* __restrict__ k_pool, const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ table,
     const int32_t* __restrict__ nctx, const float* __restrict__ q, float* __restrict__ partial, int n_head,
-    int page_tokens, int pages_per_seq, int n_splits, float scale) {
+    int page_tokens, int pages_per_seq, int n_splits, float scale, int seq_fixed) {
     constexpr int KROW = D + 8;   // halves per K row in LDS: 16 bytes of padding spread the rows over the banks
     constexpr int CH = D / 8;     // 16-byte chunks per row
     constexpr int QS = D / 4;     // dims per score thread
@@ -26,7 +26,10 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
     __shared__ float red_max[4], red_sum[4];
     __shared__ float obuf[4][D];
 
+    // blockIdx.z is the query row: its own sequence by default, or one shared sequence (seq_fixed >= 0) when
+    // several query rows attend to prefixes of the same cache (prompt processing)
     const int split = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
+    const int kv_seq = seq_fixed >= 0 ? seq_fixed : s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = nctx[s];
     const int tiles_total = (n + kTile - 1) / kTile;
@@ -45,7 +48,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
 #pragma unroll
     for (int v = 0; v < VEC; v++) o[v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
-    const int32_t* trow = table + (size_t)s * pages_per_seq;
+    const int32_t* trow = table + (size_t)kv_seq * pages_per_seq;
 
     for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
         const int nt = min(kTile, t_end - t0);
@@ -150,17 +153,40 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, float* __re
 
 }  // namespace
 
-// Shared with the decoder: attention over `kv` with per-sequence lengths read from nctx_dev (device).
-int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
-                    float* out_dev) {
+// Shared with the decoder.  n_queries query rows; row z attends to nctx_dev[z] tokens of sequence z
+// (seq_fixed < 0) or of sequence seq_fixed.  `partial` must hold n_queries * n_head * n_splits * (D + 2) floats.
+int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
+                       int seq_fixed, int n_splits, float* partial, float scale, float* out_dev) {
     const int D = kv->head_dim;
     SKN_REQUIRE(ctx, D == 64 || D == 128 || D == 256, SKN_ERR_SHAPE,
                 "skn_attn_decode: head_dim %d is not supported (64, 128 or 256)", D);
-    const int pairs = kv->n_seq * kv->n_head;
+    dim3 grid(n_splits, kv->n_head, n_queries), block(256);
+#define SKN_ATTN_LAUNCH(DD)                                                                                        \
+    skn_launch(ctx, attn_decode_split_kernel<DD>, grid, block, 0, kv->k_pool, kv->v_pool, kv->page_table_dev,     \
+               nctx_dev, q_dev, partial, kv->n_head, kv->page_tokens, kv->pages_per_seq, n_splits, scale, seq_fixed)
+    if (D == 64) SKN_ATTN_LAUNCH(64);
+    else if (D == 128) SKN_ATTN_LAUNCH(128);
+    else SKN_ATTN_LAUNCH(256);
+#undef SKN_ATTN_LAUNCH
+    SKN_LAUNCH_CHECK(ctx);
+    skn_launch(ctx, attn_merge_kernel, dim3(n_queries * kv->n_head), dim3(D), 0, (const float*)partial, out_dev,
+               n_splits, D);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+int skn_attn_splits(skn_ctx* ctx, int pairs, int max_ctx) {
     const int tiles = (max_ctx + kTile - 1) / kTile;
-    int n_splits = (4 * ctx->compute_units + pairs - 1) / pairs;
+    int n_splits = ctx->opt_attn_splits > 0 ? ctx->opt_attn_splits : (4 * ctx->compute_units + pairs - 1) / pairs;
     if (n_splits > tiles) n_splits = tiles;
-    if (n_splits < 1) n_splits = 1;
+    return n_splits < 1 ? 1 : n_splits;
+}
+
+int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
+                    float* out_dev) {
+    const int D = kv->head_dim;
+    const int pairs = kv->n_seq * kv->n_head;
+    const int n_splits = skn_attn_splits(ctx, pairs, max_ctx);
     const size_t need = (size_t)pairs * n_splits * (D + 2) * sizeof(float);
     if (need > ctx->attn_scratch_bytes) {
         SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -175,20 +201,8 @@ int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t*
         }
         ctx->attn_scratch_bytes = grow;
     }
-    float* partial = (float*)ctx->attn_scratch;
-    dim3 grid(n_splits, kv->n_head, kv->n_seq), block(256);
-#define SKN_ATTN_LAUNCH(DD)                                                                                           \
-    skn_launch(ctx, attn_decode_split_kernel<DD>, grid, block, 0, kv->k_pool, kv->v_pool,             \
-                       kv->page_table_dev, nctx_dev, q_dev, partial, kv->n_head, kv->page_tokens, kv->pages_per_seq,  \
-                       n_splits, scale)
-    if (D == 64) SKN_ATTN_LAUNCH(64);
-    else if (D == 128) SKN_ATTN_LAUNCH(128);
-    else SKN_ATTN_LAUNCH(256);
-#undef SKN_ATTN_LAUNCH
-    SKN_LAUNCH_CHECK(ctx);
-    skn_launch(ctx, attn_merge_kernel, dim3(pairs), dim3(D), 0, partial, out_dev, n_splits, D);
-    SKN_LAUNCH_CHECK(ctx);
-    return SKN_OK;
+    return skn_attn_launch_ex(ctx, kv, q_dev, nctx_dev, kv->n_seq, -1, n_splits, (float*)ctx->attn_scratch, scale,
+                              out_dev);
 }
 
 extern "C" int skn_attn_decode(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* n_ctx_host, float scale,

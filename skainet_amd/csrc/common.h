@@ -28,11 +28,17 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1;
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
+    // GEMM workspace (fp16 activations, dequantized weight pairs), grown on demand
+    void* gemm_ws = nullptr;
+    size_t gemm_ws_bytes = 0;
 };
+
+// One-time kernel attribute setup (large dynamic LDS), called by skn_init.
+int skn_matvec_init(skn_ctx* ctx);
 
 // Records a failure on the context (or on the context-less slot) and returns `code`.
 int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);

@@ -1,18 +1,524 @@
-// Llama-style decoder over the quantized kernels (placeholder entry points until the decoder lands).
+// Llama-style decoder over the quantized kernels: batched prompt processing (GEMM) and greedy decode (matvec)
+// for one sequence.  Per layer:  x += Wo . attn(rope(Wq xn), cache(rope(Wk xn), Wv xn)),  xn = rmsnorm(x);
+// x += Wdown . (silu(Wgate xn) * (Wup xn)).  Logits = Whead . rmsnorm(x).
+//
+// A decode step reads every scalar that changes from step to step (token id, position, context length, step
+// index) from device memory, so that one captured HIP graph of the ~480 kernel launches of a step can be
+// replayed for every token.  The graph holds kernels only (no memset / memcpy nodes).
 #include "kv.h"
 
+struct skn_llama {
+    skn_llama_config cfg;
+    skn_llama_weights w;
+    std::vector<skn_llama_layer> layers;
+    std::vector<skn_kv*> kv;  // one single-sequence cache per layer
+    // decode-step buffers
+    float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *att = nullptr, *proj = nullptr;
+    float *gate = nullptr, *up = nullptr, *mid = nullptr, *logits = nullptr, *attn_partial = nullptr;
+    int32_t* state = nullptr;       // [0] token, [1] position, [2] context length, [3] step index
+    int32_t* tokens_out = nullptr;  // device array of produced tokens
+    int tokens_cap = 0;
+    int pos = 0;                    // host mirror of the position
+    // prompt buffers (grown to the longest prompt seen)
+    int prompt_cap = 0;
+    float *px = nullptr, *pxn = nullptr, *pq = nullptr, *pk = nullptr, *pv = nullptr, *patt = nullptr, *pproj = nullptr;
+    float *pgate = nullptr, *pup = nullptr, *pmid = nullptr, *ppartial = nullptr;
+    uint16_t *pb16 = nullptr, *pk16 = nullptr, *pv16 = nullptr;
+    int32_t *ptok = nullptr, *pnctx = nullptr;
+    // captured decode step
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    int graph_splits = 0;
+    std::vector<void*> owned;
+};
+
+namespace {
+
+// ---- kernels that read their step-dependent scalars from device memory -----------------------------------
+
+// One row of a [vocab, hidden] quantized embedding table -> fp32.  grid = rows to embed, tokens from device.
+__global__ __launch_bounds__(256) void embed_rows_kernel(const uint8_t* __restrict__ table, int type, int hidden,
+                                                         const int32_t* __restrict__ tokens, float* __restrict__ out) {
+    const int row = blockIdx.x;
+    const int tok = tokens[row];
+    float* dst = out + (size_t)row * hidden;
+    if (type == SKN_TYPE_Q4_K) {
+        const uint8_t* src = table + (size_t)tok * (hidden / 256) * 144;
+        for (int e = threadIdx.x; e < hidden; e += 256) {
+            const uint8_t* b = src + (size_t)(e >> 8) * 144;
+            const int i = e & 255, c = i >> 6, r = i & 63, j = 2 * c + (r >= 32);
+            const uint8_t* s = b + 4;
+            int sc, m;
+            if (j < 4) {
+                sc = s[j] & 63;
+                m = s[j + 4] & 63;
+            } else {
+                sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+                m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+            }
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(b);
+            const uint8_t byte = b[16 + 32 * c + (r & 31)];
+            const int qv = (r < 32) ? (byte & 0xF) : (byte >> 4);
+            dst[e] = __fsub_rn(__fmul_rn(__fmul_rn(h2f_bits(dd & 0xFFFF), (float)sc), (float)qv),
+                               __fmul_rn(h2f_bits(dd >> 16), (float)m));
+        }
+    } else if (type == SKN_TYPE_Q8_0) {
+        const uint8_t* src = table + (size_t)tok * (hidden / 32) * 34;
+        for (int e = threadIdx.x; e < hidden; e += 256) {
+            const uint8_t* b = src + (size_t)(e >> 5) * 34;
+            dst[e] = __fmul_rn(h2f_bits(load_u16_a2(b)), (float)(int8_t)b[2 + (e & 31)]);
+        }
+    } else if (type == SKN_TYPE_Q6_K) {
+        const uint8_t* src = table + (size_t)tok * (hidden / 256) * 210;
+        for (int e = threadIdx.x; e < hidden; e += 256) {
+            const uint8_t* b = src + (size_t)(e >> 8) * 210;
+            const int i = e & 255, n = i >> 7, r = i & 127, quarter = r >> 5, l = r & 31;
+            uint32_t lo = b[64 * n + l + 32 * (quarter & 1)];
+            lo = quarter >= 2 ? lo >> 4 : lo & 0xF;
+            const uint32_t hi = (b[128 + 32 * n + l] >> (2 * quarter)) & 3;
+            const float sc = (float)(int8_t)b[192 + 8 * n + 2 * quarter + (l >> 4)];
+            dst[e] = __fmul_rn(__fmul_rn(h2f_bits(load_u16_a2(b + 208)), sc), (float)((int)(lo | (hi << 4)) - 32));
+        }
+    } else {  // F32
+        const float* src = reinterpret_cast<const float*>(table) + (size_t)tok * hidden;
+        for (int e = threadIdx.x; e < hidden; e += 256) dst[e] = src[e];
+    }
+}
+
+// Rotary embedding of q and k rows at positions pos0 + row (pos0 from device), then k and v rows go to the
+// cache as fp16 at those positions.  grid = (rows, n_head), block = head_dim / 2 threads (one pair each).
+__global__ void rope_store_kernel(float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                  uint16_t* __restrict__ k_pool, uint16_t* __restrict__ v_pool,
+                                  const int32_t* __restrict__ table, const int32_t* __restrict__ pos0_dev, int n_head,
+                                  int head_dim, int page_tokens, float log2_base) {
+    const int row = blockIdx.x, h = blockIdx.y, i = threadIdx.x;
+    const int pos = pos0_dev[0] + row;
+    const float inv_freq = exp2f(-2.0f * (float)i / (float)head_dim * log2_base);
+    float sn, cs;
+    sincosf((float)pos * inv_freq, &sn, &cs);
+    const size_t base = ((size_t)row * n_head + h) * head_dim + 2 * i;
+    const float qa = q[base], qb = q[base + 1];
+    q[base] = qa * cs - qb * sn;
+    q[base + 1] = qa * sn + qb * cs;
+    const float ka = k[base], kb = k[base + 1];
+    const float k0 = ka * cs - kb * sn, k1 = ka * sn + kb * cs;
+    const int page = table[pos / page_tokens];
+    const size_t dst = (((size_t)page * n_head + h) * page_tokens + (pos % page_tokens)) * head_dim + 2 * i;
+    const uint32_t kk = (uint32_t)__half_as_ushort(__float2half_rn(k0)) | ((uint32_t)__half_as_ushort(__float2half_rn(k1)) << 16);
+    const uint32_t vv = (uint32_t)__half_as_ushort(__float2half_rn(v[base])) |
+                        ((uint32_t)__half_as_ushort(__float2half_rn(v[base + 1])) << 16);
+    *reinterpret_cast<uint32_t*>(k_pool + dst) = kk;
+    *reinterpret_cast<uint32_t*>(v_pool + dst) = vv;
+}
+
+__global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ y,
+                                    int n, float eps) {
+    __shared__ float red[4];
+    const float* xr = x + (size_t)blockIdx.x * n;
+    float* yr = y + (size_t)blockIdx.x * n;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float r = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)n + eps);
+    for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * r * w[i];
+}
+
+__global__ void add_rows_kernel(float* __restrict__ y, const float* __restrict__ x, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] += x[i];
+}
+
+__global__ void swiglu_rows_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ out,
+                                   int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float a = g[i];
+        out[i] = a / (1.0f + expf(-a)) * u[i];
+    }
+}
+
+__global__ void f32_to_bf16_rows_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        uint32_t u = __float_as_uint(x[i]);
+        u += 0x7FFFu + ((u >> 16) & 1u);
+        out[i] = (uint16_t)(u >> 16);
+    }
+}
+
+// state = {token, position, context length, step}
+__global__ void set_state_kernel(int32_t* state, int token, int pos) {
+    if (threadIdx.x == 0) {
+        state[0] = token;
+        state[1] = pos;
+        state[2] = pos + 1;
+        state[3] = 0;
+    }
+}
+
+// single workgroup: argmax of the logits (first maximum) becomes the next token; the step's scalars advance
+__global__ __launch_bounds__(1024) void finish_step_kernel(const float* __restrict__ x, int n, int32_t* state,
+                                                           int32_t* __restrict__ tokens_out, int advance) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    float best = -INFINITY;
+    int besti = 0x7FFFFFFF;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float v = x[i];
+        if (v > best || (v == best && i < besti)) {
+            best = v;
+            besti = i;
+        }
+    }
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(besti, off, 64);
+        if (ov > best || (ov == best && oi < besti)) {
+            best = ov;
+            besti = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        bv[threadIdx.x >> 6] = best;
+        bi[threadIdx.x >> 6] = besti;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < besti)) {
+                best = bv[w];
+                besti = bi[w];
+            }
+        const int tok = besti == 0x7FFFFFFF ? 0 : besti;
+        if (advance) {
+            tokens_out[state[3]] = tok;
+            state[0] = tok;
+            state[1] += 1;
+            state[2] += 1;
+            state[3] += 1;
+        } else {
+            tokens_out[0] = tok;
+        }
+    }
+}
+
+__global__ void iota_kernel(int32_t* out, int n, int start) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = start + i;
+}
+
+template <typename T>
+int dev_alloc(skn_ctx* ctx, skn_llama* m, T** p, size_t count) {
+    hipError_t e = hipMalloc((void**)p, count * sizeof(T) < 16 ? 16 : count * sizeof(T));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return skn_fail(ctx, SKN_ERR_OOM, "skn_llama: %zu bytes: %s", count * sizeof(T), hipGetErrorString(e));
+    }
+    m->owned.push_back((void*)*p);
+    return SKN_OK;
+}
+
+unsigned nblk(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+#define SKN_TRY(expr)              \
+    do {                           \
+        int rc_ = (expr);          \
+        if (rc_ != SKN_OK) return rc_; \
+    } while (0)
+
+// the launches of one decode step (eagerly or under stream capture)
+int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
+    const skn_llama_config& c = m->cfg;
+    const int H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim;
+    const float scale = 1.0f / sqrtf((float)D);
+    skn_launch(ctx, embed_rows_kernel, dim3(1), dim3(256), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
+               (const int32_t*)m->state, m->x);
+    SKN_LAUNCH_CHECK(ctx);
+    for (int l = 0; l < c.n_layer; l++) {
+        const skn_llama_layer& L = m->layers[l];
+        skn_kv* kv = m->kv[l];
+        skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wq, H, H, m->xn, m->q));
+        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wk, H, H, m->xn, m->k));
+        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wv, H, H, m->xn, m->v));
+        skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
+                   kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                   kv->page_tokens, log2f(c.rope_base));
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, scale, m->att));
+        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wo, H, H, m->att, m->proj));
+        skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
+        SKN_LAUNCH_CHECK(ctx);
+        skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.ffn_norm, m->xn, H, c.rms_eps);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_gate, F, H, m->xn, m->gate));
+        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_up, F, H, m->xn, m->up));
+        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk(F)), dim3(256), 0, (const float*)m->gate, (const float*)m->up,
+                   m->mid, (int64_t)F);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_down, H, F, m->mid, m->proj));
+        skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
+        SKN_LAUNCH_CHECK(ctx);
+    }
+    skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, m->w.out_norm, m->xn, H, c.rms_eps);
+    SKN_LAUNCH_CHECK(ctx);
+    SKN_TRY(skn_matvec_q(ctx, m->w.type_head, m->w.out_head, c.vocab, H, m->xn, m->logits));
+    skn_launch(ctx, finish_step_kernel, dim3(1), dim3(1024), 0, (const float*)m->logits, c.vocab, m->state,
+               m->tokens_out, 1);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+void drop_graph(skn_llama* m) {
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    m->graph_exec = nullptr;
+    m->graph = nullptr;
+    m->graph_splits = 0;
+}
+
+int ensure_prompt_buffers(skn_ctx* ctx, skn_llama* m, int T) {
+    if (T <= m->prompt_cap) return SKN_OK;
+    const skn_llama_config& c = m->cfg;
+    const size_t H = c.hidden, F = c.ffn;
+    // earlier, smaller prompt buffers stay owned by the model until it is freed
+    SKN_TRY(dev_alloc(ctx, m, &m->px, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pxn, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pq, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pk, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pv, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->patt, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pproj, T * H));
+    SKN_TRY(dev_alloc(ctx, m, &m->pgate, T * F));
+    SKN_TRY(dev_alloc(ctx, m, &m->pup, T * F));
+    SKN_TRY(dev_alloc(ctx, m, &m->pmid, T * F));
+    SKN_TRY(dev_alloc(ctx, m, &m->pb16, T * (F > H ? F : H)));
+    SKN_TRY(dev_alloc(ctx, m, &m->ptok, (size_t)T));
+    SKN_TRY(dev_alloc(ctx, m, &m->pnctx, (size_t)T));
+    // splits = ceil(4 * CUs / pairs) bounds pairs * splits by pairs + 4 * CUs
+    SKN_TRY(dev_alloc(ctx, m, &m->ppartial, ((size_t)T * c.n_head + 4 * (size_t)ctx->compute_units) * (c.head_dim + 2)));
+    m->prompt_cap = T;
+    return SKN_OK;
+}
+
+int to_bf16(skn_ctx* ctx, const float* x, uint16_t* out, int64_t n) {
+    skn_launch(ctx, f32_to_bf16_rows_kernel, dim3(nblk(n)), dim3(256), 0, x, out, n);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+}  // namespace
+
 extern "C" {
-int skn_llama_create(skn_ctx* ctx, const skn_llama_config*, const skn_llama_weights*, skn_llama** out) {
-    if (out) *out = nullptr;
-    return skn_fail(ctx, SKN_ERR_STATE, "skn_llama_create: decoder not built");
+
+int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_weights* w, skn_llama** out) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_create: ctx is null");
+    SKN_REQUIRE(ctx, cfg && w && out, SKN_ERR_ARG, "skn_llama_create: null pointer");
+    *out = nullptr;
+    SKN_REQUIRE(ctx, cfg->n_layer > 0 && cfg->hidden > 0 && cfg->ffn > 0 && cfg->n_head > 0 && cfg->head_dim > 0 &&
+                         cfg->vocab > 0 && cfg->max_tokens > 0 && cfg->page_tokens > 0,
+                SKN_ERR_ARG, "skn_llama_create: sizes must be positive");
+    SKN_REQUIRE(ctx, cfg->n_head * cfg->head_dim == cfg->hidden, SKN_ERR_SHAPE,
+                "skn_llama_create: n_head * head_dim (%d) must equal hidden (%d)", cfg->n_head * cfg->head_dim,
+                cfg->hidden);
+    SKN_REQUIRE(ctx, cfg->head_dim == 64 || cfg->head_dim == 128 || cfg->head_dim == 256, SKN_ERR_SHAPE,
+                "skn_llama_create: head_dim %d is not supported (64, 128 or 256)", cfg->head_dim);
+    SKN_REQUIRE(ctx, cfg->hidden % 256 == 0 && cfg->ffn % 256 == 0, SKN_ERR_SHAPE,
+                "skn_llama_create: hidden and ffn must be multiples of 256");
+    SKN_REQUIRE(ctx, w->layers && w->tok_embd && w->out_norm && w->out_head, SKN_ERR_ARG,
+                "skn_llama_create: missing weights");
+    SKN_REQUIRE(ctx, (skn_is_quant(w->type_embd) || w->type_embd == SKN_TYPE_F32) && skn_is_quant(w->type_head),
+                SKN_ERR_TYPE, "skn_llama_create: unsupported embedding / head type");
+    for (int l = 0; l < cfg->n_layer; l++) {
+        const skn_llama_layer& L = w->layers[l];
+        SKN_REQUIRE(ctx, L.wq && L.wk && L.wv && L.wo && L.w_gate && L.w_up && L.w_down && L.attn_norm && L.ffn_norm,
+                    SKN_ERR_ARG, "skn_llama_create: layer %d has a null weight", l);
+        SKN_REQUIRE(ctx, skn_is_quant(L.type_attn) && skn_is_quant(L.type_ffn), SKN_ERR_TYPE,
+                    "skn_llama_create: layer %d has an unsupported weight type", l);
+    }
+    skn_llama* m = new (std::nothrow) skn_llama();
+    SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_OOM, "skn_llama_create: host allocation failed");
+    m->cfg = *cfg;
+    m->w = *w;
+    m->layers.assign(w->layers, w->layers + cfg->n_layer);
+    m->w.layers = m->layers.data();
+    int rc = SKN_OK;
+    for (int l = 0; l < cfg->n_layer && rc == SKN_OK; l++) {
+        skn_kv* kv = nullptr;
+        rc = skn_kv_create(ctx, 1, cfg->n_head, cfg->head_dim, cfg->page_tokens, cfg->max_tokens, &kv);
+        if (rc == SKN_OK) m->kv.push_back(kv);
+    }
+    const size_t H = cfg->hidden, F = cfg->ffn;
+    const int max_splits = (cfg->max_tokens + 63) / 64;
+    auto A = [&](auto** p, size_t n) {
+        if (rc == SKN_OK) rc = dev_alloc(ctx, m, p, n);
+    };
+    A(&m->x, H); A(&m->xn, H); A(&m->q, H); A(&m->k, H); A(&m->v, H); A(&m->att, H); A(&m->proj, H);
+    A(&m->gate, F); A(&m->up, F); A(&m->mid, F); A(&m->logits, (size_t)cfg->vocab);
+    A(&m->attn_partial, (size_t)cfg->n_head * max_splits * (cfg->head_dim + 2));
+    A(&m->state, (size_t)4);
+    m->tokens_cap = cfg->max_tokens;
+    A(&m->tokens_out, (size_t)m->tokens_cap);
+    if (rc != SKN_OK) {
+        skn_llama_free(ctx, m);
+        return rc;
+    }
+    *out = m;
+    return SKN_OK;
 }
-int skn_llama_free(skn_ctx* ctx, skn_llama*) { return skn_fail(ctx, SKN_ERR_STATE, "decoder not built"); }
-int skn_llama_reset(skn_ctx* ctx, skn_llama*) { return skn_fail(ctx, SKN_ERR_STATE, "decoder not built"); }
-int skn_llama_prefill(skn_ctx* ctx, skn_llama*, const int32_t*, int, int32_t*) {
-    return skn_fail(ctx, SKN_ERR_STATE, "decoder not built");
+
+int skn_llama_free(skn_ctx* ctx, skn_llama* m) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_free: ctx is null");
+    if (!m) return SKN_OK;
+    (void)hipStreamSynchronize(ctx->stream);
+    drop_graph(m);
+    for (skn_kv* kv : m->kv) skn_kv_free(ctx, kv);
+    for (void* p : m->owned) (void)hipFree(p);
+    delete m;
+    return SKN_OK;
 }
-int skn_llama_decode(skn_ctx* ctx, skn_llama*, int32_t, int, int32_t*) {
-    return skn_fail(ctx, SKN_ERR_STATE, "decoder not built");
+
+int skn_llama_reset(skn_ctx* ctx, skn_llama* m) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_reset: ctx is null");
+    SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_ARG, "skn_llama_reset: model is null");
+    for (skn_kv* kv : m->kv) SKN_TRY(skn_kv_reset(ctx, kv, 0));
+    m->pos = 0;
+    return SKN_OK;
 }
-int skn_llama_logits(skn_ctx* ctx, skn_llama*, const float**) { return skn_fail(ctx, SKN_ERR_STATE, "decoder not built"); }
+
+int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, int n_tokens, int32_t* next_token_host) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_prefill: ctx is null");
+    SKN_REQUIRE(ctx, m && tokens_host, SKN_ERR_ARG, "skn_llama_prefill: null pointer");
+    SKN_REQUIRE(ctx, n_tokens > 0, SKN_ERR_ARG, "skn_llama_prefill: the prompt is empty");
+    const skn_llama_config& c = m->cfg;
+    SKN_REQUIRE(ctx, m->pos + n_tokens <= c.max_tokens, SKN_ERR_POOL, "sequence is full (%d tokens, capacity %d)",
+                m->pos + n_tokens, c.max_tokens);
+    for (int i = 0; i < n_tokens; i++)
+        SKN_REQUIRE(ctx, tokens_host[i] >= 0 && tokens_host[i] < c.vocab, SKN_ERR_RANGE,
+                    "skn_llama_prefill: token %d of a vocabulary of %d", tokens_host[i], c.vocab);
+    const int T = n_tokens, H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim, pos0 = m->pos;
+    SKN_TRY(ensure_prompt_buffers(ctx, m, T));
+    SKN_HIP(ctx, hipMemcpyAsync(m->ptok, tokens_host, (size_t)T * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    skn_launch(ctx, set_state_kernel, dim3(1), dim3(64), 0, m->state, 0, pos0);
+    SKN_LAUNCH_CHECK(ctx);
+    skn_launch(ctx, iota_kernel, dim3(nblk(T)), dim3(256), 0, m->pnctx, T, pos0 + 1);
+    SKN_LAUNCH_CHECK(ctx);
+    skn_launch(ctx, embed_rows_kernel, dim3(T), dim3(256), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
+               (const int32_t*)m->ptok, m->px);
+    SKN_LAUNCH_CHECK(ctx);
+    const float scale = 1.0f / sqrtf((float)D);
+    int n_splits = (4 * ctx->compute_units + T * NH - 1) / (T * NH);
+    if (n_splits > (pos0 + T + 63) / 64) n_splits = (pos0 + T + 63) / 64;
+    for (int l = 0; l < c.n_layer; l++) {
+        const skn_llama_layer& L = m->layers[l];
+        skn_kv* kv = m->kv[l];
+        SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
+        skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
+        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wq, H, H, m->pb16, T, m->pq));
+        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wk, H, H, m->pb16, T, m->pk));
+        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wv, H, H, m->pb16, T, m->pv));
+        skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
+                   kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                   kv->page_tokens, log2f(c.rope_base));
+        SKN_LAUNCH_CHECK(ctx);
+        // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, scale, m->patt));
+        SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
+        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
+        skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
+                   (int64_t)T * H);
+        SKN_LAUNCH_CHECK(ctx);
+        skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
+        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_gate, F, H, m->pb16, T, m->pgate));
+        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_up, F, H, m->pb16, T, m->pup));
+        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                   (const float*)m->pup, m->pmid, (int64_t)T * F);
+        SKN_LAUNCH_CHECK(ctx);
+        SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
+        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_down, H, F, m->pb16, T, m->pproj));
+        skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
+                   (int64_t)T * H);
+        SKN_LAUNCH_CHECK(ctx);
+        // the cache of this layer now holds pos0 + T tokens
+        kv->len[0] = pos0 + T;
+    }
+    // logits of the last prompt token only
+    skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)(m->px + (size_t)(T - 1) * H),
+               m->w.out_norm, m->xn, H, c.rms_eps);
+    SKN_LAUNCH_CHECK(ctx);
+    SKN_TRY(skn_matvec_q(ctx, m->w.type_head, m->w.out_head, c.vocab, H, m->xn, m->logits));
+    skn_launch(ctx, finish_step_kernel, dim3(1), dim3(1024), 0, (const float*)m->logits, c.vocab, m->state,
+               m->tokens_out, 0);
+    SKN_LAUNCH_CHECK(ctx);
+    m->pos = pos0 + T;
+    int32_t next = 0;
+    SKN_HIP(ctx, hipMemcpyAsync(&next, m->tokens_out, sizeof(int32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (next_token_host) *next_token_host = next;
+    return SKN_OK;
 }
+
+int skn_llama_decode(skn_ctx* ctx, skn_llama* m, int32_t first_token, int n_steps, int32_t* tokens_out_host) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_decode: ctx is null");
+    SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_ARG, "skn_llama_decode: model is null");
+    SKN_REQUIRE(ctx, n_steps >= 0, SKN_ERR_ARG, "skn_llama_decode: negative step count");
+    if (n_steps == 0) return SKN_OK;
+    const skn_llama_config& c = m->cfg;
+    SKN_REQUIRE(ctx, tokens_out_host != nullptr, SKN_ERR_ARG, "skn_llama_decode: tokens_out is null");
+    SKN_REQUIRE(ctx, first_token >= 0 && first_token < c.vocab, SKN_ERR_RANGE,
+                "skn_llama_decode: token %d of a vocabulary of %d", first_token, c.vocab);
+    SKN_REQUIRE(ctx, m->pos + n_steps <= c.max_tokens, SKN_ERR_POOL, "sequence is full (%d tokens, capacity %d)",
+                m->pos + n_steps, c.max_tokens);
+    SKN_REQUIRE(ctx, !ctx->prof_on, SKN_ERR_STATE, "skn_llama_decode: not available while per-launch timing is on");
+    // every page the run will touch is mapped now; the step itself never talks to the host
+    for (skn_kv* kv : m->kv) SKN_TRY(skn_kv_reserve(ctx, kv, 0, m->pos + n_steps));
+    skn_launch(ctx, set_state_kernel, dim3(1), dim3(64), 0, m->state, (int)first_token, m->pos);
+    SKN_LAUNCH_CHECK(ctx);
+    // a fixed split count that suits the longest context of this run (the kernel derives its ranges from the
+    // actual length, so one captured step serves every position)
+    const int n_splits = skn_attn_splits(ctx, c.n_head, m->pos + n_steps);
+    if (ctx->opt_llama_graph == 0) {
+        for (int i = 0; i < n_steps; i++) SKN_TRY(decode_step(ctx, m, n_splits));
+    } else {
+        if (m->graph_exec && m->graph_splits != n_splits) drop_graph(m);
+        if (!m->graph_exec) {
+            SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+            SKN_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+            int rc = decode_step(ctx, m, n_splits);
+            hipGraph_t g = nullptr;
+            hipError_t e = hipStreamEndCapture(ctx->stream, &g);
+            if (rc != SKN_OK) {
+                if (g) (void)hipGraphDestroy(g);
+                return rc;
+            }
+            if (e != hipSuccess) return skn_fail(ctx, SKN_ERR_HIP, "stream capture failed: %s", hipGetErrorString(e));
+            m->graph = g;
+            SKN_HIP(ctx, hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+            m->graph_splits = n_splits;
+        }
+        for (int i = 0; i < n_steps; i++) SKN_HIP(ctx, hipGraphLaunch(m->graph_exec, ctx->stream));
+    }
+    SKN_HIP(ctx, hipMemcpyAsync(tokens_out_host, m->tokens_out, (size_t)n_steps * sizeof(int32_t), hipMemcpyDeviceToHost,
+                                ctx->stream));
+    SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    m->pos += n_steps;
+    for (skn_kv* kv : m->kv) kv->len[0] = m->pos;
+    return SKN_OK;
+}
+
+int skn_llama_logits(skn_ctx* ctx, skn_llama* m, const float** logits_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_logits: ctx is null");
+    SKN_REQUIRE(ctx, m && logits_dev, SKN_ERR_ARG, "skn_llama_logits: null pointer");
+    *logits_dev = m->logits;
+    return SKN_OK;
+}
+
+}  // extern "C"

@@ -28,7 +28,6 @@ namespace {
 //
 //   y = 2^24 * sum_blocks [ d * (sc_lo * A_lo + sc_hi * A_hi) - dmin * (m_lo * S_lo + m_hi * S_hi) ]
 
-constexpr int kQ4kBlockBytes = 144;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 // 6-bit scales / mins of sub-blocks 2p and 2p+1 out of the header chunk h = (d|dmin, scales[0..3], [4..7], [8..11]).
@@ -177,7 +176,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
         rp[r] = reinterpret_cast<const uint4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + 1 + 2 * p;
     }
-    auto issue = [&](int s, int tie, Q4kLoads (&L)[R]) {
+    auto issue = [&](int s, int tie, Q4kLoads (&L)[R]) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
         const int off = min(blk, nb - 1) * 9 + tie;
 #pragma unroll
@@ -306,9 +305,6 @@ int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, fl
     SKN_REQUIRE(ctx, lds <= 160 * 1024, SKN_ERR_SHAPE, "skn_matvec_q: k = %d needs %zu bytes of LDS (limit 163840)",
                 nb * 256, lds);
     auto kern = matvec_q4k_kernel<STEPS, R>;
-    if (lds > 48 * 1024)
-        SKN_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds));
     const int rows_per_wg = waves * R;
     dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block((unsigned)(waves * 64));
     skn_launch(ctx, kern, grid, block, lds, w, x, y, n, nb);
@@ -327,7 +323,24 @@ int dispatch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, 
     }
 }
 
+template <int STEPS, int R>
+hipError_t allow_big_lds() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
 }  // namespace
+
+// Dynamic LDS above 48 KiB must be allowed per kernel; done once here so that no launch path (which may run under
+// stream capture) has to.
+int skn_matvec_init(skn_ctx* ctx) {
+    hipError_t (*fns[])() = {allow_big_lds<0, 1>, allow_big_lds<1, 1>, allow_big_lds<2, 1>, allow_big_lds<3, 1>,
+                             allow_big_lds<4, 1>, allow_big_lds<0, 2>, allow_big_lds<1, 2>, allow_big_lds<2, 2>,
+                             allow_big_lds<3, 2>, allow_big_lds<4, 2>, allow_big_lds<0, 4>, allow_big_lds<1, 4>,
+                             allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>};
+    for (auto f : fns) SKN_HIP(ctx, f());
+    return SKN_OK;
+}
 
 extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev,
                             float* y_dev) {

@@ -1,0 +1,127 @@
+"""Host side of the Llama-style decoder: seeded random-init GGUF-block weights, upload, prefill and greedy decode.
+
+The module graph is the reference's nested Module.forward composition (core/src/commonMain/kotlin/sk/ai/net/nn/
+Module.kt:6-16, nn/topology/MLP.kt:13-19) instantiated for a Llama block stack; every Linear
+(nn/Linear.kt:43-49, y = x . W^T, no bias here) holds a quantized [out, in] weight on the device.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import runtime, synth
+from .runtime import Q4_K, Q6_K, LlamaConfig, LlamaLayer, LlamaWeights
+
+
+@dataclass
+class Config:
+    n_layer: int = 32
+    hidden: int = 4096
+    ffn: int = 11008
+    n_head: int = 32
+    head_dim: int = 128
+    vocab: int = 32000
+    max_tokens: int = 1024
+    page_tokens: int = 256
+    rope_base: float = 10000.0
+    rms_eps: float = 1e-5
+    type_attn: int = Q4_K
+    type_ffn: int = Q4_K
+    type_embd: int = Q4_K
+    type_head: int = Q6_K
+
+
+LLAMA_7B = Config()
+
+
+def random_weights(cfg: Config, seed: int):
+    """Host copy of a seeded random-init model: dict name -> (ggml type or None for fp32, ndarray)."""
+    h, f, v = cfg.hidden, cfg.ffn, cfg.vocab
+    w = {}
+    rng = np.random.default_rng(seed)
+    w["tok_embd"] = (cfg.type_embd, synth.weight(cfg.type_embd, v, h, seed + 1))
+    w["out_head"] = (cfg.type_head, synth.weight(cfg.type_head, v, h, seed + 2))
+    w["out_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+    for l in range(cfg.n_layer):
+        s = seed + 100 * (l + 1)
+        for i, name in enumerate(("wq", "wk", "wv", "wo")):
+            w[f"l{l}.{name}"] = (cfg.type_attn, synth.weight(cfg.type_attn, h, h, s + i))
+        w[f"l{l}.w_gate"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, f, h, s + 10))
+        w[f"l{l}.w_up"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, f, h, s + 11))
+        w[f"l{l}.w_down"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, h, f, s + 12))
+        w[f"l{l}.attn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+        w[f"l{l}.ffn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+    return w
+
+
+class LlamaModel:
+    """Device-resident model: owns the uploaded weights and the skn_llama handle."""
+
+    def __init__(self, ctx: runtime.Context, cfg: Config, weights=None, seed: int = 0, share_layers: bool = False):
+        """share_layers=True uploads one layer's weights and points every layer at them (shape-faithful timing
+        of a model larger than one wants to generate on the host; never used for parity)."""
+        self.ctx, self.cfg = ctx, cfg
+        self.bufs = {}
+        if weights is None:
+            gen_cfg = cfg if not share_layers else Config(**{**cfg.__dict__, "n_layer": 1})
+            weights = random_weights(gen_cfg, seed)
+        self.host_weights = weights if not share_layers else None
+        for name, (_, arr) in weights.items():
+            self.bufs[name] = ctx.to_device(arr)
+        layers = (LlamaLayer * cfg.n_layer)()
+        for l in range(cfg.n_layer):
+            src = 0 if share_layers else l
+            L = layers[l]
+            for f in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "attn_norm", "ffn_norm"):
+                setattr(L, f, self.bufs[f"l{src}.{f}"].ptr)
+            L.type_attn, L.type_ffn = cfg.type_attn, cfg.type_ffn
+        self._layers = layers
+        wts = LlamaWeights(self.bufs["tok_embd"].ptr, self.bufs["out_norm"].ptr, self.bufs["out_head"].ptr,
+                           cfg.type_embd, cfg.type_head, layers)
+        c = LlamaConfig(cfg.n_layer, cfg.hidden, cfg.ffn, cfg.n_head, cfg.head_dim, cfg.vocab, cfg.max_tokens,
+                        cfg.page_tokens, cfg.rope_base, cfg.rms_eps)
+        h = C.c_void_p()
+        ctx._check(ctx.lib.skn_llama_create(ctx.handle, C.byref(c), C.byref(wts), C.byref(h)))
+        self.handle = h.value
+
+    def reset(self):
+        self.ctx._check(self.ctx.lib.skn_llama_reset(self.ctx.handle, self.handle))
+
+    def prefill(self, tokens):
+        arr = (C.c_int32 * len(tokens))(*[int(t) for t in tokens])
+        nxt = C.c_int32()
+        self.ctx._check(self.ctx.lib.skn_llama_prefill(self.ctx.handle, self.handle, arr, len(tokens), C.byref(nxt)))
+        return nxt.value
+
+    def decode(self, first_token, n_steps):
+        out = (C.c_int32 * max(n_steps, 1))()
+        self.ctx._check(self.ctx.lib.skn_llama_decode(self.ctx.handle, self.handle, int(first_token), n_steps, out))
+        return list(out[:n_steps])
+
+    def logits(self):
+        p = C.c_void_p()
+        self.ctx._check(self.ctx.lib.skn_llama_logits(self.ctx.handle, self.handle, C.byref(p)))
+        out = np.empty(self.cfg.vocab, dtype=np.float32)
+        self.ctx._check(self.ctx.lib.skn_download(self.ctx.handle, out.ctypes.data, p.value, out.nbytes))
+        return out
+
+    def free(self):
+        if self.handle:
+            self.ctx.lib.skn_llama_free(self.ctx.handle, self.handle)
+            self.handle = None
+        for b in self.bufs.values():
+            b.free()
+        self.bufs = {}
+
+    def weight_bytes_per_token(self):
+        """Bytes of weights one decode step streams (embedding row excluded): the HBM floor of a token."""
+        c = self.cfg
+
+        def rb(t, n, k):
+            be, bb = synth.BLOCK[t]
+            return n * (k // be) * bb
+
+        per_layer = 4 * rb(c.type_attn, c.hidden, c.hidden) + 2 * rb(c.type_ffn, c.ffn, c.hidden) + rb(c.type_ffn, c.hidden, c.ffn)
+        return c.n_layer * per_layer + rb(c.type_head, c.vocab, c.hidden)

@@ -1,0 +1,87 @@
+"""GPU parity: batched quantized GEMM (bf16 activations, fp32 out) through the C ABI vs the fp64-accumulated oracle."""
+import numpy as np
+import pytest
+
+from oracle import oracle_c, oracle_np
+from skainet_amd import runtime, synth
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+TOL = 1e-3  # max |a - r| / max(|r|, 1e-3 * max|r|)
+
+
+@pytest.mark.parametrize(
+    "qtype,m,n,k",
+    [
+        (Q4_K, 512, 256, 4096),
+        (Q6_K, 512, 256, 4096),
+        (Q8_0, 64, 128, 1024),
+        (Q4_K, 1, 64, 256),       # a single activation row
+        (Q4_K, 33, 100, 768),     # ragged in m and n
+        (Q6_K, 130, 65, 512),
+        (Q4_K, 200, 192, 11008),  # the FFN-down row length (43 superblocks)
+    ],
+)
+def test_gemm_vs_oracle(hip, qtype, m, n, k):
+    raw = synth.weight(qtype, n, k, seed=3 * n + k + qtype)
+    a = synth.activation_bf16((m, k), seed=m + 17)
+    got = hip.gemm_q_host(qtype, raw, n, k, a, m)
+    want = oracle_c.gemm_q(qtype, raw, n, k, a, m)
+    err = oracle_np.rel_err(got, want)
+    assert err <= TOL, f"rel err {err}"
+
+
+@pytest.mark.parametrize("qtype", [Q4_K, Q6_K])
+def test_gemm_rows_match_matvec(hip, qtype):
+    m, n, k = 8, 128, 2048
+    raw = synth.weight(qtype, n, k, seed=77)
+    a = synth.activation_bf16((m, k), seed=78)
+    c = hip.gemm_q_host(qtype, raw, n, k, a, m)
+    af = oracle_np.bf16_to_f32(a).reshape(m, k)
+    for r in range(m):
+        y = hip.matvec_q_host(qtype, raw, n, k, af[r])
+        assert oracle_np.rel_err(c[r], y) <= TOL
+
+
+def test_gemm_large_activations_are_rescaled(hip):
+    # rows far outside fp16 range (|a| up to ~1e6) and tiny rows must both come out right
+    m, n, k = 4, 64, 1024
+    raw = synth.weight(Q4_K, n, k, seed=5)
+    x = np.random.default_rng(6).standard_normal((m, k)).astype(np.float32)
+    x[0] *= 3.0e5
+    x[1] *= 1.0e-3
+    x[2, 17] = 9.0e5
+    a = synth.f32_to_bf16_bits(x)
+    got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    want = oracle_c.gemm_q(Q4_K, raw, n, k, a, m)
+    for r in range(m):
+        assert oracle_np.rel_err(got[r], want[r]) <= TOL, r
+
+
+def test_gemm_full_width_slice(hip):
+    """The benchmark shape M=512, K=4096 at N=4096: checked on a strided sample of the oracle's columns."""
+    m, n, k = 512, 4096, 4096
+    raw = synth.weight(Q4_K, n, k, seed=9)
+    a = synth.activation_bf16((m, k), seed=10)
+    got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    rows = np.arange(0, n, 61)
+    rb = raw.reshape(n, -1)[rows].reshape(-1)
+    want = oracle_c.gemm_q(Q4_K, rb, len(rows), k, a, m)
+    # normalise with the whole output's scale, as the metric is defined over the full result
+    floor = 1e-3 * np.abs(got).max()
+    err = np.max(np.abs(got[:, rows] - want) / np.maximum(np.abs(want), floor))
+    assert err <= TOL, err
+
+
+def test_gemm_errors(hip):
+    buf = hip.alloc(1 << 16)
+    with pytest.raises(runtime.SknError) as e:
+        hip.gemm_q(Q4_K, buf, 4, 200, buf, 2, buf)
+    assert e.value.code == runtime.ERR_SHAPE
+    with pytest.raises(runtime.SknError) as e:
+        hip.gemm_q(3, buf, 4, 256, buf, 2, buf)
+    assert e.value.code == runtime.ERR_TYPE
+    with pytest.raises(runtime.SknError) as e:
+        hip.gemm_q(Q4_K, None, 4, 256, buf, 2, buf)
+    assert e.value.code == runtime.ERR_ARG
+    hip.gemm_q(Q4_K, buf, 4, 256, buf, 0, buf)  # no activation rows: nothing to do
