@@ -174,6 +174,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--mode", choices=["bench", "copy"], default="bench",
+                    help="copy: run --steps plain device copies of the headline weight size instead (the known-size "
+                         "workload that hardware traffic counters are calibrated against)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -182,6 +185,19 @@ def main():
     ctx = runtime.Context(0)
     info = ctx.device_info()
     n, k = 4096, 11008
+    if args.mode == "copy":
+        nbytes = n * (k // 256) * 144
+        srcs = [ctx.to_device(synth.weight(Q4_K, n, k, seed=1234 + c)) for c in range(N_COPIES)]
+        dst = ctx.alloc(nbytes)
+        ctx.prof_start(args.steps)
+        for i in range(args.steps):
+            ctx.copy(dst, srcs[i % N_COPIES], nbytes)
+        ms, launches = ctx.prof_stop()
+        print(json.dumps({"mode": "copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": launches,
+                          "kernel": "copy16_kernel", "kernel_us": round(ms / launches * 1e3, 3),
+                          "read_plus_write_gbs": round(2 * nbytes / (ms / launches * 1e-3) / 1e9, 1)}))
+        ctx.close()
+        return
     head = bench_matvec(ctx, Q4_K, n, k, args.steps, args.warmup)
 
     extra = {"device": info["name"], "compute_units": info["compute_units"]}

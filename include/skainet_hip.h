@@ -79,6 +79,8 @@ int skn_free(skn_ctx* ctx, void* dev);
 int skn_upload(skn_ctx* ctx, void* dev, const void* host, size_t bytes);
 int skn_download(skn_ctx* ctx, void* host, const void* dev, size_t bytes);
 int skn_memset(skn_ctx* ctx, void* dev, int byte_value, size_t bytes);
+/* Device-to-device copy by a streaming kernel on the context's stream (ranges must not overlap). */
+int skn_copy(skn_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
 int skn_sync(skn_ctx* ctx);
 /* Adopt a caller-owned hipStream_t (NULL restores the context's own stream). */
 int skn_set_stream(skn_ctx* ctx, void* hip_stream);

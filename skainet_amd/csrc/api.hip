@@ -177,6 +177,39 @@ int skn_memset(skn_ctx* ctx, void* dev, int byte_value, size_t bytes) {
     return SKN_OK;
 }
 
+__global__ __launch_bounds__(256) void copy16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+__global__ void copy_bytes_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
+
+int skn_copy(skn_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_copy: ctx is null");
+    if (bytes == 0) return SKN_OK;
+    SKN_REQUIRE(ctx, dst_dev && src_dev, SKN_ERR_ARG, "skn_copy: null pointer");
+    // a plain streaming kernel (128-bit loads and stores when both ends are 16-byte aligned); it doubles as the
+    // known-size workload against which hardware traffic counters are calibrated
+    if ((((uintptr_t)dst_dev | (uintptr_t)src_dev | bytes) & 15) == 0) {
+        const size_t n16 = bytes / 16;
+        size_t blocks = (n16 + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        skn_launch(ctx, copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, (const uint4*)src_dev, (uint4*)dst_dev, n16);
+    } else {
+        size_t blocks = (bytes + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        skn_launch(ctx, copy_bytes_kernel, dim3((unsigned)blocks), dim3(256), 0, (const uint8_t*)src_dev,
+                   (uint8_t*)dst_dev, bytes);
+    }
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
 int skn_sync(skn_ctx* ctx) {
     SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_sync: ctx is null");
     SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));

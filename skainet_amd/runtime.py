@@ -65,6 +65,7 @@ _SIGNATURES = {
     "skn_upload": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "skn_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "skn_memset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t]),
+    "skn_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "skn_sync": (C.c_int, [C.c_void_p]),
     "skn_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
@@ -271,6 +272,9 @@ class Context:
 
     def sync(self):
         self._check(self.lib.skn_sync(self.handle))
+
+    def copy(self, dst_dev, src_dev, nbytes):
+        self._check(self.lib.skn_copy(self.handle, _ptr(dst_dev), _ptr(src_dev), nbytes))
 
     def set_stream(self, stream_ptr):
         self._check(self.lib.skn_set_stream(self.handle, stream_ptr))
