@@ -1,0 +1,100 @@
+"""GPU: the reference-shaped tensor wrappers (QuantizedTensor / DeviceTensor / QuantizedLinear) and a GGUF file
+loaded to the device end to end.  The known answers are the reference's own TensorTest matmul cases, carried
+through Q8_0 weights that represent them exactly."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle_c, oracle_np
+from skainet_amd import gguf, synth
+from skainet_amd.tensor import DeviceTensor, QuantizedLinear, QuantizedTensor, Shape
+
+pytestmark = pytest.mark.gpu
+
+
+def _q8_exact(rows):
+    """[n, k<=32-multiple] small-integer matrix -> Q8_0 bytes holding it exactly (d = 1)."""
+    rows = np.asarray(rows)
+    n, k = rows.shape
+    kp = -(-k // 32) * 32
+    q = np.zeros((n, kp), dtype=np.int8)
+    q[:, :k] = rows
+    blocks = np.zeros((n, kp // 32, 34), dtype=np.uint8)
+    blocks[:, :, 0:2] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    blocks[:, :, 2:] = q.reshape(n, kp // 32, 32).view(np.uint8)
+    return blocks.reshape(-1), kp
+
+
+def test_reference_matmul_known_answers_through_quantized_weights(hip, golden_dir):
+    cases = json.load(open(os.path.join(golden_dir, "tensor_test_vectors.json")))["cases"]
+    # TensorTest.kt:39-45: [1,2] . [[1,2,3],[4,5,6]] = [9,12,15]; as Linear: W = B^T is [out=3, in=2]
+    c = cases["matmulOfVectorAndMatrix"]
+    x = np.array(c["tensors"][0]["values"])
+    b = np.array(c["tensors"][1]["values"]).reshape(c["tensors"][1]["shape"])
+    raw, kp = _q8_exact(b.T)
+    w = QuantizedTensor.from_bytes(hip, synth.Q8_0, 3, kp, raw)
+    xp = np.zeros(kp, dtype=np.float32)
+    xp[: x.size] = x
+    y = DeviceTensor.from_numpy(hip, xp).matmul(w.t())
+    assert y.shape == Shape(3) and y.numpy().tolist() == c["expected"]
+    # TensorTest.kt:56-62: the rank-2 case through the GEMM path (k padded to the GEMM's 64-element granule)
+    c = cases["matmulOfMatrixAndMatrix"]
+    a = np.array(c["tensors"][0]["values"]).reshape(2, 3)
+    b = np.array(c["tensors"][1]["values"]).reshape(3, 2)
+    bt = np.zeros((2, 64))
+    bt[:, :3] = b.T
+    raw, kp = _q8_exact(bt)
+    w = QuantizedTensor.from_bytes(hip, synth.Q8_0, 2, kp, raw)
+    ap = np.zeros((2, kp), dtype=np.float32)
+    ap[:, :3] = a
+    got = DeviceTensor.from_numpy(hip, ap).matmul(w.t())
+    assert got.shape == Shape(2, 2) and got.numpy().reshape(-1).tolist() == c["expected"]
+
+
+def test_shape_errors_follow_the_reference(hip):
+    w = QuantizedTensor.from_bytes(hip, synth.Q4_K, 4, 256, synth.weight(synth.Q4_K, 4, 256, seed=1))
+    x = DeviceTensor.from_numpy(hip, np.zeros(512, dtype=np.float32))
+    with pytest.raises(ValueError, match="Shapes do not align."):  # TensorTest.kt:65-70
+        x.matmul(w.t())
+    with pytest.raises(ValueError, match="Unsupported tensor shapes for multiplication"):
+        x.matmul(w)  # not transposed: [512] x [4, 256] is no Linear
+    with pytest.raises(ValueError, match="Unsupported tensor shapes for multiplication"):
+        w.matmul(x)
+    assert w.t().shape == Shape(256, 4) and w.t().t().shape == Shape(4, 256) and w.t().buf is w.buf
+    with pytest.raises(Exception, match="not a multiple of block size"):
+        QuantizedTensor(hip, synth.Q4_K, Shape(4, 200), w.buf)
+
+
+def test_quantized_linear_with_bias_and_dequantize(hip):
+    n, k = 48, 1024
+    raw = synth.weight(synth.Q6_K, n, k, seed=4)
+    w = QuantizedTensor.from_bytes(hip, synth.Q6_K, n, k, raw)
+    bias = np.random.default_rng(1).standard_normal(n).astype(np.float32)
+    lin = QuantizedLinear(w, DeviceTensor.from_numpy(hip, bias))
+    x = synth.activation_f32(k, seed=2)
+    y = lin(DeviceTensor.from_numpy(hip, x)).numpy()
+    want = oracle_c.matvec_q(synth.Q6_K, raw, n, k, x).astype(np.float64) + bias
+    assert oracle_np.rel_err(y, want) <= 1e-3
+    xs = np.random.default_rng(3).standard_normal((5, k)).astype(np.float32)
+    ys = lin(DeviceTensor.from_numpy(hip, xs)).numpy()
+    want = oracle_c.gemm_q(synth.Q6_K, raw, n, k, synth.f32_to_bf16_bits(xs), 5).astype(np.float64) + bias
+    assert oracle_np.rel_err(ys, want) <= 1e-3
+    deq = w.dequantize().numpy()
+    assert np.array_equal(deq.view(np.uint32), oracle_c.dequant(synth.Q6_K, raw).reshape(n, k).view(np.uint32))
+
+
+def test_gguf_file_to_device(hip, tmp_path):
+    path = str(tmp_path / "m.gguf")
+    n, k = 32, 512
+    raw = synth.weight(synth.Q4_K, n, k, seed=9)
+    gguf.write_gguf(path, {"general.architecture": "llama"}, [("blk.0.ffn_up.weight", 12, (n, k), raw)])
+    r = gguf.GGUFReader(path)
+    t = r.tensor("blk.0.ffn_up.weight")
+    w = QuantizedTensor.from_bytes(hip, t.tensor_type, t.shape[0], t.shape[1], t.data)
+    x = synth.activation_f32(k, seed=10)
+    y = DeviceTensor.from_numpy(hip, x).matmul(w.t()).numpy()
+    assert oracle_np.rel_err(y, oracle_c.matvec_q(12, raw, n, k, x)) <= 1e-3
+    del t
+    r.close()
