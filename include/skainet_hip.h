@@ -86,7 +86,8 @@ int skn_sync(skn_ctx* ctx);
 int skn_set_stream(skn_ctx* ctx, void* hip_stream);
 /* Launch-shape tuning knobs, 0 = library default: "q4k.waves" (wavefronts per workgroup of the Q4_K matvec),
  * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention),
- * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel). */
+ * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel),
+ * "llama.fused" (1 = fused per-layer kernels in the decode step when every layer matrix is Q4_K, the default). */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
 int skn_timer_start(skn_ctx* ctx);

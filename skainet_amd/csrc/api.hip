@@ -230,6 +230,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     else if (!strcmp(key, "q4k.rows")) ctx->opt_q4k_rows = value;
     else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
     else if (!strcmp(key, "llama.graph")) ctx->opt_llama_graph = value;
+    else if (!strcmp(key, "llama.fused")) ctx->opt_llama_fused = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
     return SKN_OK;
 }

@@ -28,7 +28,7 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1;
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
@@ -39,6 +39,16 @@ struct skn_ctx {
 
 // One-time kernel attribute setup (large dynamic LDS), called by skn_init.
 int skn_matvec_init(skn_ctx* ctx);
+
+// Fused Q4_K matvec used by the decoder: up to three [rows_i, k] matrices stacked along the output axis,
+// optional RMSNorm of x (norm_w != nullptr) and a store / add-into / SwiGLU epilogue.
+struct skn_q4k_segments {
+    const uint8_t* w[3];
+    int rows[3];
+};
+enum { SKN_EPI_STORE = 0, SKN_EPI_ADD = 1, SKN_EPI_SWIGLU = 2 };
+int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
+                         float eps, float* y, int epi);
 
 // Records a failure on the context (or on the context-less slot) and returns `code`.
 int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);

@@ -19,6 +19,7 @@ struct skn_llama {
     int32_t* tokens_out = nullptr;  // device array of produced tokens
     int tokens_cap = 0;
     int pos = 0;                    // host mirror of the position
+    bool fused = false;             // every layer matrix is Q4_K with k <= 16384: the fused decode path applies
     // prompt buffers (grown to the longest prompt seen)
     int prompt_cap = 0;
     float *px = nullptr, *pxn = nullptr, *pq = nullptr, *pk = nullptr, *pv = nullptr, *patt = nullptr, *pproj = nullptr;
@@ -239,6 +240,24 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
+        if (m->fused && ctx->opt_llama_fused) {
+            // seven launches per layer: [norm + q,k,v], rope + cache store, attention (2), [Wo + residual],
+            // [norm + gate,up + SwiGLU], [Wdown + residual]
+            skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, H, H}};
+            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, 3 * H, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_STORE));
+            skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
+                       kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                       kv->page_tokens, log2f(c.rope_base));
+            SKN_LAUNCH_CHECK(ctx);
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, scale, m->att));
+            skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));
+            skn_q4k_segments gu = {{(const uint8_t*)L.w_gate, (const uint8_t*)L.w_up, nullptr}, {F, F, 0}};
+            SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU));
+            skn_q4k_segments wd = {{(const uint8_t*)L.w_down, nullptr, nullptr}, {H, 0, 0}};
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD));
+            continue;
+        }
         skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
         SKN_LAUNCH_CHECK(ctx);
         SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wq, H, H, m->xn, m->q));
@@ -356,7 +375,14 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
     auto A = [&](auto** p, size_t n) {
         if (rc == SKN_OK) rc = dev_alloc(ctx, m, p, n);
     };
-    A(&m->x, H); A(&m->xn, H); A(&m->q, H); A(&m->k, H); A(&m->v, H); A(&m->att, H); A(&m->proj, H);
+    A(&m->x, H); A(&m->xn, H); A(&m->q, 3 * H); A(&m->att, H); A(&m->proj, H);
+    if (rc == SKN_OK) {  // q, k, v are one buffer so that the three projections can be one launch
+        m->k = m->q + H;
+        m->v = m->q + 2 * H;
+    }
+    m->fused = cfg->hidden <= 16384 && cfg->ffn <= 16384;
+    for (int l = 0; l < cfg->n_layer; l++)
+        if (m->layers[l].type_attn != SKN_TYPE_Q4_K || m->layers[l].type_ffn != SKN_TYPE_Q4_K) m->fused = false;
     A(&m->gate, F); A(&m->up, F); A(&m->mid, F); A(&m->logits, (size_t)cfg->vocab);
     A(&m->attn_partial, (size_t)cfg->n_head * max_splits * (cfg->head_dim + 2));
     A(&m->state, (size_t)4);

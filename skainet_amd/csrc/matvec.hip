@@ -30,6 +30,10 @@ namespace {
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
+// LDS pitch (in float4) of one row of 64 lane slots: 65 puts the sixteen float4 of one column, which the staging
+// stores write from sixteen consecutive lanes, into different banks; the per-lane reads stay contiguous.
+constexpr int kXPitch = 65;
+
 // 6-bit scales / mins of sub-blocks 2p and 2p+1 out of the header chunk h = (d|dmin, scales[0..3], [4..7], [8..11]).
 // Branch-free and two values at a time: both packings are formed as byte pairs and the lane's pair index
 // selects one, so the header registers are only ever read by straight-line code.
@@ -65,30 +69,46 @@ __device__ __forceinline__ void q4k_dot_dword(uint32_t q, const float4& xl, cons
     ahi = fmaf((float)h13.y, xh.w, ahi);
 }
 
-// Staging of x, split in two so that the weight loads can be issued in between: the global loads of one
-// half column (32 activations of one (superblock, pair) column) into registers, and later their LDS stores.
+// Staging of x, split in two so that the weight loads can be issued in between: coalesced global loads
+// (thread t takes float4 t, t + blockDim, ...: a wavefront reads 1 KiB contiguous per instruction) into
+// registers, and later the LDS stores, which do the transposition into lane order.  float4 f of x belongs to
+// column f / 16 (64 activations of one (superblock, pair)), position f % 16 in it; the eight threads that
+// hold one half column are eight consecutive lanes, so its sum is a DPP reduction.
+template <int J>
 struct Q4kStage {
-    float4 v[8];
+    float4 v[J];
 };
 
-__device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int hc, Q4kStage& st) {
-    const float4* src = reinterpret_cast<const float4*>(x + 32 * hc);
+template <int J>
+__device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int n4, int tid, int nthreads,
+                                               Q4kStage<J>& st) {
+    const float4* x4 = reinterpret_cast<const float4*>(x);
 #pragma unroll
-    for (int i = 0; i < 8; i++) st.v[i] = src[i];
+    for (int j = 0; j < J; j++) st.v[j] = x4[min(tid + j * nthreads, n4 - 1)];
 }
 
-__device__ __forceinline__ void q4k_stage_store(const Q4kStage& st, int hc, float4* xs, float* ss) {
-    const int cc = hc >> 1, half = hc & 1;
-    const int step = cc >> 6, lane = cc & 63;
-    const float mul = half ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
-    float sum = 0.f;
+__device__ __forceinline__ void q4k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
+    const int cc = f >> 4, i16 = f & 15;
+    const int step = cc >> 6, ln = cc & 63;
+    const float mul = (i16 & 8) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
+    xs[(step * 16 + i16) * kXPitch + ln] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
+    float sum = (v.x + v.y) + (v.z + v.w);
+    sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));   // lane ^ 1
+    sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x4E, 0xF, 0xF, true));   // lane ^ 2
+    sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x141, 0xF, 0xF, true));  // 7 - lane
+    if ((f & 7) == 0) ss[f >> 3] = sum * 5.9604644775390625e-08f;  // 2^-24, see the scaling note above
+}
+
+template <int J>
+__device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, int tid, int nthreads, float4* xs,
+                                                float* ss) {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const float4 v = st.v[i];
-        sum += (v.x + v.y) + (v.z + v.w);
-        xs[(step * 16 + 8 * half + i) * 64 + lane] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
+    for (int j = 0; j < J; j++) {
+        // a float4 index past the end repeats the last one: same data to the same slot (no branch; whole
+        // groups of eight lanes are clamped together because n4 is a multiple of 64)
+        const int f = min(tid + j * nthreads, n4 - 1);
+        q4k_stage_store_one(st.v[j], f, xs, ss);
     }
-    ss[2 * cc + half] = sum * 5.9604644775390625e-08f;  // 2^-24, see the scaling note above
 }
 
 struct Q4kLoads {
@@ -109,8 +129,8 @@ __device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* _
         float4 xl[4], xh[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            xl[j] = xs[(s * 16 + 4 * half + j) * 64 + lane];
-            xh[j] = xs[(s * 16 + 8 + 4 * half + j) * 64 + lane];
+            xl[j] = xs[(s * 16 + 4 * half + j) * kXPitch + lane];
+            xh[j] = xs[(s * 16 + 8 + 4 * half + j) * kXPitch + lane];
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -148,7 +168,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
-    float* ss = reinterpret_cast<float*>(lds4 + steps * 16 * 64);
+    float* ss = reinterpret_cast<float*>(lds4 + steps * 16 * kXPitch);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -158,13 +178,13 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     const int sub = lane >> 2;  // superblock within the step
     const int p = lane & 3;     // sub-block pair within the superblock
     const size_t row_chunks = (size_t)nb * 9;
-    const int n_half_cols = nb * 8;
+    const int n4 = nb * 64;  // float4 count of x
 
-    // this thread's first half column of x goes into registers (threads past the last half column repeat the
-    // last one: same data to the same slot, no branch)
-    Q4kStage st;
-    const int hc0 = min(tid, n_half_cols - 1);
-    q4k_stage_load(x, hc0, st);
+    // the first J float4 per thread go into registers now; J covers all of x in the unrolled kernels
+    // (the launcher runs them with 512 threads: 2 * STEPS * 512 float4 >= k / 4)
+    constexpr int J = STEPS > 0 ? 2 * STEPS : 2;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, blockDim.x, st);
 
     float acc[R];
     const uint4* rp[R];
@@ -192,8 +212,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     if constexpr (STEPS > 0) {
         Q4kLoads L[STEPS][R];
         issue(0, 0, L[0]);
-        // the launcher guarantees blockDim.x >= nb * 8 here: one half column per thread covers x, no loop
-        q4k_stage_store(st, hc0, xs, ss);
+        q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
         __syncthreads();
         // `tie` is always 0; an empty asm after each step makes it look rewritten from the finished accumulator,
         // which pins the loads of step s+1 between the arithmetic of steps s-1 and s (one step of lookahead) and
@@ -210,11 +229,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     } else {
         Q4kLoads bufa[R], bufb[R];
         issue(0, 0, bufa);
-        q4k_stage_store(st, hc0, xs, ss);
-        for (int hc = tid + blockDim.x; hc < n_half_cols; hc += blockDim.x) {
-            q4k_stage_load(x, hc, st);
-            q4k_stage_store(st, hc, xs, ss);
-        }
+        q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
+        for (int f = tid + J * blockDim.x; f < n4; f += blockDim.x)
+            q4k_stage_store_one(reinterpret_cast<const float4*>(x)[f], f, xs, ss);
         __syncthreads();
         for (int s = 0; s < steps; s += 2) {
             if (s + 1 < steps) issue(s + 1, 0, bufb);
@@ -297,11 +314,169 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
     if (lane == 0) y[row] = acc;
 }
 
+// ---- fused forms used by the decoder ---------------------------------------------------------------------
+// Up to three weight matrices with the same k stacked along the output axis (q, k, v projections in one launch;
+// gate and up paired row by row), optional RMSNorm of x folded into the staging (every workgroup needs all of
+// x anyway, so it also forms sum(x^2) and stores x * r * norm_w), and an epilogue that stores, adds into the
+// residual stream, or applies SwiGLU to a (gate, up) row pair.  Two rows per wavefront.
+template <int STEPS, int EPI, bool NORM>
+__global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments seg, const float* __restrict__ x,
+                                                               const float* __restrict__ norm_w, float eps,
+                                                               float* __restrict__ y, int n_out, int nb) {
+    constexpr int R = 2;
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
+    float* red = ss + STEPS * 128;  // eight partial sums of x^2 (all LDS here is dynamic)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 2, p = lane & 3;
+    const int n4 = nb * 64;
+    constexpr int J = 2 * STEPS;  // 512 threads x J float4 cover k <= STEPS * 4096
+
+    Q4kStage<J> st, nw;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+    if (NORM) q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
+
+    // the two rows of this wavefront: consecutive rows of the stacked matrices, or row i of gate and of up
+    const int unit = blockIdx.x * 8 + wave;
+    const uint8_t* rowp[R];
+    bool row_ok[R];
+    const size_t row_bytes = (size_t)nb * 144;
+    if (EPI == SKN_EPI_SWIGLU) {
+        const int i = min(unit, n_out - 1);
+        row_ok[0] = row_ok[1] = unit < n_out;
+        rowp[0] = seg.w[0] + (size_t)i * row_bytes;
+        rowp[1] = seg.w[1] + (size_t)i * row_bytes;
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = unit * R + r;
+            row_ok[r] = row < n_out;
+            row = min(row, n_out - 1);
+            const uint8_t* base = seg.w[0];
+            if (row >= seg.rows[0]) {
+                row -= seg.rows[0];
+                base = seg.w[1];
+                if (row >= seg.rows[1]) {
+                    row -= seg.rows[1];
+                    base = seg.w[2];
+                }
+            }
+            rowp[r] = base + (size_t)row * row_bytes;
+        }
+    }
+    Q4kLoads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int blk = s * 16 + sub;
+        const int off = min(blk, nb - 1) * 9 + 1 + 2 * p + tie;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint4* bp = reinterpret_cast<const uint4*>(rowp[r]) + off;
+            L[s][r].qa = bp[0];
+            L[s][r].qb = bp[1];
+            L[s][r].h = bp[-1 - 2 * p];
+            L[s][r].ok = row_ok[r] && blk < nb;
+        }
+    };
+    issue(0, 0);
+
+    if (NORM) {
+        float sq = 0.f;
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            if (tid + j * 512 < n4) {
+                const float4 v = st.v[j];
+                sq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+            }
+        }
+        sq = wave_sum(sq);
+        if (lane == 0) red[wave] = sq;
+        __syncthreads();
+        const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
+        const float rinv = 1.0f / sqrtf(total / (float)(nb * 256) + eps);
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            st.v[j].x *= rinv * nw.v[j].x;
+            st.v[j].y *= rinv * nw.v[j].y;
+            st.v[j].z *= rinv * nw.v[j].z;
+            st.v[j].w *= rinv * nw.v[j].w;
+        }
+    }
+    q4k_stage_store<J>(st, n4, tid, 512, xs, ss);
+    __syncthreads();
+
+    float acc[R] = {0.f, 0.f};
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+    const float t0 = wave_sum(acc[0]) * 16777216.0f;
+    const float t1 = wave_sum(acc[1]) * 16777216.0f;
+    if (lane == 0) {
+        if (EPI == SKN_EPI_SWIGLU) {
+            if (row_ok[0]) y[unit] = t0 / (1.0f + expf(-t0)) * t1;
+        } else if (EPI == SKN_EPI_ADD) {
+            if (row_ok[0]) y[unit * R] += t0;
+            if (row_ok[1]) y[unit * R + 1] += t1;
+        } else {
+            if (row_ok[0]) y[unit * R] = t0;
+            if (row_ok[1]) y[unit * R + 1] = t1;
+        }
+    }
+}
+
+template <int STEPS, int EPI, bool NORM>
+int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
+                     float eps, float* y) {
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2)) + 8 * sizeof(float);
+    const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
+    dim3 grid((unsigned)((units + 7) / 8)), block(512);
+    skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int STEPS>
+int dispatch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
+                       float eps, float* y, int epi) {
+    const bool norm = norm_w != nullptr;
+    if (epi == SKN_EPI_SWIGLU)
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
+                    : launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
+    if (epi == SKN_EPI_ADD)
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ADD, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
+                    : launch_q4k_fused<STEPS, SKN_EPI_ADD, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
+    return norm ? launch_q4k_fused<STEPS, SKN_EPI_STORE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
+                : launch_q4k_fused<STEPS, SKN_EPI_STORE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
+}
+
+template <int STEPS, int EPI, bool NORM>
+hipError_t allow_big_lds_fused() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_fused_kernel<STEPS, EPI, NORM>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
+template <int STEPS>
+hipError_t allow_big_lds_fused_all() {
+    hipError_t e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, false>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, true>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, false>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, true>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, false>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, true>();
+    return e;
+}
+
 template <int STEPS, int R>
 int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
-    if (STEPS > 0 && waves * 64 < nb * 8) return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
+    if (STEPS > 0 && waves != 8) return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
     const int steps = (nb + 15) / 16;
-    const size_t lds = (size_t)steps * 64 * (16 * sizeof(float4) + sizeof(float2));
+    const size_t lds = (size_t)steps * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
     SKN_REQUIRE(ctx, lds <= 160 * 1024, SKN_ERR_SHAPE, "skn_matvec_q: k = %d needs %zu bytes of LDS (limit 163840)",
                 nb * 256, lds);
     auto kern = matvec_q4k_kernel<STEPS, R>;
@@ -339,7 +514,24 @@ int skn_matvec_init(skn_ctx* ctx) {
                              allow_big_lds<3, 2>, allow_big_lds<4, 2>, allow_big_lds<0, 4>, allow_big_lds<1, 4>,
                              allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>};
     for (auto f : fns) SKN_HIP(ctx, f());
+    SKN_HIP(ctx, allow_big_lds_fused_all<1>());
+    SKN_HIP(ctx, allow_big_lds_fused_all<2>());
+    SKN_HIP(ctx, allow_big_lds_fused_all<3>());
+    SKN_HIP(ctx, allow_big_lds_fused_all<4>());
     return SKN_OK;
+}
+
+// Fused Q4_K matvec for the decoder; k <= 16384 (four unrolled steps).  Returns SKN_ERR_SHAPE otherwise.
+int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
+                         float eps, float* y, int epi) {
+    SKN_REQUIRE(ctx, k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_SHAPE, "fused Q4_K matvec: unsupported k %d", k);
+    const int nb = k / 256;
+    switch ((nb + 15) / 16) {
+        case 1: return dispatch_q4k_fused<1>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
+        case 2: return dispatch_q4k_fused<2>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
+        case 3: return dispatch_q4k_fused<3>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
+        default: return dispatch_q4k_fused<4>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
+    }
 }
 
 extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev,
@@ -365,6 +557,7 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         if (waves <= 0) waves = 8;
         if (rows <= 0) rows = 2;
         if (waves > 8) waves = 8;
+        if (rows >= 4 && nb > 32) rows = 2;  // four rows of three or more unrolled steps do not fit the registers
         return rows >= 4   ? dispatch_q4k<4>(ctx, w, n, nb, x_dev, y_dev, waves)
                : rows >= 2 ? dispatch_q4k<2>(ctx, w, n, nb, x_dev, y_dev, waves)
                            : dispatch_q4k<1>(ctx, w, n, nb, x_dev, y_dev, waves);

@@ -84,6 +84,30 @@ def test_graph_replay_equals_eager(hip):
     model.free()
 
 
+def test_fused_and_unfused_decode_agree(hip):
+    w = llama.random_weights(SMALL, seed=13)
+    outs = {}
+    for fused in (0, 1):
+        hip.set_option("llama.fused", fused)
+        model = llama.LlamaModel(hip, SMALL, weights=w)
+        first = model.prefill([3, 1, 4, 1, 5, 9, 2, 6])
+        toks = model.decode(first, 12)
+        outs[fused] = (first, toks, model.logits())
+        model.free()
+    hip.set_option("llama.fused", 1)
+    assert outs[0][0] == outs[1][0]
+    assert oracle_np.rel_err(outs[1][2], outs[0][2]) <= TOL
+    ora = OracleLlama(SMALL, w)
+    ora.prefill([3, 1, 4, 1, 5, 9, 2, 6], bf16_gemm=True)
+    tok = outs[0][0]
+    for i in range(12):
+        want = ora.step(tok)
+        if not _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+            break
+        assert outs[0][1][i] == want and outs[1][1][i] == want, i
+        tok = want
+
+
 def test_llama_argument_errors(hip):
     w = llama.random_weights(SMALL, seed=1)
     model = llama.LlamaModel(hip, SMALL, weights=w)
