@@ -29,6 +29,10 @@ namespace {
 //   y = 2^24 * sum_blocks [ d * (sc_lo * A_lo + sc_hi * A_hi) - dmin * (m_lo * S_lo + m_hi * S_hi) ]
 
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+// 16 loaded bytes as a native vector: the value stays one four-register tuple from the load to its use.  With
+// HIP's uint4 (a struct) the four words are split at the load and the register allocator parks and re-copies
+// them, which puts a wait for the load in front of each copy.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // LDS pitch (in float4) of one row of 64 lane slots: 65 puts the sixteen float4 of one column, which the staging
 // stores write from sixteen consecutive lanes, into different banks; the per-lane reads stay contiguous.
@@ -37,7 +41,7 @@ constexpr int kXPitch = 65;
 // 6-bit scales / mins of sub-blocks 2p and 2p+1 out of the header chunk h = (d|dmin, scales[0..3], [4..7], [8..11]).
 // Branch-free and two values at a time: both packings are formed as byte pairs and the lane's pair index
 // selects one, so the header registers are only ever read by straight-line code.
-__device__ __forceinline__ void q4k_pair_scales(const uint4& h, int pair, float& sc0, float& sc1, float& m0,
+__device__ __forceinline__ void q4k_pair_scales(const u32x4& h, int pair, float& sc0, float& sc1, float& m0,
                                                 float& m1) {
     const int sh = 16 * (pair & 1);
     const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
@@ -112,7 +116,7 @@ __device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, i
 }
 
 struct Q4kLoads {
-    uint4 h, qa, qb;
+    u32x4 h, qa, qb;
     bool ok;  // false: the slot lies past the row end / past the last row and must contribute nothing
 };
 
@@ -134,7 +138,7 @@ __device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* _
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const uint4 qq = half == 0 ? L[r].qa : L[r].qb;
+            const u32x4 qq = half == 0 ? L[r].qa : L[r].qb;
             q4k_dot_dword(qq.x, xl[0], xh[0], alo[r], ahi[r]);
             q4k_dot_dword(qq.y, xl[1], xh[1], alo[r], ahi[r]);
             q4k_dot_dword(qq.z, xl[2], xh[2], alo[r], ahi[r]);
@@ -187,21 +191,21 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     q4k_stage_load<J>(x, n4, tid, blockDim.x, st);
 
     float acc[R];
-    const uint4* rp[R];
+    const u32x4* rp[R];
     bool row_ok[R];
 #pragma unroll
     for (int r = 0; r < R; r++) {
         acc[r] = 0.f;
         row_ok[r] = row0 + r < n_rows;
         // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
-        rp[r] = reinterpret_cast<const uint4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + 1 + 2 * p;
+        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + 1 + 2 * p;
     }
     auto issue = [&](int s, int tie, Q4kLoads (&L)[R]) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
         const int off = min(blk, nb - 1) * 9 + tie;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const uint4* bp = rp[r] + off;
+            const u32x4* bp = rp[r] + off;
             L[r].qa = bp[0];
             L[r].qb = bp[1];
             L[r].h = bp[-1 - 2 * p];
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         const int off = min(blk, nb - 1) * 9 + 1 + 2 * p + tie;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const uint4* bp = reinterpret_cast<const uint4*>(rowp[r]) + off;
+            const u32x4* bp = reinterpret_cast<const u32x4*>(rowp[r]) + off;
             L[s][r].qa = bp[0];
             L[s][r].qb = bp[1];
             L[s][r].h = bp[-1 - 2 * p];
