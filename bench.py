@@ -174,9 +174,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy"], default="bench",
-                    help="copy: run --steps plain device copies of the headline weight size instead (the known-size "
+    ap.add_argument("--mode", choices=["bench", "copy", "decode"], default="bench",
+                    help="decode: only the 7B-shape decode leg (for kernel traces of one token step).  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="decode without the captured step graph (kernel tracers that cannot follow graph launches)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -184,6 +186,8 @@ def main():
 
     ctx = runtime.Context(0)
     info = ctx.device_info()
+    if args.no_graph:
+        ctx.set_option("llama.graph", 0)
     n, k = 4096, 11008
     if args.mode == "copy":
         nbytes = n * (k // 256) * 144
@@ -196,6 +200,11 @@ def main():
         print(json.dumps({"mode": "copy", "bytes_read": nbytes, "bytes_written": nbytes, "launches": launches,
                           "kernel": "copy16_kernel", "kernel_us": round(ms / launches * 1e3, 3),
                           "read_plus_write_gbs": round(2 * nbytes / (ms / launches * 1e-3) / 1e9, 1)}))
+        ctx.close()
+        return
+    if args.mode == "decode":
+        from skainet_amd import llama_bench
+        print(json.dumps({"mode": "decode", **llama_bench.run(ctx, steps=min(args.steps, 128))}))
         ctx.close()
         return
     head = bench_matvec(ctx, Q4_K, n, k, args.steps, args.warmup)

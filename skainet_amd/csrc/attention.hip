@@ -2,184 +2,284 @@
 //
 // One query row per (sequence, head), so every K and V byte is used exactly once: the kernel is an HBM
 // stream of 2 * n_ctx * head_dim * 2 bytes per (sequence, head) at 1 flop per byte.  The context is split
-// across workgroups (flash-decoding): grid = (splits, heads, sequences); each workgroup walks its token
-// range in 64-token tiles, stages the K and V tiles through LDS with 128-bit loads, keeps a running
-// (max, sum, output) triple, and writes one partial; a small second kernel merges the partials.
+// across workgroups (flash-decoding): grid = (splits, heads, sequences).
+//
+// Inside a workgroup there is no staging and no barrier while tokens stream: a token row (head_dim halves)
+// is spread over head_dim / 8 consecutive lanes, 16 bytes each, so one wavefront load instruction covers
+// 64 * 8 / head_dim consecutive tokens (1 KiB contiguous in a page).  The lanes of a token form a group that
+// owns a private softmax stream: the score is the group's DPP all-reduce of eight products per lane, every
+// lane of the group then holds the same (running max, running sum) and its own eight output dimensions, and
+// the V row is loaded with the same lane mapping as the K row.  The streams of a workgroup are merged once at
+// the end through LDS; the partials of the splits are merged by whichever workgroup of a (sequence, head)
+// finishes last (a counter in device memory, reset by that workgroup), so the whole step is one launch.
 #include "kv.h"
 
 namespace {
 
-constexpr int kTile = 64;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-template <int D>
-__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+constexpr int kAttnThreads = 256;
+constexpr int kMaxSplits = 512;
+constexpr int kUnroll = 4;  // tokens per stream in flight per iteration (K and V: 8 x 16 bytes per lane)
+
+template <int LPT>
+__device__ __forceinline__ float group_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));   // lane ^ 1
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));   // lane ^ 2
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));  // 7 - lane
+    if constexpr (LPT >= 16) v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x140, 0xF, 0xF, true));
+    if constexpr (LPT >= 32) v += __shfl_xor(v, 16, 64);
+    return v;
+}
+
+__device__ __forceinline__ float dot8(const u32x4& k, const float (&qf)[8]) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t w = k[j];  // (a bit cast applied directly to a vector element reads element 0)
+        const half2_t h = __builtin_bit_cast(half2_t, w);
+        s = fmaf((float)h.x, qf[2 * j], s);
+        s = fmaf((float)h.y, qf[2 * j + 1], s);
+    }
+    return s;
+}
+
+template <int D, bool POW2>
+__global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const uint16_t* __restrict__ k_pool, const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ table,
-    const int32_t* __restrict__ nctx, const float* __restrict__ q, float* __restrict__ partial, int n_head,
-    int page_tokens, int pages_per_seq, int n_splits, float scale, int seq_fixed) {
-    constexpr int KROW = D + 8;   // halves per K row in LDS: 16 bytes of padding spread the rows over the banks
-    constexpr int CH = D / 8;     // 16-byte chunks per row
-    constexpr int QS = D / 4;     // dims per score thread
-    constexpr int VEC = D / 64;   // dims per output lane
-    __shared__ __align__(16) uint16_t ks[kTile * KROW];
-    __shared__ __align__(16) uint16_t vs[kTile * D];
-    __shared__ float ps[kTile];
-    __shared__ float red_max[4], red_sum[4];
-    __shared__ float obuf[4][D];
+    const int32_t* __restrict__ nctx, const float* __restrict__ q, float* partial, int* counters, float* __restrict__ out,
+    int n_head, int page_tokens, int page_shift, int pages_per_seq, int n_splits, float scale, int seq_fixed) {
+    constexpr int LPT = D / 8;                        // lanes per token
+    constexpr int G = 64 / LPT;                       // token groups (streams) per wavefront
+    constexpr int NS = (kAttnThreads / 64) * G;       // streams per workgroup
+    constexpr int U = kUnroll;
+    __shared__ float so[NS][D];
+    __shared__ float sm[NS], sl[NS];
+    __shared__ float pm[kMaxSplits], pl[kMaxSplits];
+    __shared__ int last_flag;
+    static_assert(kAttnThreads / (D / 4) <= NS, "the split merge reuses the stream rows");
 
     // blockIdx.z is the query row: its own sequence by default, or one shared sequence (seq_fixed >= 0) when
     // several query rows attend to prefixes of the same cache (prompt processing)
     const int split = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
     const int kv_seq = seq_fixed >= 0 ? seq_fixed : s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane % LPT, g = lane / LPT;
+    const int stream = wave * G + g;
     const int n = nctx[s];
-    const int tiles_total = (n + kTile - 1) / kTile;
-    const int tiles_per_split = (tiles_total + n_splits - 1) / n_splits;
-    const int t_begin = split * tiles_per_split * kTile;
-    const int t_end = min(n, t_begin + tiles_per_split * kTile);
+    const int per = ((n + n_splits - 1) / n_splits + NS - 1) / NS * NS;  // whole wavefront loads per split
+    const int t_begin = split * per;
+    const int t_end = min(n, t_begin + per);
 
-    const int tt = tid >> 2, sl = tid & 3;  // score phase: token of the tile, quarter of the head dimension
-    float qr[QS];
+    float qf[8];
     {
-        const float* qp = q + ((size_t)s * n_head + h) * D + sl * QS;
-#pragma unroll
-        for (int i = 0; i < QS; i++) qr[i] = qp[i] * scale;
+        const float4* qp = reinterpret_cast<const float4*>(q + ((size_t)s * n_head + h) * D + c * 8);
+        const float4 a = qp[0], b = qp[1];
+        qf[0] = a.x * scale, qf[1] = a.y * scale, qf[2] = a.z * scale, qf[3] = a.w * scale;
+        qf[4] = b.x * scale, qf[5] = b.y * scale, qf[6] = b.z * scale, qf[7] = b.w * scale;
     }
-    float o[VEC];
+    float o[8];
 #pragma unroll
-    for (int v = 0; v < VEC; v++) o[v] = 0.f;
+    for (int j = 0; j < 8; j++) o[j] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* trow = table + (size_t)kv_seq * pages_per_seq;
 
-    for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
-        const int nt = min(kTile, t_end - t0);
-        for (int idx = tid; idx < kTile * CH; idx += 256) {
-            const int r = idx / CH, c = idx % CH;
-            uint4 kk = make_uint4(0, 0, 0, 0), vv = kk;
-            if (r < nt) {
-                const int t = t0 + r;
-                const int page = trow[t / page_tokens];
-                const size_t off = (((size_t)page * n_head + h) * page_tokens + (t % page_tokens)) * D + c * 8;
-                kk = *reinterpret_cast<const uint4*>(k_pool + off);
-                vv = *reinterpret_cast<const uint4*>(v_pool + off);
-            }
-            *reinterpret_cast<uint4*>(ks + r * KROW + c * 8) = kk;
-            *reinterpret_cast<uint4*>(vs + r * D + c * 8) = vv;
-        }
-        __syncthreads();
-
-        // scores: four lanes per token, each over a quarter of the head dimension
-        float sc = 0.f;
-        {
-            const uint16_t* kr = ks + tt * KROW + sl * QS;
+    for (int base = t_begin; base < t_end; base += NS * U) {
+        u32x4 kk[U], vv[U];
+        bool ok[U];
+        int page[U], slot[U];
 #pragma unroll
-            for (int i = 0; i < QS; i += 8) {
-                const uint4 u = *reinterpret_cast<const uint4*>(kr + i);
-                const uint32_t wds[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    sc = fmaf(h2f_bits(wds[j] & 0xFFFF), qr[i + 2 * j], sc);
-                    sc = fmaf(h2f_bits(wds[j] >> 16), qr[i + 2 * j + 1], sc);
-                }
-            }
+        for (int u = 0; u < U; u++) {
+            const int t = base + u * NS + stream;
+            ok[u] = t < t_end;
+            const int tc = min(t, t_end - 1);  // past the end: a valid row, masked below
+            const int pi = POW2 ? tc >> page_shift : tc / page_tokens;
+            slot[u] = tc - pi * page_tokens;
+            page[u] = trow[pi];
         }
-        sc += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sc), 0xB1, 0xF, 0xF, true));
-        sc += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sc), 0x4E, 0xF, 0xF, true));
-        if (tt >= nt) sc = -INFINITY;
-        const float wmax = wave_max(sc);
-        if (lane == 0) red_max[wave] = wmax;
-        __syncthreads();
-        const float tile_max = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
-        const float m_new = fmaxf(m_run, tile_max);
-        const float p = (tt < nt) ? __expf(sc - m_new) : 0.f;
-        if (sl == 0) ps[tt] = p;
-        const float wsum = wave_sum(sl == 0 ? p : 0.f);
-        if (lane == 0) red_sum[wave] = wsum;
-        const float alpha = __expf(m_run - m_new);  // 0 on the first tile (m_run = -inf)
-        __syncthreads();
-        l_run = l_run * alpha + ((red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]));
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t off = (((size_t)page[u] * n_head + h) * page_tokens + slot[u]) * D + c * 8;
+            kk[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
+            vv[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
+        }
+        float sc[U];
+        float m_new = m_run;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float d = group_sum<LPT>(dot8(kk[u], qf));
+            sc[u] = ok[u] ? d : -INFINITY;
+            m_new = fmaxf(m_new, sc[u]);
+        }
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // keeps exp(-inf - -inf) out of the arithmetic
+        const float alpha = __expf(m_run - m_safe);
+        float p[U], psum = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            p[u] = __expf(sc[u] - m_safe);
+            psum += p[u];
+        }
+        l_run = fmaf(l_run, alpha, psum);
         m_run = m_new;
-
-        // output: wave w takes tokens 16w..16w+15 of the tile, lane l the dims VEC*l..
 #pragma unroll
-        for (int v = 0; v < VEC; v++) o[v] *= alpha;
-#pragma unroll 4
-        for (int j = 0; j < 16; j++) {
-            const int t = wave * 16 + j;
-            const float pj = ps[t];
-            const uint16_t* vr = vs + t * D + lane * VEC;
-            if constexpr (VEC == 1) {
-                o[0] = fmaf(pj, h2f_bits(vr[0]), o[0]);
-            } else if constexpr (VEC == 2) {
-                const uint32_t u = *reinterpret_cast<const uint32_t*>(vr);
-                o[0] = fmaf(pj, h2f_bits(u & 0xFFFF), o[0]);
-                o[1] = fmaf(pj, h2f_bits(u >> 16), o[1]);
-            } else {
-                const uint2 u = *reinterpret_cast<const uint2*>(vr);
-                o[0] = fmaf(pj, h2f_bits(u.x & 0xFFFF), o[0]);
-                o[1] = fmaf(pj, h2f_bits(u.x >> 16), o[1]);
-                o[2] = fmaf(pj, h2f_bits(u.y & 0xFFFF), o[2]);
-                o[3] = fmaf(pj, h2f_bits(u.y >> 16), o[3]);
+        for (int j = 0; j < 8; j++) o[j] *= alpha;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t w = vv[u][j];
+                const half2_t hv = __builtin_bit_cast(half2_t, w);
+                o[2 * j] = fmaf(p[u], (float)hv.x, o[2 * j]);
+                o[2 * j + 1] = fmaf(p[u], (float)hv.y, o[2 * j + 1]);
             }
         }
-        __syncthreads();  // the next tile overwrites ks / vs / ps
     }
 
+    // merge the streams of the workgroup
 #pragma unroll
-    for (int v = 0; v < VEC; v++) obuf[wave][lane * VEC + v] = o[v];
+    for (int j = 0; j < 8; j++) so[stream][c * 8 + j] = o[j];
+    if (c == 0) {
+        sm[stream] = m_run;
+        sl[stream] = l_run;
+    }
     __syncthreads();
-    float* dst = partial + (((size_t)s * n_head + h) * n_splits + split) * (D + 2);
-    if (tid < D) dst[tid] = (obuf[0][tid] + obuf[1][tid]) + (obuf[2][tid] + obuf[3][tid]);
+    const int pair = s * n_head + h;
+    float M = -INFINITY, acc = 0.f, L = 0.f;
+    if (tid < D) {
+#pragma unroll
+        for (int i = 0; i < NS; i++) M = fmaxf(M, sm[i]);
+        const float m_safe = M == -INFINITY ? 0.f : M;
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            const float wgt = __expf(sm[i] - m_safe);
+            acc = fmaf(wgt, so[i][tid], acc);
+            L = fmaf(wgt, sl[i], L);
+        }
+    }
+    if (n_splits == 1) {
+        if (tid < D) out[(size_t)pair * D + tid] = L > 0.f ? acc / L : 0.f;
+        return;
+    }
+    // partial: per (pair, split) D + 2 floats: unnormalised output, max, sum
+    float* mine = partial + ((size_t)pair * n_splits + split) * (D + 2);
+    // Partials and counters are written and read as device-scope atomics (relaxed): such stores go through to
+    // the level all compute dies share and such loads never hit a stale line, so no cache-wide write-back or
+    // invalidate is needed; order comes from waiting for the stores (vmcnt) before the barrier that precedes
+    // the counter increment.
+    if (tid < D) __hip_atomic_store(&mine[tid], acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) {
-        dst[D] = m_run;
-        dst[D + 1] = l_run;
+        __hip_atomic_store(&mine[D], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&mine[D + 1], L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-}
-
-// grid = sequences * heads, block = head_dim threads
-__global__ void attn_merge_kernel(const float* __restrict__ partial, float* __restrict__ out, int n_splits, int D) {
-    const float* base = partial + (size_t)blockIdx.x * n_splits * (D + 2);
-    const int d = threadIdx.x;
-    float M = -INFINITY;
-    for (int i = 0; i < n_splits; i++) M = fmaxf(M, base[i * (D + 2) + D]);
-    float acc = 0.f, L = 0.f;
-    for (int i = 0; i < n_splits; i++) {
-        const float mi = base[i * (D + 2) + D];
-        const float wgt = (mi == -INFINITY) ? 0.f : __expf(mi - M);
-        L = fmaf(wgt, base[i * (D + 2) + D + 1], L);
-        acc = fmaf(wgt, base[i * (D + 2) + d], acc);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    // the last workgroup of this (sequence, head) to get here merges the splits
+    if (tid == 0)
+        last_flag = __hip_atomic_fetch_add(&counters[pair], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_splits - 1;
+    __syncthreads();
+    if (!last_flag) return;
+    // split maxima and sums into LDS with one round of loads, then rows of partial outputs as float4:
+    // D / 4 threads per split row, P rows in flight
+    const float* base_p = partial + (size_t)pair * n_splits * (D + 2);
+    for (int i = tid; i < n_splits; i += kAttnThreads) {
+        pm[i] = __hip_atomic_load(&base_p[i * (D + 2) + D], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        pl[i] = __hip_atomic_load(&base_p[i * (D + 2) + D + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    out[(size_t)blockIdx.x * D + d] = L > 0.f ? acc / L : 0.f;
+    __syncthreads();  // also: every thread is past the stream merge, so / sl are free again
+    float M2 = -INFINITY;
+    for (int i = 0; i < n_splits; i++) M2 = fmaxf(M2, pm[i]);
+    const float m2_safe = M2 == -INFINITY ? 0.f : M2;
+    constexpr int DV = D / 4, P = kAttnThreads / DV;
+    const int dq = tid % DV, part = tid / DV;
+    float4 a4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    float L2 = 0.f;
+#pragma unroll 4
+    for (int i = part; i < n_splits; i += P) {
+        const float wgt = __expf(pm[i] - m2_safe);
+        // rows are 8-byte aligned: two 64-bit loads per thread
+        const unsigned long long* row = reinterpret_cast<const unsigned long long*>(base_p + (size_t)i * (D + 2)) + 2 * dq;
+        const unsigned long long u0 = __hip_atomic_load(row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long u1 = __hip_atomic_load(row + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float2 lo = make_float2(__uint_as_float((uint32_t)u0), __uint_as_float((uint32_t)(u0 >> 32)));
+        const float2 hi = make_float2(__uint_as_float((uint32_t)u1), __uint_as_float((uint32_t)(u1 >> 32)));
+        a4.x = fmaf(wgt, lo.x, a4.x);
+        a4.y = fmaf(wgt, lo.y, a4.y);
+        a4.z = fmaf(wgt, hi.x, a4.z);
+        a4.w = fmaf(wgt, hi.y, a4.w);
+        L2 = fmaf(wgt, pl[i], L2);
+    }
+    *reinterpret_cast<float4*>(&so[part][dq * 4]) = a4;
+    if (dq == 0) sl[part] = L2;
+    __syncthreads();
+    if (tid < D) {
+        float acc2 = 0.f;
+        L2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < P; i++) {
+            acc2 += so[i][tid];
+            L2 += sl[i];
+        }
+        out[(size_t)pair * D + tid] = L2 > 0.f ? acc2 / L2 : 0.f;
+    }
+    if (tid == 0) __hip_atomic_store(&counters[pair], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
 }
 
 }  // namespace
 
 // Shared with the decoder.  n_queries query rows; row z attends to nctx_dev[z] tokens of sequence z
-// (seq_fixed < 0) or of sequence seq_fixed.  `partial` must hold n_queries * n_head * n_splits * (D + 2) floats.
+// (seq_fixed < 0) or of sequence seq_fixed.  With more than one split, `partial` holds n_queries * n_head *
+// n_splits * (head_dim + 2) floats and `counters` n_queries * n_head ints that are zero between launches:
+// zeroed once by their owner, left zero by every launch.
 int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
-                       int seq_fixed, int n_splits, float* partial, float scale, float* out_dev) {
+                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev) {
     const int D = kv->head_dim;
     SKN_REQUIRE(ctx, D == 64 || D == 128 || D == 256, SKN_ERR_SHAPE,
                 "skn_attn_decode: head_dim %d is not supported (64, 128 or 256)", D);
-    dim3 grid(n_splits, kv->n_head, n_queries), block(256);
+    SKN_REQUIRE(ctx, n_splits <= kMaxSplits, SKN_ERR_ARG, "skn_attn_decode: %d splits (at most %d)", n_splits, kMaxSplits);
+    SKN_REQUIRE(ctx, n_splits >= 1 && (n_splits == 1 || (partial != nullptr && counters != nullptr)), SKN_ERR_ARG,
+                "skn_attn_decode: %d splits without scratch", n_splits);
+    int page_shift = -1;
+    if ((kv->page_tokens & (kv->page_tokens - 1)) == 0)
+        for (page_shift = 0; (1 << page_shift) < kv->page_tokens; page_shift++) {}
+    dim3 grid(n_splits, kv->n_head, n_queries), block(kAttnThreads);
 #define SKN_ATTN_LAUNCH(DD)                                                                                        \
-    skn_launch(ctx, attn_decode_split_kernel<DD>, grid, block, 0, kv->k_pool, kv->v_pool, kv->page_table_dev,     \
-               nctx_dev, q_dev, partial, kv->n_head, kv->page_tokens, kv->pages_per_seq, n_splits, scale, seq_fixed)
+    do {                                                                                                           \
+        if (page_shift >= 0)                                                                                       \
+            skn_launch(ctx, attn_decode_kernel<DD, true>, grid, block, 0, kv->k_pool, kv->v_pool,                  \
+                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, kv->n_head,                \
+                       kv->page_tokens, page_shift, kv->pages_per_seq, n_splits, scale, seq_fixed);                \
+        else                                                                                                       \
+            skn_launch(ctx, attn_decode_kernel<DD, false>, grid, block, 0, kv->k_pool, kv->v_pool,                 \
+                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, kv->n_head,                \
+                       kv->page_tokens, page_shift, kv->pages_per_seq, n_splits, scale, seq_fixed);                \
+    } while (0)
     if (D == 64) SKN_ATTN_LAUNCH(64);
     else if (D == 128) SKN_ATTN_LAUNCH(128);
     else SKN_ATTN_LAUNCH(256);
 #undef SKN_ATTN_LAUNCH
     SKN_LAUNCH_CHECK(ctx);
-    skn_launch(ctx, attn_merge_kernel, dim3(n_queries * kv->n_head), dim3(D), 0, (const float*)partial, out_dev,
-               n_splits, D);
-    SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
 
 int skn_attn_splits(skn_ctx* ctx, int pairs, int max_ctx) {
-    const int tiles = (max_ctx + kTile - 1) / kTile;
+    const int chunks = (max_ctx + 63) / 64;  // a split should hold at least one full iteration of a workgroup
     int n_splits = ctx->opt_attn_splits > 0 ? ctx->opt_attn_splits : (4 * ctx->compute_units + pairs - 1) / pairs;
-    if (n_splits > tiles) n_splits = tiles;
+    if (n_splits > chunks) n_splits = chunks;
+    if (n_splits > kMaxSplits) n_splits = kMaxSplits;
     return n_splits < 1 ? 1 : n_splits;
+}
+
+// Allocates zeroed split counters; shared with the decoder, which owns its own.
+int skn_attn_alloc_counters(skn_ctx* ctx, int n_pairs, int** out) {
+    *out = nullptr;
+    hipError_t e = hipMalloc((void**)out, (size_t)n_pairs * sizeof(int));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return skn_fail(ctx, SKN_ERR_OOM, "attention split counters (%d): %s", n_pairs, hipGetErrorString(e));
+    }
+    SKN_HIP(ctx, hipMemsetAsync(*out, 0, (size_t)n_pairs * sizeof(int), ctx->stream));
+    return SKN_OK;
 }
 
 int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
@@ -201,8 +301,18 @@ int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t*
         }
         ctx->attn_scratch_bytes = grow;
     }
-    return skn_attn_launch_ex(ctx, kv, q_dev, nctx_dev, kv->n_seq, -1, n_splits, (float*)ctx->attn_scratch, scale,
-                              out_dev);
+    if (pairs > ctx->attn_counters_cap) {
+        SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        if (ctx->attn_counters) SKN_HIP(ctx, hipFree(ctx->attn_counters));
+        ctx->attn_counters = nullptr;
+        ctx->attn_counters_cap = 0;
+        const int cap = pairs < 1024 ? 1024 : pairs;
+        const int rc = skn_attn_alloc_counters(ctx, cap, &ctx->attn_counters);
+        if (rc != SKN_OK) return rc;
+        ctx->attn_counters_cap = cap;
+    }
+    return skn_attn_launch_ex(ctx, kv, q_dev, nctx_dev, kv->n_seq, -1, n_splits, (float*)ctx->attn_scratch,
+                              ctx->attn_counters, scale, out_dev);
 }
 
 extern "C" int skn_attn_decode(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* n_ctx_host, float scale,

@@ -32,6 +32,8 @@ struct skn_ctx {
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
+    int* attn_counters = nullptr;  // one per (sequence, head): workgroups of a split attention count themselves in
+    int attn_counters_cap = 0;
     // GEMM workspace (fp16 activations, dequantized weight pairs), grown on demand
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;

@@ -15,6 +15,7 @@ struct skn_llama {
     // decode-step buffers
     float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *att = nullptr, *proj = nullptr;
     float *gate = nullptr, *up = nullptr, *mid = nullptr, *logits = nullptr, *attn_partial = nullptr;
+    int *attn_counters = nullptr, *pcounters = nullptr;  // split counters of the attention launches (zero between launches)
     int32_t* state = nullptr;       // [0] token, [1] position, [2] context length, [3] step index
     int32_t* tokens_out = nullptr;  // device array of produced tokens
     int tokens_cap = 0;
@@ -249,7 +250,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
                        kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
                        kv->page_tokens, log2f(c.rope_base));
             SKN_LAUNCH_CHECK(ctx);
-            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, scale, m->att));
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));
             skn_q4k_segments gu = {{(const uint8_t*)L.w_gate, (const uint8_t*)L.w_up, nullptr}, {F, F, 0}};
@@ -267,7 +268,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
                    kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
                    kv->page_tokens, log2f(c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, scale, m->att));
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
         SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wo, H, H, m->att, m->proj));
         skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
         SKN_LAUNCH_CHECK(ctx);
@@ -319,6 +320,8 @@ int ensure_prompt_buffers(skn_ctx* ctx, skn_llama* m, int T) {
     SKN_TRY(dev_alloc(ctx, m, &m->pnctx, (size_t)T));
     // splits = ceil(4 * CUs / pairs) bounds pairs * splits by pairs + 4 * CUs
     SKN_TRY(dev_alloc(ctx, m, &m->ppartial, ((size_t)T * c.n_head + 4 * (size_t)ctx->compute_units) * (c.head_dim + 2)));
+    SKN_TRY(dev_alloc(ctx, m, &m->pcounters, (size_t)T * c.n_head));
+    SKN_HIP(ctx, hipMemsetAsync(m->pcounters, 0, (size_t)T * c.n_head * sizeof(int), ctx->stream));
     m->prompt_cap = T;
     return SKN_OK;
 }
@@ -385,6 +388,11 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
         if (m->layers[l].type_attn != SKN_TYPE_Q4_K || m->layers[l].type_ffn != SKN_TYPE_Q4_K) m->fused = false;
     A(&m->gate, F); A(&m->up, F); A(&m->mid, F); A(&m->logits, (size_t)cfg->vocab);
     A(&m->attn_partial, (size_t)cfg->n_head * max_splits * (cfg->head_dim + 2));
+    A(&m->attn_counters, (size_t)cfg->n_head);
+    if (rc == SKN_OK && hipMemsetAsync(m->attn_counters, 0, (size_t)cfg->n_head * sizeof(int), ctx->stream) != hipSuccess) {
+        (void)hipGetLastError();
+        rc = skn_fail(ctx, SKN_ERR_HIP, "skn_llama_create: clearing the attention counters failed");
+    }
     A(&m->state, (size_t)4);
     m->tokens_cap = cfg->max_tokens;
     A(&m->tokens_out, (size_t)m->tokens_cap);
@@ -454,7 +462,7 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
                    kv->page_tokens, log2f(c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, scale, m->patt));
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
         SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
         SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
         skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,

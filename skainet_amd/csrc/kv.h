@@ -25,5 +25,5 @@ int skn_kv_reserve(skn_ctx* ctx, skn_kv* kv, int seq, int new_len);
 int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
                     float* out_dev);
 int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
-                       int seq_fixed, int n_splits, float* partial, float scale, float* out_dev);
+                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev);
 int skn_attn_splits(skn_ctx* ctx, int pairs, int max_ctx);

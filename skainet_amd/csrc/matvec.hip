@@ -150,7 +150,8 @@ __device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* _
     for (int r = 0; r < R; r++) {
         float sc0, sc1, m0, m1;
         q4k_pair_scales(L[r].h, pair, sc0, sc1, m0, m1);
-        const half2_t dd = __builtin_bit_cast(half2_t, L[r].h.x);
+        const uint32_t dword0 = L[r].h.x;  // by value: a bit cast of a vector element reads the whole vector's start
+        const half2_t dd = __builtin_bit_cast(half2_t, dword0);
         const float t1 = fmaf(sc1, ahi[r], sc0 * alo[r]);
         const float t2 = fmaf(m1, sx.y, m0 * sx.x);
         const float v = fmaf((float)dd.x, t1, -((float)dd.y * t2));
