@@ -48,9 +48,20 @@ struct skn_q4k_segments {
     const uint8_t* w[3];
     int rows[3];
 };
-enum { SKN_EPI_STORE = 0, SKN_EPI_ADD = 1, SKN_EPI_SWIGLU = 2 };
+// SKN_EPI_ROPE: the three segments are the q, k and v projections of one token.  A wavefront's two rows are
+// one rotary pair: q pairs are rotated and stored to y (fp32), k pairs are rotated and stored as fp16 into the
+// cache page of the token's position, v pairs are stored as fp16 beside them.
+enum { SKN_EPI_STORE = 0, SKN_EPI_ADD = 1, SKN_EPI_SWIGLU = 2, SKN_EPI_ROPE = 3 };
+struct skn_rope_epilogue {
+    const int32_t* pos_dev = nullptr;     // position of the token (device scalar)
+    const int32_t* page_table = nullptr;  // page table row of the token's sequence
+    uint16_t* k_pool = nullptr;
+    uint16_t* v_pool = nullptr;
+    int n_head = 0, head_dim = 0, page_tokens = 0;
+    float log2_base = 0.f;
+};
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
-                         float eps, float* y, int epi);
+                         float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr);
 
 // Records a failure on the context (or on the context-less slot) and returns `code`.
 int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);

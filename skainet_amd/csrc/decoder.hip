@@ -39,40 +39,48 @@ namespace {
 // ---- kernels that read their step-dependent scalars from device memory -----------------------------------
 
 // One row of a [vocab, hidden] quantized embedding table -> fp32.  grid = rows to embed, tokens from device.
-__global__ __launch_bounds__(256) void embed_rows_kernel(const uint8_t* __restrict__ table, int type, int hidden,
+__global__ __launch_bounds__(1024) void embed_rows_kernel(const uint8_t* __restrict__ table, int type, int hidden,
                                                          const int32_t* __restrict__ tokens, float* __restrict__ out) {
     const int row = blockIdx.x;
     const int tok = tokens[row];
     float* dst = out + (size_t)row * hidden;
     if (type == SKN_TYPE_Q4_K) {
+        // four consecutive elements per thread: one sub-block, four consecutive nibble bytes (one aligned dword)
         const uint8_t* src = table + (size_t)tok * (hidden / 256) * 144;
-        for (int e = threadIdx.x; e < hidden; e += 256) {
+        for (int e = 4 * threadIdx.x; e < hidden; e += 4 * blockDim.x) {
             const uint8_t* b = src + (size_t)(e >> 8) * 144;
             const int i = e & 255, c = i >> 6, r = i & 63, j = 2 * c + (r >= 32);
-            const uint8_t* s = b + 4;
+            const uint4 hdr = *reinterpret_cast<const uint4*>(b);  // d | dmin, scales[0..11]
+            const uint32_t w[3] = {hdr.y, hdr.z, hdr.w};
+            auto sbyte = [&](int k) { return (w[k >> 2] >> (8 * (k & 3))) & 0xFFu; };
             int sc, m;
             if (j < 4) {
-                sc = s[j] & 63;
-                m = s[j + 4] & 63;
+                sc = sbyte(j) & 63;
+                m = sbyte(j + 4) & 63;
             } else {
-                sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
-                m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+                sc = (sbyte(j + 4) & 0x0F) | ((sbyte(j - 4) >> 6) << 4);
+                m = (sbyte(j + 4) >> 4) | ((sbyte(j) >> 6) << 4);
             }
-            const uint32_t dd = *reinterpret_cast<const uint32_t*>(b);
-            const uint8_t byte = b[16 + 32 * c + (r & 31)];
-            const int qv = (r < 32) ? (byte & 0xF) : (byte >> 4);
-            dst[e] = __fsub_rn(__fmul_rn(__fmul_rn(h2f_bits(dd & 0xFFFF), (float)sc), (float)qv),
-                               __fmul_rn(h2f_bits(dd >> 16), (float)m));
+            const uint32_t q4 = *reinterpret_cast<const uint32_t*>(b + 16 + 32 * c + (r & 31));
+            const float ds = __fmul_rn(h2f_bits(hdr.x & 0xFFFF), (float)sc);
+            const float mm = __fmul_rn(h2f_bits(hdr.x >> 16), (float)m);
+            const int sh = (r < 32) ? 0 : 4;
+            float4 o;
+            o.x = __fsub_rn(__fmul_rn(ds, (float)((q4 >> sh) & 0xF)), mm);
+            o.y = __fsub_rn(__fmul_rn(ds, (float)((q4 >> (8 + sh)) & 0xF)), mm);
+            o.z = __fsub_rn(__fmul_rn(ds, (float)((q4 >> (16 + sh)) & 0xF)), mm);
+            o.w = __fsub_rn(__fmul_rn(ds, (float)((q4 >> (24 + sh)) & 0xF)), mm);
+            *reinterpret_cast<float4*>(dst + e) = o;
         }
     } else if (type == SKN_TYPE_Q8_0) {
         const uint8_t* src = table + (size_t)tok * (hidden / 32) * 34;
-        for (int e = threadIdx.x; e < hidden; e += 256) {
+        for (int e = threadIdx.x; e < hidden; e += blockDim.x) {
             const uint8_t* b = src + (size_t)(e >> 5) * 34;
             dst[e] = __fmul_rn(h2f_bits(load_u16_a2(b)), (float)(int8_t)b[2 + (e & 31)]);
         }
     } else if (type == SKN_TYPE_Q6_K) {
         const uint8_t* src = table + (size_t)tok * (hidden / 256) * 210;
-        for (int e = threadIdx.x; e < hidden; e += 256) {
+        for (int e = threadIdx.x; e < hidden; e += blockDim.x) {
             const uint8_t* b = src + (size_t)(e >> 8) * 210;
             const int i = e & 255, n = i >> 7, r = i & 127, quarter = r >> 5, l = r & 31;
             uint32_t lo = b[64 * n + l + 32 * (quarter & 1)];
@@ -83,7 +91,7 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(const uint8_t* __restri
         }
     } else {  // F32
         const float* src = reinterpret_cast<const float*>(table) + (size_t)tok * hidden;
-        for (int e = threadIdx.x; e < hidden; e += 256) dst[e] = src[e];
+        for (int e = threadIdx.x; e < hidden; e += blockDim.x) dst[e] = src[e];
     }
 }
 
@@ -113,18 +121,45 @@ __global__ void rope_store_kernel(float* __restrict__ q, const float* __restrict
     *reinterpret_cast<uint32_t*>(v_pool + dst) = vv;
 }
 
-__global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ y,
-                                    int n, float eps) {
+// grid = rows, block = 256.  Rows of up to 8192 elements (multiple of 4) stay in registers between the two
+// passes and all loads are issued before the first use.
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                           float* __restrict__ y, int n, float eps) {
     __shared__ float red[4];
     const float* xr = x + (size_t)blockIdx.x * n;
     float* yr = y + (size_t)blockIdx.x * n;
+    const int tid = threadIdx.x;
+    const bool in_regs = (n & 3) == 0 && n <= 8192;
+    float4 v[8], g[8];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    if (in_regs) {
+        const int n4 = n >> 2;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = min(tid + 256 * j, n4 - 1);
+            v[j] = reinterpret_cast<const float4*>(xr)[i];
+            g[j] = reinterpret_cast<const float4*>(w)[i];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (tid + 256 * j < n4) ss += (v[j].x * v[j].x + v[j].y * v[j].y) + (v[j].z * v[j].z + v[j].w * v[j].w);
+    } else {
+        for (int i = tid; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    }
     ss = wave_sum(ss);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
     __syncthreads();
     const float r = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)n + eps);
-    for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * r * w[i];
+    if (in_regs) {
+        const int n4 = n >> 2;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (tid + 256 * j < n4)
+                reinterpret_cast<float4*>(yr)[tid + 256 * j] =
+                    make_float4(v[j].x * r * g[j].x, v[j].y * r * g[j].y, v[j].z * r * g[j].z, v[j].w * r * g[j].w);
+    } else {
+        for (int i = tid; i < n; i += 256) yr[i] = xr[i] * r * w[i];
+    }
 }
 
 __global__ void add_rows_kernel(float* __restrict__ y, const float* __restrict__ x, int64_t n) {
@@ -167,13 +202,30 @@ __global__ __launch_bounds__(1024) void finish_step_kernel(const float* __restri
     __shared__ int bi[16];
     float best = -INFINITY;
     int besti = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const float v = x[i];
+    auto take = [&](float v, int i) {
         if (v > best || (v == best && i < besti)) {
             best = v;
             besti = i;
         }
+    };
+    // eight float4 per thread and round, all loaded before the first compare
+    const int n4 = n >> 2;
+    for (int base = 0; base < n4; base += 8 * 1024) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = reinterpret_cast<const float4*>(x)[min(base + j * 1024 + (int)threadIdx.x, n4 - 1)];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i4 = base + j * 1024 + (int)threadIdx.x;
+            if (i4 < n4) {
+                take(v[j].x, 4 * i4);
+                take(v[j].y, 4 * i4 + 1);
+                take(v[j].z, 4 * i4 + 2);
+                take(v[j].w, 4 * i4 + 3);
+            }
+        }
     }
+    for (int i = 4 * n4 + threadIdx.x; i < n; i += 1024) take(x[i], i);
     for (int off = 32; off >= 1; off >>= 1) {
         const float ov = __shfl_xor(best, off, 64);
         const int oi = __shfl_xor(besti, off, 64);
@@ -235,21 +287,26 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     const skn_llama_config& c = m->cfg;
     const int H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim;
     const float scale = 1.0f / sqrtf((float)D);
-    skn_launch(ctx, embed_rows_kernel, dim3(1), dim3(256), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
+    skn_launch(ctx, embed_rows_kernel, dim3(1), dim3(1024), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
                (const int32_t*)m->state, m->x);
     SKN_LAUNCH_CHECK(ctx);
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
         if (m->fused && ctx->opt_llama_fused) {
-            // seven launches per layer: [norm + q,k,v], rope + cache store, attention (2), [Wo + residual],
+            // five launches per layer: [norm + q,k,v + rope + cache store], attention, [Wo + residual],
             // [norm + gate,up + SwiGLU], [Wdown + residual]
             skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, H, H}};
-            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, 3 * H, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_STORE));
-            skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
-                       kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
-                       kv->page_tokens, log2f(c.rope_base));
-            SKN_LAUNCH_CHECK(ctx);
+            skn_rope_epilogue rope;
+            rope.pos_dev = m->state + 1;
+            rope.page_table = kv->page_table_dev;
+            rope.k_pool = kv->k_pool;
+            rope.v_pool = kv->v_pool;
+            rope.n_head = NH;
+            rope.head_dim = D;
+            rope.page_tokens = kv->page_tokens;
+            rope.log2_base = log2f(c.rope_base);
+            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, 3 * H, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope));
             SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));

@@ -327,7 +327,8 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
 template <int STEPS, int EPI, bool NORM>
 __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments seg, const float* __restrict__ x,
                                                                const float* __restrict__ norm_w, float eps,
-                                                               float* __restrict__ y, int n_out, int nb) {
+                                                               float* __restrict__ y, int n_out, int nb,
+                                                               skn_rope_epilogue rope) {
     constexpr int R = 2;
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
@@ -423,7 +424,35 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const float t0 = wave_sum(acc[0]) * 16777216.0f;
     const float t1 = wave_sum(acc[1]) * 16777216.0f;
     if (lane == 0) {
-        if (EPI == SKN_EPI_SWIGLU) {
+        if (EPI == SKN_EPI_ROPE) {
+            // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
+            int row = unit * R;
+            if (row_ok[0]) {
+                const int pos = rope.pos_dev[0];
+                const int which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
+                row -= which == 2 ? seg.rows[0] + seg.rows[1] : which == 1 ? seg.rows[0] : 0;
+                const int h = row / rope.head_dim, e = row % rope.head_dim;
+                float a = t0, b = t1;
+                if (which < 2) {
+                    const float inv_freq = exp2f(-(float)e / (float)rope.head_dim * rope.log2_base);
+                    float sn, cs;
+                    sincosf((float)pos * inv_freq, &sn, &cs);
+                    a = t0 * cs - t1 * sn;
+                    b = t0 * sn + t1 * cs;
+                }
+                if (which == 0) {
+                    y[row] = a;
+                    y[row + 1] = b;
+                } else {
+                    const int page = rope.page_table[pos / rope.page_tokens];
+                    const size_t dst =
+                        (((size_t)page * rope.n_head + h) * rope.page_tokens + (pos % rope.page_tokens)) * rope.head_dim + e;
+                    const uint32_t packed = (uint32_t)__half_as_ushort(__float2half_rn(a)) |
+                                            ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+                    *reinterpret_cast<uint32_t*>((which == 1 ? rope.k_pool : rope.v_pool) + dst) = packed;
+                }
+            }
+        } else if (EPI == SKN_EPI_SWIGLU) {
             if (row_ok[0]) y[unit] = t0 / (1.0f + expf(-t0)) * t1;
         } else if (EPI == SKN_EPI_ADD) {
             if (row_ok[0]) y[unit * R] += t0;
@@ -437,27 +466,30 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
 
 template <int STEPS, int EPI, bool NORM>
 int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
-                     float eps, float* y) {
+                     float eps, float* y, const skn_rope_epilogue& rope) {
     const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2)) + 8 * sizeof(float);
     const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
     dim3 grid((unsigned)((units + 7) / 8)), block(512);
-    skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb);
+    skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
 
 template <int STEPS>
 int dispatch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
-                       float eps, float* y, int epi) {
+                       float eps, float* y, int epi, const skn_rope_epilogue& rope) {
     const bool norm = norm_w != nullptr;
+    if (epi == SKN_EPI_ROPE)
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ROPE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_ROPE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
     if (epi == SKN_EPI_SWIGLU)
-        return norm ? launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
-                    : launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
     if (epi == SKN_EPI_ADD)
-        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ADD, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
-                    : launch_q4k_fused<STEPS, SKN_EPI_ADD, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
-    return norm ? launch_q4k_fused<STEPS, SKN_EPI_STORE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y)
-                : launch_q4k_fused<STEPS, SKN_EPI_STORE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y);
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ADD, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_ADD, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
+    return norm ? launch_q4k_fused<STEPS, SKN_EPI_STORE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                : launch_q4k_fused<STEPS, SKN_EPI_STORE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
 }
 
 template <int STEPS, int EPI, bool NORM>
@@ -474,6 +506,8 @@ hipError_t allow_big_lds_fused_all() {
     if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, true>();
     if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, false>();
     if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, true>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, false>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, true>();
     return e;
 }
 
@@ -528,14 +562,24 @@ int skn_matvec_init(skn_ctx* ctx) {
 
 // Fused Q4_K matvec for the decoder; k <= 16384 (four unrolled steps).  Returns SKN_ERR_SHAPE otherwise.
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
-                         float eps, float* y, int epi) {
+                         float eps, float* y, int epi, const skn_rope_epilogue* rope_in) {
     SKN_REQUIRE(ctx, k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_SHAPE, "fused Q4_K matvec: unsupported k %d", k);
+    skn_rope_epilogue rope;
+    if (epi == SKN_EPI_ROPE) {
+        SKN_REQUIRE(ctx, rope_in && rope_in->pos_dev && rope_in->page_table && rope_in->k_pool && rope_in->v_pool,
+                    SKN_ERR_ARG, "fused Q4_K matvec: the rotary epilogue needs its cache arguments");
+        rope = *rope_in;
+        SKN_REQUIRE(ctx, rope.head_dim > 0 && rope.head_dim % 2 == 0 && seg.rows[0] % rope.head_dim == 0 &&
+                             seg.rows[1] == rope.n_head * rope.head_dim && seg.rows[2] == seg.rows[1],
+                    SKN_ERR_SHAPE, "fused Q4_K matvec: q/k/v rows do not match %d heads of %d", rope.n_head,
+                    rope.head_dim);
+    }
     const int nb = k / 256;
     switch ((nb + 15) / 16) {
-        case 1: return dispatch_q4k_fused<1>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
-        case 2: return dispatch_q4k_fused<2>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
-        case 3: return dispatch_q4k_fused<3>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
-        default: return dispatch_q4k_fused<4>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi);
+        case 1: return dispatch_q4k_fused<1>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
+        case 2: return dispatch_q4k_fused<2>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
+        case 3: return dispatch_q4k_fused<3>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
+        default: return dispatch_q4k_fused<4>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
     }
 }
 

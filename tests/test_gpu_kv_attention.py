@@ -188,3 +188,27 @@ def test_benchmark_shape_step(hip):
     gk, gv = _gather(hip, kv, 5, 4095, 4096)
     assert np.array_equal(gk[0], k1[5]) and np.array_equal(gv[0], v1[5])
     kv.free()
+
+
+def test_attention_split_counts_and_repeated_launches(hip):
+    """Every split count gives the same answer, launch after launch: the per-(sequence, head) counters that
+    elect the merging workgroup are left at zero by each launch.  Pages of 48 tokens (not a power of two)."""
+    n_seq, n_head, dim = 3, 4, 128
+    lens = [700, 5, 193]
+    kv = hip.kv_cache(n_seq, n_head, dim, 48, 720)
+    k, v = _fill(hip, kv, lens, seed=41)
+    q = np.random.default_rng(6).standard_normal((n_seq, n_head, dim)).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle_c.attn_decode(q, k, v, lens, scale)
+    out = hip.alloc(q.nbytes)
+    qd = hip.to_device(q)
+    try:
+        for splits in (1, 2, 3, 7, 11, 64, 0, 5, 5, 5):
+            hip.set_option("attn.splits", splits)
+            out.upload(np.full(q.shape, np.nan, np.float32))
+            kv.attn_decode(qd, out, scale)
+            got = out.download(np.float32, q.size).reshape(q.shape)
+            assert oracle_np.rel_err(got, want) <= TOL, splits
+    finally:
+        hip.set_option("attn.splits", 0)
+    kv.free()
