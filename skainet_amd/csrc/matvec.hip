@@ -319,6 +319,52 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
     if (lane == 0) y[row] = acc;
 }
 
+// What the first lane does with the two row totals of unit `unit` (rows 2*unit, 2*unit + 1; for SwiGLU: row
+// `unit` of gate and of up).
+template <int EPI>
+__device__ __forceinline__ void q4k_epilogue(const skn_q4k_segments& seg, const skn_rope_epilogue& rope,
+                                             float* __restrict__ y, int n_out, int unit, float t0, float t1) {
+    const bool ok0 = EPI == SKN_EPI_SWIGLU ? unit < n_out : 2 * unit < n_out;
+    const bool ok1 = EPI == SKN_EPI_SWIGLU ? ok0 : 2 * unit + 1 < n_out;
+    if (EPI == SKN_EPI_ROPE) {
+        // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
+        int row = unit * 2;
+        if (ok0) {
+            const int pos = rope.pos_dev[0];
+            const int which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
+            row -= which == 2 ? seg.rows[0] + seg.rows[1] : which == 1 ? seg.rows[0] : 0;
+            const int h = row / rope.head_dim, e = row % rope.head_dim;
+            float a = t0, b = t1;
+            if (which < 2) {
+                const float inv_freq = exp2f(-(float)e / (float)rope.head_dim * rope.log2_base);
+                float sn, cs;
+                sincosf((float)pos * inv_freq, &sn, &cs);
+                a = t0 * cs - t1 * sn;
+                b = t0 * sn + t1 * cs;
+            }
+            if (which == 0) {
+                y[row] = a;
+                y[row + 1] = b;
+            } else {
+                const int page = rope.page_table[pos / rope.page_tokens];
+                const size_t dst =
+                    (((size_t)page * rope.n_head + h) * rope.page_tokens + (pos % rope.page_tokens)) * rope.head_dim + e;
+                const uint32_t packed = (uint32_t)__half_as_ushort(__float2half_rn(a)) |
+                                        ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
+                *reinterpret_cast<uint32_t*>((which == 1 ? rope.k_pool : rope.v_pool) + dst) = packed;
+            }
+        }
+    } else if (EPI == SKN_EPI_SWIGLU) {
+        if (ok0) y[unit] = t0 / (1.0f + expf(-t0)) * t1;
+    } else if (EPI == SKN_EPI_ADD) {
+        if (ok0) y[unit * 2] += t0;
+        if (ok1) y[unit * 2 + 1] += t1;
+    } else {
+        if (ok0) y[unit * 2] = t0;
+        if (ok1) y[unit * 2 + 1] = t1;
+    }
+}
+
 // ---- fused forms used by the decoder ---------------------------------------------------------------------
 // Up to three weight matrices with the same k stacked along the output axis (q, k, v projections in one launch;
 // gate and up paired row by row), optional RMSNorm of x folded into the staging (every workgroup needs all of
@@ -423,45 +469,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     }
     const float t0 = wave_sum(acc[0]) * 16777216.0f;
     const float t1 = wave_sum(acc[1]) * 16777216.0f;
-    if (lane == 0) {
-        if (EPI == SKN_EPI_ROPE) {
-            // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
-            int row = unit * R;
-            if (row_ok[0]) {
-                const int pos = rope.pos_dev[0];
-                const int which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
-                row -= which == 2 ? seg.rows[0] + seg.rows[1] : which == 1 ? seg.rows[0] : 0;
-                const int h = row / rope.head_dim, e = row % rope.head_dim;
-                float a = t0, b = t1;
-                if (which < 2) {
-                    const float inv_freq = exp2f(-(float)e / (float)rope.head_dim * rope.log2_base);
-                    float sn, cs;
-                    sincosf((float)pos * inv_freq, &sn, &cs);
-                    a = t0 * cs - t1 * sn;
-                    b = t0 * sn + t1 * cs;
-                }
-                if (which == 0) {
-                    y[row] = a;
-                    y[row + 1] = b;
-                } else {
-                    const int page = rope.page_table[pos / rope.page_tokens];
-                    const size_t dst =
-                        (((size_t)page * rope.n_head + h) * rope.page_tokens + (pos % rope.page_tokens)) * rope.head_dim + e;
-                    const uint32_t packed = (uint32_t)__half_as_ushort(__float2half_rn(a)) |
-                                            ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
-                    *reinterpret_cast<uint32_t*>((which == 1 ? rope.k_pool : rope.v_pool) + dst) = packed;
-                }
-            }
-        } else if (EPI == SKN_EPI_SWIGLU) {
-            if (row_ok[0]) y[unit] = t0 / (1.0f + expf(-t0)) * t1;
-        } else if (EPI == SKN_EPI_ADD) {
-            if (row_ok[0]) y[unit * R] += t0;
-            if (row_ok[1]) y[unit * R + 1] += t1;
-        } else {
-            if (row_ok[0]) y[unit * R] = t0;
-            if (row_ok[1]) y[unit * R + 1] = t1;
-        }
-    }
+    if (lane == 0) q4k_epilogue<EPI>(seg, rope, y, n_out, unit, t0, t1);
 }
 
 template <int STEPS, int EPI, bool NORM>
