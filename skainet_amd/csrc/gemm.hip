@@ -18,7 +18,10 @@
 namespace {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kBM = 128;  // workgroup tile rows (activations)
@@ -27,12 +30,9 @@ constexpr int kKC = 64;   // k elements staged in LDS per iteration
 constexpr int kRow = kKC + 8;  // LDS row pitch in halves: 144 bytes keeps 128-bit reads of 16 rows conflict-free
 
 // ---- activation preparation: bf16 [m,k] -> fp16 [m,k] with a per-row power-of-two scale -------------------
-// One workgroup per row.  Also emits, for the Q4_K path, the per-32-element sums of the fp16 row as an fp16
-// pair (hi, lo), and can write the row in the element order the Q4_K kernel consumes (PERMUTE).
-template <bool Q4K>
+// One workgroup per row.
 __global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict__ a, _Float16* __restrict__ a16,
-                                                     float* __restrict__ inv_scale, _Float16* __restrict__ sum_hi,
-                                                     _Float16* __restrict__ sum_lo, int k) {
+                                                     float* __restrict__ inv_scale, int k) {
     __shared__ float red[4];
     const int m = blockIdx.x;
     const uint16_t* ar = a + (size_t)m * k;
@@ -51,26 +51,82 @@ __global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict_
     const float scale = __uint_as_float((uint32_t)(127 - e) << 23);
     if (threadIdx.x == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 + e) << 23);
     _Float16* out = a16 + (size_t)m * k;
-    if (!Q4K) {
-        for (int i = threadIdx.x; i < k; i += 256) out[i] = (_Float16)(__uint_as_float((uint32_t)ar[i] << 16) * scale);
-    } else {
-        // one thread per 32-element sub-block: its sum, and the permuted store
-        const int nsub = k >> 5;
-        for (int s = threadIdx.x; s < nsub; s += 256) {
-            float sum = 0.f;
-            const int chunk = s >> 1, upper = s & 1;  // 64-element chunk, lower / upper 32 elements
-            for (int i = 0; i < 32; i++) {
-                const _Float16 h = (_Float16)(__uint_as_float((uint32_t)ar[32 * s + i] << 16) * scale);
-                sum += (float)h;
-                // element 32*upper + 4*dw + b of the chunk (dw = dword of nibble bytes, b = byte in it) goes to
-                // position dw*8 + {0,4,1,5}[b] + 2*upper: the order the nibble masks of the Q4_K kernel produce
-                const int dw = i >> 2, b = i & 3;
-                const int pos = dw * 8 + ((b & 1) << 2) + (b >> 1) + 2 * upper;
-                out[64 * chunk + pos] = h;
+    for (int i = threadIdx.x; i < k; i += 256) out[i] = (_Float16)(__uint_as_float((uint32_t)ar[i] << 16) * scale);
+}
+
+// Q4_K path.  The row is scaled by a power of two so that its largest magnitude lies in [2^9, 2^10): the
+// conversion to fp16 is exact down to 2^-24 (34 binades below the row maximum) and the sum of a 32-element
+// sub-block (needed for the "- dmin * m" term) stays below the fp16 maximum; each sum is kept as an fp16 pair
+// (hi, lo).  The row is written in the element order in which the Q4_K kernel unpacks weights: task (c, dw) =
+// (64-element chunk, dword of its 32 nibble bytes) gathers elements 4*dw + {0,1,2,3} of the chunk's lower and
+// upper half and writes them as [lo0, lo2, hi0, hi2, lo1, lo3, hi1, hi3] at 64*c + 8*dw.
+// One workgroup per row, eight tasks at most per thread (k <= 16384); eight consecutive lanes share a chunk.
+__global__ __launch_bounds__(256) void prep_a_q4k_kernel(const uint16_t* __restrict__ a, _Float16* __restrict__ a16,
+                                                         float* __restrict__ inv_scale, _Float16* __restrict__ sum_hi,
+                                                         _Float16* __restrict__ sum_lo, int k) {
+    __shared__ float red[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    const uint16_t* ar = a + (size_t)m * k;
+    const int tasks = k >> 3;
+    uint2 lo[8], hi[8];
+    float mx = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int task = min(tid + 256 * j, tasks - 1);
+        const int c = task >> 3, dw = task & 7;
+        lo[j] = *reinterpret_cast<const uint2*>(ar + 64 * c + 4 * dw);
+        hi[j] = *reinterpret_cast<const uint2*>(ar + 64 * c + 32 + 4 * dw);
+    }
+    auto widen = [](uint32_t pair, int which) { return __uint_as_float(which ? pair & 0xFFFF0000u : pair << 16); };
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t w4[4] = {lo[j].x, lo[j].y, hi[j].x, hi[j].y};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float v = fabsf(widen(w4[i >> 1], i & 1));
+            if (v == v && v < INFINITY) mx = fmaxf(mx, v);
+        }
+    }
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int e = 9;  // a zero row keeps scale 1
+    if (mx > 0.f) e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+    e = max(e, -100);  // (a subnormal maximum: exponent field 0)
+    const float scale = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
+    if (tid == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+    _Float16* out = a16 + (size_t)m * k;
+    const int nsub = k >> 5;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int task = tid + 256 * j;
+        const int c = task >> 3, dw = task & 7;
+        _Float16 l[4], u[4];
+        l[0] = (_Float16)(widen(lo[j].x, 0) * scale), l[1] = (_Float16)(widen(lo[j].x, 1) * scale);
+        l[2] = (_Float16)(widen(lo[j].y, 0) * scale), l[3] = (_Float16)(widen(lo[j].y, 1) * scale);
+        u[0] = (_Float16)(widen(hi[j].x, 0) * scale), u[1] = (_Float16)(widen(hi[j].x, 1) * scale);
+        u[2] = (_Float16)(widen(hi[j].y, 0) * scale), u[3] = (_Float16)(widen(hi[j].y, 1) * scale);
+        float sl = ((float)l[0] + (float)l[1]) + ((float)l[2] + (float)l[3]);
+        float su = ((float)u[0] + (float)u[1]) + ((float)u[2] + (float)u[3]);
+        // totals over the eight lanes of the chunk (all lanes run the permutations; tail tasks are clamped copies)
+        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0xB1, 0xF, 0xF, true));
+        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0xB1, 0xF, 0xF, true));
+        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x4E, 0xF, 0xF, true));
+        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x4E, 0xF, 0xF, true));
+        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x141, 0xF, 0xF, true));
+        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x141, 0xF, 0xF, true));
+        if (task < tasks) {
+            half8_t o;
+            o[0] = l[0], o[1] = l[2], o[2] = u[0], o[3] = u[2], o[4] = l[1], o[5] = l[3], o[6] = u[1], o[7] = u[3];
+            *reinterpret_cast<half8_t*>(out + 64 * c + 8 * dw) = o;
+            if (dw == 0) {
+                const _Float16 h0 = (_Float16)sl, h1 = (_Float16)su;
+                sum_hi[(size_t)m * nsub + 2 * c] = h0;
+                sum_lo[(size_t)m * nsub + 2 * c] = (_Float16)(sl - (float)h0);
+                sum_hi[(size_t)m * nsub + 2 * c + 1] = h1;
+                sum_lo[(size_t)m * nsub + 2 * c + 1] = (_Float16)(su - (float)h1);
             }
-            const _Float16 hi = (_Float16)sum;
-            sum_hi[(size_t)m * nsub + s] = hi;
-            sum_lo[(size_t)m * nsub + s] = (_Float16)(sum - (float)hi);
         }
     }
 }
@@ -179,6 +235,171 @@ __global__ __launch_bounds__(256) void gemm_dense_hilo_kernel(const _Float16* __
 #undef SKN_STASH
 }
 
+// ---- Q4_K path: weights unpacked in the kernel, one MFMA per k-step ----------------------------------------
+// w[n, 256 b + e] = d * (sc_j * q) - dmin * m_j  (j = sub-block of e).  sc_j * q is an integer below 2^10: the
+// nibble masked in place is the fp16 subnormal q * 2^-24 (or 16 q * 2^-24 for a high nibble) and one packed
+// fp16 multiply by sc_j (or sc_j / 16) gives sc_j * q * 2^-24 exactly -- an fp16 operand the matrix core takes
+// as is.  Per superblock the products are accumulated in a partial tile, which is then folded into the total
+// with the column's d * 2^24; the "- dmin * m_j" term is a second, eight-deep product per superblock between
+// the activation sub-block sums (fp16 hi + lo) and the integers m_j, folded in with dmin.
+// Workgroup tile 128 x 64, 64 k per iteration (one chunk of every weight row: 32 nibble bytes, a quarter per
+// thread, unpacked into 64 fp16).
+__global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restrict__ a16,
+                                                       const _Float16* __restrict__ sum_hi,
+                                                       const _Float16* __restrict__ sum_lo,
+                                                       const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
+                                                       float* __restrict__ c, int m, int n, int k) {
+    // 2 x 2 wavefronts, each a 64 x 32 part of the tile.
+    // Two LDS buffers (one barrier per iteration) and a ring of four register stages: the global loads of
+    // iterations it+1 .. it+3 are in flight while iteration it is multiplied.  Four iterations = one superblock,
+    // so the position in the ring is also the chunk index within the superblock.  Every thread issues the same
+    // loads every iteration (no load sits in a conditional block): the wait counters then say exactly which
+    // stage is complete.
+    __shared__ __align__(16) _Float16 sa[2][kBM * kRow];
+    __shared__ __align__(16) _Float16 sb[2][kBN * kRow];
+    __shared__ float sd[2][kBN], sdm[2][kBN];
+    __shared__ __align__(8) _Float16 smin[2][kBN * 8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+    const int nb = k >> 8, nsub = k >> 5;
+
+    struct Stage {
+        u32x4 a0, a1, a2, a3, h;
+        u32x2 q;
+    };
+    Stage st[4];
+    // activation staging: 128 rows x 8 chunks of 16 bytes, four per thread
+    const int srow = tid >> 3, sch = (tid & 7) * 8;
+    const _Float16* ga0 = a16 + (size_t)min(m0 + srow, m - 1) * k + sch;
+    const _Float16* ga1 = a16 + (size_t)min(m0 + srow + 32, m - 1) * k + sch;
+    const _Float16* ga2 = a16 + (size_t)min(m0 + srow + 64, m - 1) * k + sch;
+    const _Float16* ga3 = a16 + (size_t)min(m0 + srow + 96, m - 1) * k + sch;
+    // weight staging: thread t owns row t / 4 of the tile and quarter t % 4 of the 32 nibble bytes of a chunk
+    const int brow = tid >> 2, bq = tid & 3;
+    const uint8_t* gw = w + (size_t)min(n0 + brow, n - 1) * nb * 144;
+
+    auto fetch = [&](int sbk, int cc, Stage& s) __attribute__((always_inline)) {
+        const int k0 = (4 * sbk + cc) * kKC;
+        s.a0 = *reinterpret_cast<const u32x4*>(ga0 + k0);
+        s.a1 = *reinterpret_cast<const u32x4*>(ga1 + k0);
+        s.a2 = *reinterpret_cast<const u32x4*>(ga2 + k0);
+        s.a3 = *reinterpret_cast<const u32x4*>(ga3 + k0);
+        s.h = *reinterpret_cast<const u32x4*>(gw + (size_t)sbk * 144);
+        s.q = *reinterpret_cast<const u32x2*>(gw + (size_t)sbk * 144 + 16 + 32 * cc + 8 * bq);
+    };
+    auto stash = [&](int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
+        _Float16* da = sa[cc & 1];
+        _Float16* db = sb[cc & 1];
+        *reinterpret_cast<u32x4*>(da + srow * kRow + sch) = s.a0;
+        *reinterpret_cast<u32x4*>(da + (srow + 32) * kRow + sch) = s.a1;
+        *reinterpret_cast<u32x4*>(da + (srow + 64) * kRow + sch) = s.a2;
+        *reinterpret_cast<u32x4*>(da + (srow + 96) * kRow + sch) = s.a3;
+        // the whole loaded tuple counts as used here: a word that this chunk does not need (d | dmin outside
+        // chunk 0) would otherwise be recycled as a temporary while its load is in flight, and writing it
+        // would wait for that load
+        asm volatile("" ::"v"(s.h));
+        const uint32_t hw[4] = {s.h.x, s.h.y, s.h.z, s.h.w};
+        auto sbyte = [&](int i) { return (hw[1 + (i >> 2)] >> (8 * (i & 3))) & 0xFFu; };
+        auto scale_of = [&](int j) {
+            return j < 4 ? (int)(sbyte(j) & 63) : (int)((sbyte(j + 4) & 0x0F) | ((sbyte(j - 4) >> 6) << 4));
+        };
+        auto min_of = [&](int j) {
+            return j < 4 ? (int)(sbyte(j + 4) & 63) : (int)((sbyte(j + 4) >> 4) | ((sbyte(j) >> 6) << 4));
+        };
+        const _Float16 ml = (_Float16)(float)scale_of(2 * cc);
+        const _Float16 mh = (_Float16)((float)scale_of(2 * cc + 1) * 0.0625f);
+        const half2_t mul_lo = {ml, ml}, mul_hi = {mh, mh};
+        const uint32_t q2[2] = {s.q.x, s.q.y};
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t q = q2[j], q8 = q >> 8;
+            const uint32_t l02 = q & 0x000F000Fu, h02 = q & 0x00F000F0u;
+            const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
+            u32x4 o;
+            o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo);
+            o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi);
+            o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo);
+            o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi);
+            *reinterpret_cast<u32x4*>(db + brow * kRow + 16 * bq + 8 * j) = o;
+        }
+        if (cc == 0 && bq == 0) {  // per superblock: the column's d * 2^24, dmin and the eight m_j
+            const half2_t dd = __builtin_bit_cast(half2_t, hw[0]);
+            sd[sbk & 1][brow] = (float)dd.x * 16777216.0f;
+            sdm[sbk & 1][brow] = (float)dd.y;
+            half8_t mm;
+#pragma unroll
+            for (int j = 0; j < 8; j++) mm[j] = (_Float16)(float)min_of(j);
+            *reinterpret_cast<half8_t*>(smin[sbk & 1] + brow * 8) = mm;
+        }
+    };
+
+    float16_t tot0, tot1, par0, par1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) tot0[r] = tot1[r] = par0[r] = par1[r] = 0.f;
+
+    // activation sub-block sums of this wavefront's two row tiles: lane l holds row l % 32, sub-blocks
+    // 4 * (l / 32) .. + 3 of the current superblock (the operand layout of the eight-deep matrix instruction)
+    const int srow0 = min(m0 + wm * 64 + (lane & 31), m - 1), srow1 = min(m0 + wm * 64 + 32 + (lane & 31), m - 1);
+    const size_t soff0 = (size_t)srow0 * nsub + 4 * (lane >> 5), soff1 = (size_t)srow1 * nsub + 4 * (lane >> 5);
+    const int pfrag = (lane & 31) * kRow + (lane >> 5) * 8;
+
+    // (issue order pinned: oldest stage first, as in the loop, so that the wait for a stage never covers a
+    // younger one)
+    fetch(0, 0, st[0]);
+    fetch(0, 1, st[1]);
+    fetch(0, 2, st[2]);
+    for (int sbk = 0; sbk < nb; sbk++) {
+        half4_t sh0, sl0, sh1, sl1;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+            // the stage three iterations ahead
+            if (cc == 0) fetch(sbk, 3, st[3]);
+            else fetch(min(sbk + 1, nb - 1), cc - 1, st[cc - 1]);  // (past the end: repeats the last superblock, unused)
+            if (cc == 0) {
+                sh0 = *reinterpret_cast<const half4_t*>(sum_hi + soff0 + 8 * sbk);
+                sl0 = *reinterpret_cast<const half4_t*>(sum_lo + soff0 + 8 * sbk);
+                sh1 = *reinterpret_cast<const half4_t*>(sum_hi + soff1 + 8 * sbk);
+                sl1 = *reinterpret_cast<const half4_t*>(sum_lo + soff1 + 8 * sbk);
+            }
+            {
+                stash(sbk, cc, st[cc]);
+                __syncthreads();  // buffer cc & 1 is complete; the other one is free once every wavefront is here
+                const _Float16* pa0 = sa[cc & 1] + wm * 64 * kRow + pfrag;
+                const _Float16* pa1 = pa0 + 32 * kRow;
+                const _Float16* pb = sb[cc & 1] + wn * 32 * kRow + pfrag;
+#pragma unroll
+                for (int t = 0; t < kKC / 16; t++) {
+                    const half8_t fa0 = *reinterpret_cast<const half8_t*>(pa0 + 16 * t);
+                    const half8_t fa1 = *reinterpret_cast<const half8_t*>(pa1 + 16 * t);
+                    const half8_t fb = *reinterpret_cast<const half8_t*>(pb + 16 * t);
+                    par0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0, fb, par0, 0, 0, 0);
+                    par1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1, fb, par1, 0, 0, 0);
+                }
+            }
+        }
+        // end of the superblock: fold the partial tiles into the totals
+        const half4_t fm = *reinterpret_cast<const half4_t*>(smin[sbk & 1] + (wn * 32 + (lane & 31)) * 8 + 4 * (lane >> 5));
+        float16_t mn0, mn1;
+#pragma unroll
+        for (int r = 0; r < 16; r++) mn0[r] = mn1[r] = 0.f;
+        mn0 = __builtin_amdgcn_mfma_f32_32x32x8f16(sh0, fm, mn0, 0, 0, 0);
+        mn1 = __builtin_amdgcn_mfma_f32_32x32x8f16(sh1, fm, mn1, 0, 0, 0);
+        mn0 = __builtin_amdgcn_mfma_f32_32x32x8f16(sl0, fm, mn0, 0, 0, 0);
+        mn1 = __builtin_amdgcn_mfma_f32_32x32x8f16(sl1, fm, mn1, 0, 0, 0);
+        const float ds = sd[sbk & 1][wn * 32 + (lane & 31)];
+        const float dm = sdm[sbk & 1][wn * 32 + (lane & 31)];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            tot0[r] = fmaf(ds, par0[r], fmaf(-dm, mn0[r], tot0[r]));
+            tot1[r] = fmaf(ds, par1[r], fmaf(-dm, mn1[r], tot1[r]));
+            par0[r] = par1[r] = 0.f;
+        }
+    }
+    store_tile(tot0, c, n, m0 + wm * 64, n0 + wn * 32, m, n, inv_scale, lane);
+    store_tile(tot1, c, n, m0 + wm * 64 + 32, n0 + wn * 32, m, n, inv_scale, lane);
+}
+
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
 int gemm_workspace(skn_ctx* ctx, size_t bytes, uint8_t** out) {
     if (bytes > ctx->gemm_ws_bytes) {
@@ -216,6 +437,28 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     SKN_REQUIRE(ctx, w_dev && a_bf16_dev, SKN_ERR_ARG, "skn_gemm_q: null pointer");
     SKN_REQUIRE(ctx, k % kKC == 0, SKN_ERR_SHAPE, "skn_gemm_q: k (%d) must be a multiple of %d", k, kKC);
 
+    if (ggml_type == SKN_TYPE_Q4_K && k <= 16384) {
+        // workspace: permuted fp16 activations, row scales, sub-block sums (hi, lo)
+        const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
+        const size_t sum_bytes = align_up((size_t)m * (k / 32) * 2);
+        uint8_t* ws;
+        int rc = gemm_workspace(ctx, a16_bytes + sc_bytes + 2 * sum_bytes, &ws);
+        if (rc != SKN_OK) return rc;
+        _Float16* a16 = (_Float16*)ws;
+        float* inv_scale = (float*)(ws + a16_bytes);
+        _Float16* sum_hi = (_Float16*)(ws + a16_bytes + sc_bytes);
+        _Float16* sum_lo = (_Float16*)(ws + a16_bytes + sc_bytes + sum_bytes);
+        SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
+                    "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
+        skn_launch(ctx, prep_a_q4k_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, sum_hi, sum_lo, k);
+        SKN_LAUNCH_CHECK(ctx);
+        dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
+        skn_launch(ctx, gemm_q4k_kernel, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
+                   (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
+        SKN_LAUNCH_CHECK(ctx);
+        return SKN_OK;
+    }
+
     // workspace: fp16 activations + row scales, then (general path) fp32 weights and their fp16 pair
     const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
     const size_t wf_bytes = align_up((size_t)n * k * 4), wh_bytes = align_up((size_t)n * k * 2);
@@ -228,8 +471,7 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     _Float16* whi = (_Float16*)(ws + a16_bytes + sc_bytes + wf_bytes);
     _Float16* wlo = (_Float16*)(ws + a16_bytes + sc_bytes + wf_bytes + wh_bytes);
 
-    skn_launch(ctx, prep_a_kernel<false>, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, (_Float16*)nullptr,
-               (_Float16*)nullptr, k);
+    skn_launch(ctx, prep_a_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, k);
     SKN_LAUNCH_CHECK(ctx);
     rc = skn_dequant(ctx, ggml_type, w_dev, (int64_t)n * k, wf);
     if (rc != SKN_OK) return rc;
