@@ -135,6 +135,30 @@ def bench_attention(ctx, steps, warmup):
     }
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def bench_gemm(ctx, qtype, m, n, k, reps=20):
+    """Prefill GEMM C[m,n] = A[m,k] . deq(W)[n,k]^T (A bf16): summed kernel time of one call (activation
+    preparation included), 2mnk flops against the dense fp16 matrix-core peak."""
+    w = ctx.to_device(synth.weight(qtype, n, k, seed=3))
+    a = ctx.to_device(synth.activation_bf16((m, k), seed=4))
+    c = ctx.alloc(4 * m * n)
+    for _ in range(3):
+        ctx.gemm_q(qtype, w, n, k, a, m, c)
+    ctx.sync()
+    ctx.prof_start(8 * reps)
+    for _ in range(reps):
+        ctx.gemm_q(qtype, w, n, k, a, m, c)
+    ms, launches = ctx.prof_stop()
+    for buf in (w, a, c):
+        buf.free()
+    us = ms / reps * 1e3
+    tflops = 2.0 * m * n * k / us / 1e6
+    return {"us_per_gemm": round(us, 1), "launches_per_gemm": launches // reps, "tflops": round(tflops, 1),
+            "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+
 def cpu_baseline(qtype, n, k, budget_s=12.0):
     """The CPU oracle (C, OpenMP over rows) on the headline workload; a bounded number of repetitions."""
     from oracle import oracle_c  # the checker, timed as the "port" CPU baseline -- never the product path
@@ -174,8 +198,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy", "decode"], default="bench",
-                    help="decode: only the 7B-shape decode leg (for kernel traces of one token step).  copy: run --steps plain device copies of the headline weight size instead (the known-size "
+    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm"], default="bench",
+                    help="decode / attention / gemm: only that leg (for kernel traces).  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode without the captured step graph (kernel tracers that cannot follow graph launches)")
@@ -207,6 +231,17 @@ def main():
         print(json.dumps({"mode": "decode", **llama_bench.run(ctx, steps=min(args.steps, 128))}))
         ctx.close()
         return
+    gemm_shapes = [("q4_k", Q4_K, 512, 4096, 4096), ("q4_k", Q4_K, 512, 14336, 4096),
+                   ("q6_k", Q6_K, 512, 4096, 4096), ("q6_k", Q6_K, 512, 14336, 4096)]
+    if args.mode == "attention":
+        print(json.dumps({"mode": "attention", **bench_attention(ctx, min(args.steps, 200), 10)}))
+        ctx.close()
+        return
+    if args.mode == "gemm":
+        print(json.dumps({"mode": "gemm", **{f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
+                                             for nm, qt, mm, nn, kk in gemm_shapes}}))
+        ctx.close()
+        return
     head = bench_matvec(ctx, Q4_K, n, k, args.steps, args.warmup)
 
     extra = {"device": info["name"], "compute_units": info["compute_units"]}
@@ -221,6 +256,8 @@ def main():
             extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
         att = bench_attention(ctx, min(args.steps, 200), 10)
         extra["attention_8x32x128_ctx4096"] = {key: round(val, 4) for key, val in att.items()}
+        extra["prefill_gemm"] = {f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
+                                 for nm, qt, mm, nn, kk in gemm_shapes}
         try:
             from skainet_amd import llama_bench
             extra["decode_7b_q4_k"] = llama_bench.run(ctx)
@@ -253,7 +290,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(head["kernel_gbs"] / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # HBM bytes of one launch from hardware counters (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, one run
+            # each, scaled by what the same counters read for a copy kernel of this size): 1.017 x algorithmic
+            "traffic": 25850432,
             "kernel": "matvec_q4k_kernel",
             "kernel_us": round(head["kernel_us"], 3),
             "cache_hot_gbs": round(head["hot_kernel_gbs"], 2),
