@@ -91,19 +91,22 @@ __device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int 
     for (int j = 0; j < J; j++) st.v[j] = x4[min(tid + j * nthreads, n4 - 1)];
 }
 
+// Q4K: the scalings of the Q4_K kernel.  Otherwise (Q8_0): x is stored as is and the half-column sums are
+// multiplied by 128, the offset that turns the signed quants into unsigned bytes.
+template <bool Q4K = true>
 __device__ __forceinline__ void q4k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
     const int cc = f >> 4, i16 = f & 15;
     const int step = cc >> 6, ln = cc & 63;
-    const float mul = (i16 & 8) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
+    const float mul = (Q4K && (i16 & 8)) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
     xs[(step * 16 + i16) * kXPitch + ln] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
     float sum = (v.x + v.y) + (v.z + v.w);
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));   // lane ^ 1
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x4E, 0xF, 0xF, true));   // lane ^ 2
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x141, 0xF, 0xF, true));  // 7 - lane
-    if ((f & 7) == 0) ss[f >> 3] = sum * 5.9604644775390625e-08f;  // 2^-24, see the scaling note above
+    if ((f & 7) == 0) ss[f >> 3] = sum * (Q4K ? 5.9604644775390625e-08f : 128.0f);  // 2^-24, see the scaling note above
 }
 
-template <int J>
+template <int J, bool Q4K = true>
 __device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, int tid, int nthreads, float4* xs,
                                                 float* ss) {
 #pragma unroll
@@ -111,7 +114,7 @@ __device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, i
         // a float4 index past the end repeats the last one: same data to the same slot (no branch; whole
         // groups of eight lanes are clamped together because n4 is a multiple of 64)
         const int f = min(tid + j * nthreads, n4 - 1);
-        q4k_stage_store_one(st.v[j], f, xs, ss);
+        q4k_stage_store_one<Q4K>(st.v[j], f, xs, ss);
     }
 }
 
@@ -256,9 +259,127 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
 
 // ------------------------------------------------------------------------------------------ Q8_0
 //
-// 34-byte blocks (f16 d, 32 x int8), only 2-byte aligned.  One wavefront per row; lane l takes blocks
-// l, l+64, ...  The lane's 34 bytes are fetched as seventeen 16-bit loads (consecutive lanes read
-// consecutive blocks, so the wavefront still walks one contiguous range) and x as eight aligned float4.
+// 34-byte blocks (f16 d, 32 x int8), only 2-byte aligned.  Two consecutive blocks are 68 bytes = 17 dwords:
+//   dword 0 = d0 | q0 q1, dwords 1..7 = q2..q29, dword 8 = q30 q31 | d1, dwords 9..16 = the 32 quants of the
+// second block.  When the row is a whole number of pairs and 4-byte aligned, lane l of a step takes pair
+// 64 * step + l (four 16-byte loads and one dword at 4-byte alignment): the second block's quants are aligned
+// dwords, the first block's are realigned with v_alignbyte.  Signed bytes become unsigned by flipping the top
+// bit (q + 128), which v_cvt_f32_ubyteN converts with the byte select built in: one convert and one fused
+// multiply-add per weight; the offset comes back out as 128 * sum(x of the block), formed once per workgroup
+// while x is staged.  Staging, lookahead and reduction are those of the Q4_K kernel (a lane's 64 activations
+// are the same 64 consecutive elements there and here).
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+struct Q80Loads {
+    u32x4 w[4];    // dwords 0..15
+    uint32_t w16;  // dword 16
+    bool ok;
+};
+
+__device__ __forceinline__ float q80_dot_dword(uint32_t q, const float4& x, float s) {
+    const uint32_t u = q ^ 0x80808080u;
+    s = fmaf((float)(u & 0xFF), x.x, s);          // (each of these is one v_cvt_f32_ubyteN)
+    s = fmaf((float)((u >> 8) & 0xFF), x.y, s);
+    s = fmaf((float)((u >> 16) & 0xFF), x.z, s);
+    s = fmaf((float)(u >> 24), x.w, s);
+    return s;
+}
+
+template <int R>
+__device__ __forceinline__ void q80_step(const Q80Loads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, float (&acc)[R]) {
+    float sa[R], sb[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) sa[r] = sb[r] = 0.f;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        float4 xa[4], xb[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xa[j] = xs[(s * 16 + 4 * half + j) * kXPitch + lane];
+            xb[j] = xs[(s * 16 + 8 + 4 * half + j) * kXPitch + lane];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            uint32_t w[17];
+#pragma unroll
+            for (int i = 0; i < 16; i++) w[i] = L[r].w[i >> 2][i & 3];
+            w[16] = L[r].w16;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = 4 * half + j;
+                sa[r] = q80_dot_dword(__builtin_amdgcn_alignbyte(w[i + 1], w[i], 2), xa[j], sa[r]);
+                sb[r] = q80_dot_dword(w[9 + i], xb[j], sb[r]);
+            }
+        }
+    }
+    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t w0 = L[r].w[0].x, w8 = L[r].w[2].x;
+        const float d0 = h2f_bits(w0 & 0xFFFF), d1 = h2f_bits(w8 >> 16);
+        const float v = fmaf(d0, sa[r] - sx.x, d1 * (sb[r] - sx.y));
+        acc[r] += L[r].ok ? v : 0.f;
+    }
+}
+
+template <int STEPS, int R>
+__global__ __launch_bounds__(512) void matvec_q80_pairs_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                               float* __restrict__ y, int n_rows, int npairs) {
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row0 = (blockIdx.x * 8 + wave) * R;
+    const int n4 = npairs * 16;  // float4 count of x
+    constexpr int J = 2 * STEPS;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+
+    float acc[R];
+    const uint8_t* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        rp[r] = w + (size_t)min(row0 + r, n_rows - 1) * npairs * 68;
+    }
+    Q80Loads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int pr = s * 64 + lane;
+        const size_t off = (size_t)(min(pr, npairs - 1) + tie) * 68;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const u32x4_a4* bp = reinterpret_cast<const u32x4_a4*>(rp[r] + off);
+#pragma unroll
+            for (int i = 0; i < 4; i++) L[s][r].w[i] = bp[i];
+            L[s][r].w16 = *reinterpret_cast<const uint32_t*>(rp[r] + off + 64);
+            L[s][r].ok = row_ok[r] && pr < npairs;
+        }
+    };
+    issue(0, 0);
+    q4k_stage_store<J, false>(st, n4, tid, 512, xs, ss);
+    __syncthreads();
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        q80_step<R>(L[s], xs, ss, s, lane + tie, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
+    }
+}
+
+// General form (any alignment, any block count): one wavefront per row; lane l takes blocks l, l+64, ...  The
+// lane's 34 bytes are fetched as seventeen 16-bit loads (consecutive lanes read consecutive blocks, so the
+// wavefront still walks one contiguous range) and x as eight aligned float4.
 __global__ __launch_bounds__(256) void matvec_q8_0_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                           float* __restrict__ y, int n_rows, int nb) {
     const int lane = threadIdx.x & 63;
@@ -288,7 +409,156 @@ __global__ __launch_bounds__(256) void matvec_q8_0_kernel(const uint8_t* __restr
 
 // ------------------------------------------------------------------------------------------ Q6_K
 //
-// 210-byte superblocks, 2-byte aligned.  One wavefront per row, one superblock per step: lane (n, l) =
+// 210-byte superblocks (ql[128], qh[64], int8 scales[16], f16 d), 2-byte aligned.  Main kernel (k <= 16384):
+// the Q4_K scheme with four lanes per superblock.  Lane (b, j) = (lane / 4, lane % 4) of a step owns half
+// n = j / 2 of superblock b and the byte positions l = 16 * (j % 2) .. + 15 in it: 16 bytes of ql[64n + l],
+// 16 of ql[64n + 32 + l], 16 of qh[32n + l] -- three 128-bit loads at 2-byte alignment (the device takes
+// unaligned vector loads) -- plus the eight scales of the half and d.  Those bytes hold the 64 weights
+// 128n + 32q + l (q = 0..3), i.e. four runs of sixteen consecutive activations, each run under one scale.
+// Four bytes at a time: the 6-bit values of run q are assembled in place,
+//     (ql & 0x0F0F0F0F | qh << 4 & 0x30303030), (ql' & ... | qh << 2 & ...), (ql >> 4 & ... | qh & ...), ...
+// and a byte pair masked out (v & 0x00FF00FF) is a pair of fp16 subnormals u * 2^-24 that v_fma_mix_f32
+// multiplies with the fp32 activation: about 2.4 VALU operations per weight.  The zero point 32 comes back out
+// as 32 * sum(x of the run), formed while x is staged; x is staged in lane order (slot 4q + i of a lane = i-th
+// float4 of its run q) so the LDS reads are conflict-free and serve both rows of the wavefront.
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+
+struct Q6kLoads {
+    u32x4 la, lb, h;
+    u32x2 sc;
+    uint32_t d;
+    bool ok;
+};
+
+// float4 f of x -> (step, lane, slot) of the Q6_K lane order; also the run sums
+__device__ __forceinline__ void q6k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
+    const int e = 4 * f;
+    const int b = e >> 8, r = e & 255;
+    const int n = r >> 7, q = (r >> 5) & 3, l = r & 31;
+    const int lane_all = 4 * b + 2 * n + (l >> 4);
+    const int step = lane_all >> 6, ln = lane_all & 63;
+    const int slot = 4 * q + ((l & 15) >> 2);
+    xs[(step * 16 + slot) * kXPitch + ln] = v;
+    float sum = (v.x + v.y) + (v.z + v.w);
+    sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+    sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x4E, 0xF, 0xF, true));  // lane ^ 2
+    if ((f & 3) == 0) ss[(step * 64 + ln) * 4 + q] = sum * (32.0f * 5.9604644775390625e-08f);  // 32 * 2^-24
+}
+
+__device__ __forceinline__ float q6k_dot4(uint32_t v, const float4& x, float s) {
+    const half2_t b02 = __builtin_bit_cast(half2_t, v & 0x00FF00FFu);
+    const half2_t b13 = __builtin_bit_cast(half2_t, (v >> 8) & 0x00FF00FFu);
+    s = fmaf((float)b02.x, x.x, s);
+    s = fmaf((float)b13.x, x.y, s);
+    s = fmaf((float)b02.y, x.z, s);
+    s = fmaf((float)b13.y, x.w, s);
+    return s;
+}
+
+template <int R>
+__device__ __forceinline__ void q6k_step(const Q6kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, int hsel, float (&acc)[R]) {
+    float S[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) S[r][0] = S[r][1] = S[r][2] = S[r][3] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float4 xq[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) xq[q] = xs[(s * 16 + 4 * q + i) * kXPitch + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t la = L[r].la[i], lb = L[r].lb[i], h = L[r].h[i];
+            const uint32_t v0 = (la & 0x0F0F0F0Fu) | ((h << 4) & 0x30303030u);
+            const uint32_t v1 = (lb & 0x0F0F0F0Fu) | ((h << 2) & 0x30303030u);
+            const uint32_t v2 = ((la >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u);
+            const uint32_t v3 = ((lb >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u);
+            S[r][0] = q6k_dot4(v0, xq[0], S[r][0]);
+            S[r][1] = q6k_dot4(v1, xq[1], S[r][1]);
+            S[r][2] = q6k_dot4(v2, xq[2], S[r][2]);
+            S[r][3] = q6k_dot4(v3, xq[3], S[r][3]);
+        }
+    }
+    const float4 sx = reinterpret_cast<const float4*>(ss)[s * 64 + lane];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        // scales hsel, hsel + 2, hsel + 4, hsel + 6 of the half's eight
+        const uint32_t w0 = L[r].sc.x >> (8 * hsel), w1 = L[r].sc.y >> (8 * hsel);
+        const float c0 = (float)(int)(int8_t)(w0 & 0xFF), c1 = (float)(int)(int8_t)((w0 >> 16) & 0xFF);
+        const float c2 = (float)(int)(int8_t)(w1 & 0xFF), c3 = (float)(int)(int8_t)((w1 >> 16) & 0xFF);
+        float v = c0 * (S[r][0] - sx.x);
+        v = fmaf(c1, S[r][1] - sx.y, v);
+        v = fmaf(c2, S[r][2] - sx.z, v);
+        v = fmaf(c3, S[r][3] - sx.w, v);
+        acc[r] += L[r].ok ? h2f_bits(L[r].d) * v : 0.f;
+    }
+}
+
+template <int STEPS, int R>
+__global__ __launch_bounds__(512) void matvec_q6k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ y, int n_rows, int nb) {
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);  // float4 per (step, lane)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 2, j = lane & 3, n = j >> 1, hsel = j & 1;
+    const int row0 = (blockIdx.x * 8 + wave) * R;
+    const int n4 = nb * 64;
+    constexpr int J = 2 * STEPS;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+
+    float acc[R];
+    const uint8_t* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        rp[r] = w + (size_t)min(row0 + r, n_rows - 1) * nb * 210;
+    }
+    Q6kLoads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int blk = s * 16 + sub;
+        const size_t off = (size_t)(min(blk, nb - 1) + tie) * 210;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t* bp = rp[r] + off;
+            L[s][r].la = *reinterpret_cast<const u32x4_a2*>(bp + 64 * n + 16 * hsel);
+            L[s][r].lb = *reinterpret_cast<const u32x4_a2*>(bp + 64 * n + 32 + 16 * hsel);
+            L[s][r].h = *reinterpret_cast<const u32x4_a2*>(bp + 128 + 32 * n + 16 * hsel);
+            L[s][r].sc = *reinterpret_cast<const u32x2_a2*>(bp + 192 + 8 * n);
+            L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 208);
+            L[s][r].ok = row_ok[r] && blk < nb;
+        }
+    };
+    issue(0, 0);
+#pragma unroll
+    for (int jj = 0; jj < J; jj++) {
+        // a float4 index past the end repeats the last one: same data to the same slot
+        const int f = min(tid + jj * 512, n4 - 1);
+        q6k_stage_store_one(st.v[jj], f, xs, ss);
+    }
+    __syncthreads();
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        q6k_step<R>(L[s], xs, ss, s, lane + tie, hsel, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]) * 16777216.0f;
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
+    }
+}
+
+// General form (any k): one wavefront per row, one superblock per step: lane (n, l) =
 // (lane / 32, lane % 32) owns the four elements 128n + l + {0, 32, 64, 96}, which share the bytes
 // ql[64n + l], ql[64n + l + 32] and qh[32n + l]; the 64 lanes read 64 consecutive bytes per load.
 __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
@@ -545,6 +815,38 @@ int dispatch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, 
     }
 }
 
+template <int STEPS>
+int launch_q80_pairs(skn_ctx* ctx, const uint8_t* w, int n, int npairs, const float* x, float* y) {
+    constexpr int R = 2;
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
+    dim3 grid((unsigned)((n + 8 * R - 1) / (8 * R))), block(512);
+    skn_launch(ctx, matvec_q80_pairs_kernel<STEPS, R>, grid, block, lds, w, x, y, n, npairs);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int STEPS>
+int launch_q6k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y) {
+    constexpr int R = 1;
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float4));
+    dim3 grid((unsigned)((n + 8 * R - 1) / (8 * R))), block(512);
+    skn_launch(ctx, matvec_q6k_kernel<STEPS, R>, grid, block, lds, w, x, y, n, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int STEPS>
+hipError_t allow_big_lds_q6k() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q6k_kernel<STEPS, 1>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
+template <int STEPS>
+hipError_t allow_big_lds_q80() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q80_pairs_kernel<STEPS, 2>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
 template <int STEPS, int R>
 hipError_t allow_big_lds() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R>),
@@ -561,6 +863,14 @@ int skn_matvec_init(skn_ctx* ctx) {
                              allow_big_lds<3, 2>, allow_big_lds<4, 2>, allow_big_lds<0, 4>, allow_big_lds<1, 4>,
                              allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>};
     for (auto f : fns) SKN_HIP(ctx, f());
+    SKN_HIP(ctx, allow_big_lds_q6k<1>());
+    SKN_HIP(ctx, allow_big_lds_q6k<2>());
+    SKN_HIP(ctx, allow_big_lds_q6k<3>());
+    SKN_HIP(ctx, allow_big_lds_q6k<4>());
+    SKN_HIP(ctx, allow_big_lds_q80<1>());
+    SKN_HIP(ctx, allow_big_lds_q80<2>());
+    SKN_HIP(ctx, allow_big_lds_q80<3>());
+    SKN_HIP(ctx, allow_big_lds_q80<4>());
     SKN_HIP(ctx, allow_big_lds_fused_all<1>());
     SKN_HIP(ctx, allow_big_lds_fused_all<2>());
     SKN_HIP(ctx, allow_big_lds_fused_all<3>());
@@ -618,6 +928,23 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         return rows >= 4   ? dispatch_q4k<4>(ctx, w, n, nb, x_dev, y_dev, waves)
                : rows >= 2 ? dispatch_q4k<2>(ctx, w, n, nb, x_dev, y_dev, waves)
                            : dispatch_q4k<1>(ctx, w, n, nb, x_dev, y_dev, waves);
+    }
+    if (ggml_type == SKN_TYPE_Q8_0 && nb % 2 == 0 && nb <= 512 && ((uintptr_t)w_dev & 3) == 0) {
+        const int npairs = nb / 2;
+        switch ((npairs + 63) / 64) {
+            case 1: return launch_q80_pairs<1>(ctx, w, n, npairs, x_dev, y_dev);
+            case 2: return launch_q80_pairs<2>(ctx, w, n, npairs, x_dev, y_dev);
+            case 3: return launch_q80_pairs<3>(ctx, w, n, npairs, x_dev, y_dev);
+            default: return launch_q80_pairs<4>(ctx, w, n, npairs, x_dev, y_dev);
+        }
+    }
+    if (ggml_type == SKN_TYPE_Q6_K && nb <= 64) {
+        switch ((nb + 15) / 16) {
+            case 1: return launch_q6k<1>(ctx, w, n, nb, x_dev, y_dev);
+            case 2: return launch_q6k<2>(ctx, w, n, nb, x_dev, y_dev);
+            case 3: return launch_q6k<3>(ctx, w, n, nb, x_dev, y_dev);
+            default: return launch_q6k<4>(ctx, w, n, nb, x_dev, y_dev);
+        }
     }
     dim3 grid((unsigned)((n + 3) / 4)), block(256);
     if (ggml_type == SKN_TYPE_Q8_0)

@@ -73,7 +73,21 @@ MATVEC_CASES = [
     (Q4_K, 3, 57 * 256),
     (Q8_0, 33, 96),
     (Q8_0, 7, 32 * 131),
+    # Q8_0 rows that are whole block pairs: one lane step partly filled, several steps, the largest unrolled
+    # size, and one past it (general kernel)
+    (Q8_0, 3, 64),
+    (Q8_0, 5, 64 * 70),
+    (Q8_0, 17, 8192),
+    (Q8_0, 2, 12800),
+    (Q8_0, 9, 16384),
+    (Q8_0, 4, 16384 + 64),
     (Q6_K, 19, 768),
+    (Q6_K, 5, 256),
+    (Q6_K, 33, 256 * 17),
+    (Q6_K, 3, 256 * 50),
+    (Q6_K, 2, 16384),
+    (Q6_K, 2, 16384 + 256),  # past the unrolled sizes: general kernel
+    (Q6_K, 1000, 4096),
 ]
 
 
