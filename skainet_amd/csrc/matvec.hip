@@ -922,7 +922,7 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;
         if (waves <= 0) waves = 8;
-        if (rows <= 0) rows = 2;
+        if (rows <= 0) rows = nb > 32 ? 1 : 2;  // measured: long rows (three or more steps) are 2.5 % faster one per wavefront
         if (waves > 8) waves = 8;
         if (rows >= 4 && nb > 32) rows = 2;  // four rows of three or more unrolled steps do not fit the registers
         return rows >= 4   ? dispatch_q4k<4>(ctx, w, n, nb, x_dev, y_dev, waves)
