@@ -589,39 +589,53 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
     if (lane == 0) y[row] = acc;
 }
 
+// What the rotary epilogue needs beyond the row totals, formed at the top of the kernel so that its dependent
+// loads (position, then page id) and the sine / cosine are off the tail of the wavefront.
+struct Q4kRopeCtx {
+    int which = 0, h = 0, e = 0, page = 0, slot = 0;  // q / k / v, head, element pair, cache page and slot
+    float sn = 0.f, cs = 1.f;
+};
+
+__device__ __forceinline__ Q4kRopeCtx q4k_rope_prepare(const skn_q4k_segments& seg, const skn_rope_epilogue& rope,
+                                                     int unit) {
+    Q4kRopeCtx c;
+    int row = unit * 2;  // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
+    c.which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
+    row -= c.which == 2 ? seg.rows[0] + seg.rows[1] : c.which == 1 ? seg.rows[0] : 0;
+    c.h = row / rope.head_dim;
+    c.e = row % rope.head_dim;
+    const int pos = rope.pos_dev[0];
+    const int pi = pos / rope.page_tokens;
+    c.slot = pos - pi * rope.page_tokens;
+    c.page = rope.page_table[pi];
+    const float inv_freq = exp2f(-(float)c.e / (float)rope.head_dim * rope.log2_base);
+    sincosf((float)pos * inv_freq, &c.sn, &c.cs);
+    return c;
+}
+
 // What the first lane does with the two row totals of unit `unit` (rows 2*unit, 2*unit + 1; for SwiGLU: row
 // `unit` of gate and of up).
 template <int EPI>
-__device__ __forceinline__ void q4k_epilogue(const skn_q4k_segments& seg, const skn_rope_epilogue& rope,
+__device__ __forceinline__ void q4k_epilogue(const skn_rope_epilogue& rope, const Q4kRopeCtx& rc,
                                              float* __restrict__ y, int n_out, int unit, float t0, float t1) {
     const bool ok0 = EPI == SKN_EPI_SWIGLU ? unit < n_out : 2 * unit < n_out;
     const bool ok1 = EPI == SKN_EPI_SWIGLU ? ok0 : 2 * unit + 1 < n_out;
     if (EPI == SKN_EPI_ROPE) {
-        // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
-        int row = unit * 2;
         if (ok0) {
-            const int pos = rope.pos_dev[0];
-            const int which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
-            row -= which == 2 ? seg.rows[0] + seg.rows[1] : which == 1 ? seg.rows[0] : 0;
-            const int h = row / rope.head_dim, e = row % rope.head_dim;
             float a = t0, b = t1;
-            if (which < 2) {
-                const float inv_freq = exp2f(-(float)e / (float)rope.head_dim * rope.log2_base);
-                float sn, cs;
-                sincosf((float)pos * inv_freq, &sn, &cs);
-                a = t0 * cs - t1 * sn;
-                b = t0 * sn + t1 * cs;
+            if (rc.which < 2) {
+                a = t0 * rc.cs - t1 * rc.sn;
+                b = t0 * rc.sn + t1 * rc.cs;
             }
-            if (which == 0) {
-                y[row] = a;
-                y[row + 1] = b;
+            if (rc.which == 0) {
+                y[rc.h * rope.head_dim + rc.e] = a;
+                y[rc.h * rope.head_dim + rc.e + 1] = b;
             } else {
-                const int page = rope.page_table[pos / rope.page_tokens];
                 const size_t dst =
-                    (((size_t)page * rope.n_head + h) * rope.page_tokens + (pos % rope.page_tokens)) * rope.head_dim + e;
+                    (((size_t)rc.page * rope.n_head + rc.h) * rope.page_tokens + rc.slot) * rope.head_dim + rc.e;
                 const uint32_t packed = (uint32_t)__half_as_ushort(__float2half_rn(a)) |
                                         ((uint32_t)__half_as_ushort(__float2half_rn(b)) << 16);
-                *reinterpret_cast<uint32_t*>((which == 1 ? rope.k_pool : rope.v_pool) + dst) = packed;
+                *reinterpret_cast<uint32_t*>((rc.which == 1 ? rope.k_pool : rope.v_pool) + dst) = packed;
             }
         }
     } else if (EPI == SKN_EPI_SWIGLU) {
@@ -702,6 +716,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     };
     issue(0, 0);
 
+    // RMSNorm: y = sum_k W[., k] * (x_k * r * g_k) = r * sum_k W[., k] * (x_k * g_k): x * g is staged and the row
+    // totals are multiplied by r = 1 / sqrt(mean(x^2) + eps) at the end, so the sum of squares needs no
+    // barrier of its own (its eight partials are read after the staging barrier)
     if (NORM) {
         float sq = 0.f;
 #pragma unroll
@@ -710,22 +727,24 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                 const float4 v = st.v[j];
                 sq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
             }
+            st.v[j].x *= nw.v[j].x;
+            st.v[j].y *= nw.v[j].y;
+            st.v[j].z *= nw.v[j].z;
+            st.v[j].w *= nw.v[j].w;
         }
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
-        __syncthreads();
-        const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
-        const float rinv = 1.0f / sqrtf(total / (float)(nb * 256) + eps);
-#pragma unroll
-        for (int j = 0; j < J; j++) {
-            st.v[j].x *= rinv * nw.v[j].x;
-            st.v[j].y *= rinv * nw.v[j].y;
-            st.v[j].z *= rinv * nw.v[j].z;
-            st.v[j].w *= rinv * nw.v[j].w;
-        }
     }
     q4k_stage_store<J>(st, n4, tid, 512, xs, ss);
     __syncthreads();
+    // (after the staging, while the first weights are still on their way)
+    Q4kRopeCtx rc;
+    if (EPI == SKN_EPI_ROPE) rc = q4k_rope_prepare(seg, rope, min(unit, (n_out + 1) / 2 - 1));
+    float rinv = 1.0f;
+    if (NORM) {
+        const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
+        rinv = 1.0f / sqrtf(total / (float)(nb * 256) + eps);
+    }
 
     float acc[R] = {0.f, 0.f};
     int tie = 0;
@@ -737,9 +756,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
-    const float t0 = wave_sum(acc[0]) * 16777216.0f;
-    const float t1 = wave_sum(acc[1]) * 16777216.0f;
-    if (lane == 0) q4k_epilogue<EPI>(seg, rope, y, n_out, unit, t0, t1);
+    const float t0 = wave_sum(acc[0]) * (16777216.0f * rinv);
+    const float t1 = wave_sum(acc[1]) * (16777216.0f * rinv);
+    if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
 }
 
 template <int STEPS, int EPI, bool NORM>
