@@ -5,9 +5,9 @@
 // dequantized weight rounded to one fp16 / bf16 operand (11 / 8 bits) would miss it on outputs near zero.
 // Both paths below therefore feed the MFMA with operands that are exact or exact to 2^-22:
 //
-//   * Activations: bf16 -> fp16 is exact for every value whose magnitude is within fp16 range; a row whose
-//     largest magnitude exceeds 2^14 is scaled down by a power of two first and the scale undone in the
-//     epilogue (prep_a_kernel).  Products and sums are fp32 inside the MFMA.
+//   * Activations: bf16 -> fp16 is exact for every value whose magnitude is within fp16's normal range; each
+//     row is first scaled by a power of two that puts its largest magnitude just below 2^14 (2^10 on the Q4_K
+//     path) and the scale is undone in the epilogue.  Products and sums are fp32 inside the MFMA.
 //   * Weights, general path (Q8_0, Q6_K): W is dequantized once into a workspace as an fp16 pair
 //     hi = f16(w), lo = f16(w - hi) (w_hi + w_lo = w to 2^-22 relative) and each k-step issues two MFMAs.
 //   * Weights, Q4_K path: see gemm_q4k_kernel -- the 4-bit quants times their 6-bit sub-block scale are
@@ -45,11 +45,12 @@ __global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict_
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    // scale = 2^-e with the smallest e >= 0 such that mx * scale <= 2^14
-    int e = 0;
-    if (mx > 16384.f) e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127 - 14 + 1;
-    const float scale = __uint_as_float((uint32_t)(127 - e) << 23);
-    if (threadIdx.x == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 + e) << 23);
+    // the row is scaled by a power of two so that its largest magnitude lies in [2^13, 2^14): large rows fit
+    // fp16 and tiny rows do not vanish in it (a zero row keeps scale 1)
+    int e = 13;
+    if (mx > 0.f) e = max((int)((__float_as_uint(mx) >> 23) & 0xFF) - 127, -100);
+    const float scale = __uint_as_float((uint32_t)(127 + 13 - e) << 23);
+    if (threadIdx.x == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 - 13 + e) << 23);
     _Float16* out = a16 + (size_t)m * k;
     for (int i = threadIdx.x; i < k; i += 256) out[i] = (_Float16)(__uint_as_float((uint32_t)ar[i] << 16) * scale);
 }

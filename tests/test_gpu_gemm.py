@@ -58,6 +58,48 @@ def test_gemm_large_activations_are_rescaled(hip):
         assert oracle_np.rel_err(got[r], want[r]) <= TOL, r
 
 
+@pytest.mark.parametrize("qtype", [Q4_K, Q6_K])
+def test_gemm_extreme_rows(hip, qtype):
+    """Rows the activation rescaling has to survive: all zero, a single non-zero element, the smallest bf16
+    normals, a 2^40 dynamic range inside one row, negative-only and alternating signs."""
+    m, n, k = 8, 96, 2048
+    raw = synth.weight(qtype, n, k, seed=21)
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[0] = 0.0
+    x[1] = 0.0
+    x[1, 1029] = -3.0
+    x[2] *= 1.0e-30
+    x[3] *= np.exp2(rng.integers(-20, 20, size=k)).astype(np.float32)
+    x[4] = -np.abs(x[4])
+    x[5] = np.where(np.arange(k) % 2 == 0, 1.0, -1.0)
+    x[6] *= 6.0e4   # around the fp16 maximum before rescaling
+    x[7, : k // 2] = 0.0
+    a = synth.f32_to_bf16_bits(x)
+    got = hip.gemm_q_host(qtype, raw, n, k, a, m)
+    want = oracle_c.gemm_q(qtype, raw, n, k, a, m)
+    assert np.all(got[0] == 0.0)
+    w = oracle_c.dequant(qtype, raw).reshape(n, k)
+    assert np.allclose(got[1], -3.0 * w[:, 1029], rtol=1e-6, atol=0.0)
+    for r in range(2, m):
+        assert oracle_np.rel_err(got[r], want[r]) <= TOL, r
+
+
+@pytest.mark.parametrize("n", [4096, 14336])
+def test_gemm_benchmark_shapes_q6k(hip, n):
+    """M=512, K=4096 with Q6_K weights (the mixed-precision prefill case), sampled columns."""
+    m, k = 512, 4096
+    raw = synth.weight(Q6_K, n, k, seed=11)
+    a = synth.activation_bf16((m, k), seed=12)
+    got = hip.gemm_q_host(Q6_K, raw, n, k, a, m)
+    rows = np.arange(0, n, 127)
+    rb = raw.reshape(n, -1)[rows].reshape(-1)
+    want = oracle_c.gemm_q(Q6_K, rb, len(rows), k, a, m)
+    floor = 1e-3 * np.abs(got).max()
+    err = np.max(np.abs(got[:, rows] - want) / np.maximum(np.abs(want), floor))
+    assert err <= TOL, err
+
+
 def test_gemm_full_width_slice(hip):
     """The benchmark shape M=512, K=4096 at N=4096: checked on a strided sample of the oracle's columns."""
     m, n, k = 512, 4096, 4096
