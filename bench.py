@@ -159,7 +159,7 @@ def bench_gemm(ctx, qtype, m, n, k, reps=20):
             "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
-def cpu_baseline(qtype, n, k, budget_s=12.0):
+def cpu_baseline(qtype, n, k, budget_s=10.0):
     """The CPU oracle (C, OpenMP over rows) on the headline workload; a bounded number of repetitions."""
     from oracle import oracle_c  # the checker, timed as the "port" CPU baseline -- never the product path
 
@@ -172,7 +172,7 @@ def cpu_baseline(qtype, n, k, budget_s=12.0):
         oracle_c.matvec_q(qtype, raw, n, k, x)
         reps += 1
         dt = time.perf_counter() - t0
-        if dt >= budget_s or reps >= 400:
+        if dt >= budget_s or reps >= 20000:
             break
     per = dt / reps
     # the reference's own algorithm for such a weight (dequantize to fp64, transpose, i-outer loop), one thread
