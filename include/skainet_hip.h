@@ -42,9 +42,16 @@ extern "C" {
 
 #define SKN_TYPE_F32 0
 #define SKN_TYPE_F16 1
+#define SKN_TYPE_Q4_0 2
+#define SKN_TYPE_Q4_1 3
+#define SKN_TYPE_Q5_0 6
+#define SKN_TYPE_Q5_1 7
 #define SKN_TYPE_Q8_0 8
+#define SKN_TYPE_Q2_K 10
 #define SKN_TYPE_Q4_K 12
+#define SKN_TYPE_Q5_K 13
 #define SKN_TYPE_Q6_K 14
+#define SKN_TYPE_BF16 30
 
 typedef struct skn_ctx skn_ctx;
 typedef struct skn_kv skn_kv;
@@ -65,7 +72,8 @@ int skn_device_info(skn_ctx* ctx, char* name, size_t name_len, int* compute_unit
 
 /* ---- format table -------------------------------------------------------------------------------- */
 
-/* GGML_QUANT_SIZES lookup (gguf/.../Constants.kt:58-90): elements and bytes per block. */
+/* GGML_QUANT_SIZES lookup (gguf/.../Constants.kt:58-90): elements and bytes per block, for every type id of
+ * that table (the ids of gguf/.../Constants.kt:14-46).  The kernels compute with the SKN_TYPE_* ids above. */
 int skn_type_block(int ggml_type, int* block_elems, int* block_bytes);
 /* quantShapeToByteShape on the last axis (gguf/.../Quants.kt:10-20): bytes of a row of k elements, or
  * SKN_ERR_SHAPE when k is not a block multiple, SKN_ERR_TYPE for an unknown type. */
@@ -101,14 +109,15 @@ int skn_prof_stop(skn_ctx* ctx, double* kernel_ms_total, int* launches);
 /* ---- dequantization ------------------------------------------------------------------------------ */
 
 /* The dequantizer the reference leaves as a TODO (gguf/.../Quants.kt:8): n_elems consecutive elements
- * (a block multiple) of `ggml_type` at `w_dev` -> fp32 at `out_dev`.  Bit-exact with the ggml formulas. */
+ * (a block multiple) of `ggml_type` at `w_dev` -> fp32 at `out_dev`.  Bit-exact with the ggml formulas.
+ * Types: every SKN_TYPE_* id (F32 / F16 / BF16 are widened or copied). */
 int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64_t n_elems, float* out_dev);
 
 /* ---- quantized matvec / GEMM ---------------------------------------------------------------------- */
 
 /* y[n] = sum_k deq(W)[n,k] * x[k]: Linear.forward's `input.matmul(weight.t())` for a rank-1 input
  * (core/.../nn/Linear.kt:43-49 -> core/.../impl/DoublesTensor.kt:255-264), without materialising t().
- * x fp32 [k], y fp32 [n]. */
+ * x fp32 [k], y fp32 [n].  Any SKN_TYPE_* weight type; Q4_K, Q8_0 and Q6_K have the tuned kernels. */
 int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev, float* y_dev);
 /* C[m,n] = sum_k A[m,k] * deq(W)[n,k]: the rank-2 case (core/.../impl/DoublesTensor.kt:267-279).
  * A bf16 bits [m,k] row-major, C fp32 [m,n] row-major. */

@@ -20,6 +20,10 @@
  *   orc_dequant_* ..................... unpinned by the reference (it has no dequantizer); pinned by hand-built
  *                                       single-block known answers, an independent NumPy restatement
  *                                       (oracle/oracle_np.py) and the fp64 closed form rounded once
+ *   deq_q4_0/q4_1/q5_0/q5_1/q2_k/q5_k . the further formats of the reference's size table: unpinned by the reference
+ *                                       in the same way; pinned by hand-built tagged blocks (element order, fifth-bit
+ *                                       positions, scale indices), the NumPy restatement and exact rational goldens
+ *                                       (tests/golden/quant_blocks_more.npz)
  *   orc_matvec_q / orc_gemm_q ......... pinned by reduction to the dense reference semantics on dequantized weights
  *   orc_attn_decode ................... unpinned by the reference (its softmax is not max-subtracted and is untested);
  *                                       pinned by closed forms (uniform K => mean(V), one token => V0) and scipy softmax
@@ -39,7 +43,8 @@
 #define ORC_ERR_TYPE (-2)
 #define ORC_ERR_SHAPE (-3)
 
-enum { T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14 };
+enum { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8, T_Q2_K = 10, T_Q4_K = 12,
+       T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30 };
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -125,11 +130,18 @@ void orc_f2h_n(const float* f, uint16_t* h, int64_t n) {
 
 /* ------------------------------------------------------ type table / shapes */
 
-/* Constants.kt:58-90 (only the types on this path). */
+/* Constants.kt:58-90 (the types this library computes with). */
 int orc_type_sizes(int type, int* block_elems, int* block_bytes) {
     switch (type) {
         case T_F32: *block_elems = 1; *block_bytes = 4; return ORC_OK;
         case T_F16: *block_elems = 1; *block_bytes = 2; return ORC_OK;
+        case T_BF16: *block_elems = 1; *block_bytes = 2; return ORC_OK;
+        case T_Q4_0: *block_elems = 32; *block_bytes = 2 + 16; return ORC_OK;
+        case T_Q4_1: *block_elems = 32; *block_bytes = 2 + 2 + 16; return ORC_OK;
+        case T_Q5_0: *block_elems = 32; *block_bytes = 2 + 4 + 16; return ORC_OK;
+        case T_Q5_1: *block_elems = 32; *block_bytes = 2 + 2 + 4 + 16; return ORC_OK;
+        case T_Q2_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 16 + 256 / 4; return ORC_OK;
+        case T_Q5_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 256 / 8 + 12; return ORC_OK;
         case T_Q8_0: *block_elems = 32; *block_bytes = 2 + 32; return ORC_OK;
         case T_Q4_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 12; return ORC_OK;
         case T_Q6_K: *block_elems = 256; *block_bytes = 2 + 256 / 2 + 256 / 4 + 256 / 16; return ORC_OK;
@@ -215,16 +227,116 @@ static void deq_q6_k_block(const uint8_t* b, float* y) {
     }
 }
 
+/* ---- the other block formats of the reference's table (Constants.kt:58-90) that this library computes with.
+ * Their packing is the published ggml definition as well (block_q4_0/q4_1/q5_0/q5_1/q2_K/q5_K); like the three
+ * above they are unpinned by the reference.  Each value is an exact real (products of an f16 with small
+ * integers) rounded once, so the fp32 order of operations below is immaterial. */
+
+static float rd_h(const uint8_t* p) {
+    uint16_t h;
+    memcpy(&h, p, 2);
+    return orc_h2f(h);
+}
+
+/* Q4_0: d f16 @0, qs u8[16] @2.  Low nibbles are elements 0..15, high nibbles 16..31; y = d * (q - 8). */
+static void deq_q4_0_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b);
+    for (int j = 0; j < 16; j++) {
+        y[j] = d * (float)((int)(b[2 + j] & 0x0F) - 8);
+        y[j + 16] = d * (float)((int)(b[2 + j] >> 4) - 8);
+    }
+}
+
+/* Q4_1: d f16 @0, m f16 @2, qs u8[16] @4.  y = d * q + m. */
+static void deq_q4_1_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b), m = rd_h(b + 2);
+    for (int j = 0; j < 16; j++) {
+        y[j] = d * (float)(b[4 + j] & 0x0F) + m;
+        y[j + 16] = d * (float)(b[4 + j] >> 4) + m;
+    }
+}
+
+/* Q5_0: d f16 @0, qh u32 @2 (bit j = fifth bit of element j), qs u8[16] @6.  y = d * (q - 16). */
+static void deq_q5_0_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b);
+    uint32_t qh;
+    memcpy(&qh, b + 2, 4);
+    for (int j = 0; j < 16; j++) {
+        const int lo = (b[6 + j] & 0x0F) | (int)(((qh >> j) & 1u) << 4);
+        const int hi = (b[6 + j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+        y[j] = d * (float)(lo - 16);
+        y[j + 16] = d * (float)(hi - 16);
+    }
+}
+
+/* Q5_1: d f16 @0, m f16 @2, qh u32 @4, qs u8[16] @8.  y = d * q + m. */
+static void deq_q5_1_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b), m = rd_h(b + 2);
+    uint32_t qh;
+    memcpy(&qh, b + 4, 4);
+    for (int j = 0; j < 16; j++) {
+        const int lo = (b[8 + j] & 0x0F) | (int)(((qh >> j) & 1u) << 4);
+        const int hi = (b[8 + j] >> 4) | (int)(((qh >> (j + 16)) & 1u) << 4);
+        y[j] = d * (float)lo + m;
+        y[j + 16] = d * (float)hi + m;
+    }
+}
+
+/* Q2_K: scales u8[16] @0 (low nibble scale, high nibble min), qs u8[64] @16, d f16 @80, dmin f16 @82.
+ * Element e: half n = e / 128, bit pair j = (e % 128) / 32, l = e % 32: byte qs[32n + l] >> 2j, scale
+ * 8n + 2j + (l >= 16).  y = (d * sc) * q - dmin * m. */
+static void deq_q2_k_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b + 80), dmin = rd_h(b + 82);
+    for (int e = 0; e < 256; e++) {
+        const int n = e / 128, j = (e % 128) / 32, l = e % 32;
+        const uint8_t s = b[8 * n + 2 * j + (l >= 16)];
+        const int q = (b[16 + 32 * n + l] >> (2 * j)) & 3;
+        y[e] = d * (float)(s & 0x0F) * (float)q - dmin * (float)(s >> 4);
+    }
+}
+
+/* Q5_K: d f16 @0, dmin f16 @2, scales u8[12] @4 (as Q4_K), qh u8[32] @16, qs u8[128] @48.  Element e: chunk
+ * c = e / 64, r = e % 64, sub-block 2c + (r >= 32), nibble of qs[32c + r % 32] (low for r < 32), fifth bit =
+ * bit 2c + (r >= 32) of qh[r % 32].  y = (d * sc) * q - dmin * m. */
+static void deq_q5_k_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b), dmin = rd_h(b + 2);
+    for (int e = 0; e < 256; e++) {
+        const int c = e / 64, r = e % 64, up = r >= 32;
+        int sc, m;
+        q4k_scale_min(2 * c + up, b + 4, &sc, &m);
+        const uint8_t byte = b[48 + 32 * c + (r % 32)];
+        const int q = (up ? byte >> 4 : byte & 0x0F) | (((b[16 + (r % 32)] >> (2 * c + up)) & 1) << 4);
+        y[e] = d * (float)sc * (float)q - dmin * (float)m;
+    }
+}
+
+static int is_block_type(int type) {
+    return type == T_Q8_0 || type == T_Q4_K || type == T_Q6_K || type == T_Q4_0 || type == T_Q4_1 || type == T_Q5_0 ||
+           type == T_Q5_1 || type == T_Q2_K || type == T_Q5_K || type == T_F16 || type == T_BF16 || type == T_F32;
+}
+
 static void deq_block(int type, const uint8_t* b, float* y) {
-    if (type == T_Q8_0) deq_q8_0_block(b, y);
-    else if (type == T_Q4_K) deq_q4_k_block(b, y);
-    else deq_q6_k_block(b, y);
+    uint16_t h;
+    switch (type) {
+        case T_Q8_0: deq_q8_0_block(b, y); break;
+        case T_Q4_K: deq_q4_k_block(b, y); break;
+        case T_Q6_K: deq_q6_k_block(b, y); break;
+        case T_Q4_0: deq_q4_0_block(b, y); break;
+        case T_Q4_1: deq_q4_1_block(b, y); break;
+        case T_Q5_0: deq_q5_0_block(b, y); break;
+        case T_Q5_1: deq_q5_1_block(b, y); break;
+        case T_Q2_K: deq_q2_k_block(b, y); break;
+        case T_Q5_K: deq_q5_k_block(b, y); break;
+        case T_F16: memcpy(&h, b, 2); y[0] = orc_h2f(h); break;
+        case T_BF16: memcpy(&h, b, 2); y[0] = orc_bf2f(h); break;
+        default: memcpy(y, b, 4); break; /* F32 */
+    }
 }
 
 /* n_elems consecutive elements (a block multiple) of `type` -> fp32. */
 int orc_dequant(int type, const uint8_t* w, int64_t n_elems, float* out) {
     int be, bb;
-    if (type != T_Q8_0 && type != T_Q4_K && type != T_Q6_K) return ORC_ERR_TYPE;
+    if (!is_block_type(type)) return ORC_ERR_TYPE;
     orc_type_sizes(type, &be, &bb);
     if (n_elems < 0 || n_elems % be != 0) return ORC_ERR_SHAPE;
     const int64_t nb = n_elems / be;
@@ -259,7 +371,7 @@ void orc_dense_matmul(const double* A, const double* B, int M, int K, int N, dou
 int orc_matvec_q(int type, const uint8_t* w, int N, int K, const float* x, float* y) {
     int64_t rb = orc_row_bytes(type, K);
     if (rb < 0) return (int)rb;
-    if (type != T_Q8_0 && type != T_Q4_K && type != T_Q6_K) return ORC_ERR_TYPE;
+    if (!is_block_type(type)) return ORC_ERR_TYPE;
     int be, bb;
     orc_type_sizes(type, &be, &bb);
     const int nb = K / be;
@@ -307,7 +419,7 @@ int orc_matvec_q_reference_algorithm(int type, const uint8_t* w, int N, int K, c
 int orc_gemm_q(int type, const uint8_t* w, int N, int K, const uint16_t* a_bf16, int M, float* c) {
     int64_t rb = orc_row_bytes(type, K);
     if (rb < 0) return (int)rb;
-    if (type != T_Q8_0 && type != T_Q4_K && type != T_Q6_K) return ORC_ERR_TYPE;
+    if (!is_block_type(type)) return ORC_ERR_TYPE;
     int be, bb;
     orc_type_sizes(type, &be, &bb);
     float* af = (float*)malloc((size_t)M * K * sizeof(float));

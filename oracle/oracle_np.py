@@ -23,17 +23,26 @@ from __future__ import annotations
 import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
-F32, F16 = 0, 1
+F32, F16, BF16 = 0, 1, 30
+Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
 
-# Constants.kt:58-90 restricted to the types on this path: type -> (block elems, block bytes)
+# Constants.kt:58-90 restricted to the types this library computes with: type -> (block elems, block bytes)
 QUANT_SIZES = {
     F32: (1, 4),
     F16: (1, 2),
+    BF16: (1, 2),
+    Q4_0: (32, 2 + 16),
+    Q4_1: (32, 2 + 2 + 16),
+    Q5_0: (32, 2 + 4 + 16),
+    Q5_1: (32, 2 + 2 + 4 + 16),
     Q8_0: (32, 2 + 32),
+    Q2_K: (256, 2 + 2 + 256 // 16 + 256 // 4),
     Q4_K: (256, 2 + 2 + 256 // 2 + 12),
+    Q5_K: (256, 2 + 2 + 256 // 2 + 256 // 8 + 12),
     Q6_K: (256, 2 + 256 // 2 + 256 // 4 + 256 // 16),
 }
-TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", F32: "F32", F16: "F16"}
+TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", F32: "F32", F16: "F16", BF16: "BF16", Q4_0: "Q4_0",
+              Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q2_K: "Q2_K", Q5_K: "Q5_K"}
 
 
 def quant_shape_to_byte_shape(shape, qtype):
@@ -115,7 +124,90 @@ def dequant_q6_k(raw):
     return y.astype(np.float32).reshape(-1)
 
 
-_DEQ = {Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q6_K: dequant_q6_k}
+# ---- the further formats (whole-array forms; unpinned by the reference like the three above) ------------
+
+def _nibbles32(qs16):
+    """[nb,16] bytes -> [nb,32] values: low nibbles are elements 0..15, high nibbles 16..31."""
+    return np.concatenate([qs16 & 0x0F, qs16 >> 4], axis=1).astype(np.int32)
+
+
+def _fifth_bits(qh4):
+    """[nb,4] bytes of a little-endian u32 -> [nb,32] bits, bit j for element j."""
+    qh = qh4.astype(np.uint32)
+    word = qh[:, 0] | (qh[:, 1] << 8) | (qh[:, 2] << 16) | (qh[:, 3] << 24)
+    return ((word[:, None] >> np.arange(32, dtype=np.uint32)[None, :]) & 1).astype(np.int32)
+
+
+def dequant_q4_0(raw):
+    b = _blocks(raw, Q4_0)
+    return (_f16(b[:, 0:2])[:, None] * (_nibbles32(b[:, 2:18]) - 8)).astype(np.float32).reshape(-1)
+
+
+def dequant_q4_1(raw):
+    b = _blocks(raw, Q4_1)
+    y = _f16(b[:, 0:2])[:, None] * _nibbles32(b[:, 4:20]) + _f16(b[:, 2:4])[:, None]
+    return y.astype(np.float32).reshape(-1)
+
+
+def dequant_q5_0(raw):
+    b = _blocks(raw, Q5_0)
+    q = (_nibbles32(b[:, 6:22]) | (_fifth_bits(b[:, 2:6]) << 4)) - 16
+    return (_f16(b[:, 0:2])[:, None] * q).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_1(raw):
+    b = _blocks(raw, Q5_1)
+    q = _nibbles32(b[:, 8:24]) | (_fifth_bits(b[:, 4:8]) << 4)
+    y = _f16(b[:, 0:2])[:, None] * q + _f16(b[:, 2:4])[:, None]
+    return y.astype(np.float32).reshape(-1)
+
+
+def dequant_q2_k(raw):
+    b = _blocks(raw, Q2_K)
+    nb = b.shape[0]
+    s = b[:, 0:16].reshape(nb, 2, 4, 2)              # [half n][bit pair j][first / second 16 of the 32]
+    qs = b[:, 16:80].reshape(nb, 2, 1, 32)           # [half n][.][l]
+    shifts = (2 * np.arange(4, dtype=np.uint8)).reshape(1, 1, 4, 1)
+    q = ((qs >> shifts) & 3).astype(np.float64)      # [nb,2,4,32]
+    sc = np.repeat(s & 0x0F, 16, axis=3).astype(np.float64)   # [nb,2,4,32]
+    mn = np.repeat(s >> 4, 16, axis=3).astype(np.float64)
+    d = _f16(b[:, 80:82])[:, None, None, None]
+    dmin = _f16(b[:, 82:84])[:, None, None, None]
+    return ((d * sc) * q - dmin * mn).astype(np.float32).reshape(-1)
+
+
+def dequant_q5_k(raw):
+    b = _blocks(raw, Q5_K)
+    nb = b.shape[0]
+    d = _f16(b[:, 0:2])
+    dmin = _f16(b[:, 2:4])
+    sc, m = q4k_scales_mins(b[:, 4:16])
+    qh = b[:, 16:48]                                  # [nb,32]
+    qs = b[:, 48:176].reshape(nb, 4, 32)
+    lo = (qs & 0x0F).astype(np.int32)
+    hi = (qs >> 4).astype(np.int32)
+    q = np.stack([lo, hi], axis=2).reshape(nb, 8, 32)  # sub-block j = 2c + upper
+    bit = ((qh[:, None, :] >> np.arange(8, dtype=np.uint8)[None, :, None]) & 1).astype(np.int32)  # [nb,8,32]
+    q = (q | (bit << 4)).astype(np.float64)
+    y = (d[:, None, None] * sc[:, :, None].astype(np.float64)) * q - (dmin[:, None, None] * m[:, :, None].astype(np.float64))
+    return y.astype(np.float32).reshape(-1)
+
+
+def dequant_f16(raw):
+    return np.frombuffer(np.ascontiguousarray(raw), dtype="<f2").astype(np.float32)
+
+
+def dequant_bf16(raw):
+    return bf16_to_f32(np.frombuffer(np.ascontiguousarray(raw), dtype="<u2"))
+
+
+def dequant_f32(raw):
+    return np.frombuffer(np.ascontiguousarray(raw), dtype="<f4").copy()
+
+
+_DEQ = {Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q6_K: dequant_q6_k, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1,
+        Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q2_K: dequant_q2_k, Q5_K: dequant_q5_k, F16: dequant_f16,
+        BF16: dequant_bf16, F32: dequant_f32}
 
 
 def dequant(qtype, raw):

@@ -97,14 +97,44 @@ int skn_device_info(skn_ctx* ctx, char* name, size_t name_len, int* compute_unit
 
 int skn_type_block(int ggml_type, int* block_elems, int* block_bytes) {
     int be, bb;
-    switch (ggml_type) {
-        case SKN_TYPE_F32: be = 1; bb = 4; break;
-        case SKN_TYPE_F16: be = 1; bb = 2; break;
-        case SKN_TYPE_Q8_0: be = 32; bb = 34; break;
-        case SKN_TYPE_Q4_K: be = 256; bb = 144; break;
-        case SKN_TYPE_Q6_K: be = 256; bb = 210; break;
-        default: return skn_fail(nullptr, SKN_ERR_TYPE, "ggml type %d is not supported", ggml_type);
-    }
+    // the whole table of gguf/.../Constants.kt:58-90, keyed by the ids of :14-46
+    static const struct { int id, elems, bytes; } kTable[] = {
+        {0, 1, 4},          // F32
+        {1, 1, 2},          // F16
+        {2, 32, 2 + 16},    // Q4_0
+        {3, 32, 2 + 2 + 16},        // Q4_1
+        {6, 32, 2 + 4 + 16},        // Q5_0
+        {7, 32, 2 + 2 + 4 + 16},    // Q5_1
+        {8, 32, 2 + 32},            // Q8_0
+        {9, 32, 4 + 4 + 32},        // Q8_1
+        {10, 256, 2 + 2 + 256 / 16 + 256 / 4},            // Q2_K
+        {11, 256, 2 + 256 / 4 + 256 / 8 + 12},            // Q3_K
+        {12, 256, 2 + 2 + 256 / 2 + 12},                  // Q4_K
+        {13, 256, 2 + 2 + 256 / 2 + 256 / 8 + 12},        // Q5_K
+        {14, 256, 2 + 256 / 2 + 256 / 4 + 256 / 16},      // Q6_K
+        {15, 256, 4 + 256 + 256 / 8},                     // Q8_K
+        {16, 256, 2 + 256 / 4},                           // IQ2_XXS
+        {17, 256, 2 + 256 / 4 + 256 / 32},                // IQ2_XS
+        {18, 256, 2 + 256 / 4 + 256 / 8},                 // IQ3_XXS
+        {19, 256, 2 + 256 / 8 + 256 / 16},                // IQ1_S
+        {20, 32, 2 + 16},                                 // IQ4_NL
+        {21, 256, 2 + 256 / 4 + 256 / 8 + 256 / 32 + 4},  // IQ3_S
+        {22, 256, 2 + 256 / 4 + 256 / 16},                // IQ2_S
+        {23, 256, 2 + 2 + 256 / 2 + 256 / 64},            // IQ4_XS
+        {24, 1, 1}, {25, 1, 2}, {26, 1, 4}, {27, 1, 8},   // I8, I16, I32, I64
+        {28, 1, 8},                                       // F64
+        {29, 256, 256 / 8 + 256 / 16 + 256 / 32},         // IQ1_M
+        {30, 1, 2},                                       // BF16
+        {34, 256, 2 + 4 * 13},                            // TQ1_0
+        {35, 256, 2 + 64},                                // TQ2_0
+    };
+    be = bb = 0;
+    for (const auto& row : kTable)
+        if (row.id == ggml_type) {
+            be = row.elems;
+            bb = row.bytes;
+        }
+    if (be == 0) return skn_fail(nullptr, SKN_ERR_TYPE, "ggml type %d is not in the size table", ggml_type);
     if (block_elems) *block_elems = be;
     if (block_bytes) *block_bytes = bb;
     return SKN_OK;

@@ -96,7 +96,15 @@ inline void skn_launch(skn_ctx* ctx, F kernel, dim3 grid, dim3 block, size_t lds
     }
 }
 
-static inline bool skn_is_quant(int t) { return t == SKN_TYPE_Q8_0 || t == SKN_TYPE_Q4_K || t == SKN_TYPE_Q6_K; }
+// the three formats with tuned kernels (and the only ones the decoder's embedding lookup reads)
+static inline bool skn_is_core_quant(int t) { return t == SKN_TYPE_Q8_0 || t == SKN_TYPE_Q4_K || t == SKN_TYPE_Q6_K; }
+// every format the library computes with
+static inline bool skn_is_quant(int t) {
+    return skn_is_core_quant(t) || t == SKN_TYPE_Q4_0 || t == SKN_TYPE_Q4_1 || t == SKN_TYPE_Q5_0 || t == SKN_TYPE_Q5_1 ||
+           t == SKN_TYPE_Q2_K || t == SKN_TYPE_Q5_K || t == SKN_TYPE_F32 || t == SKN_TYPE_F16 || t == SKN_TYPE_BF16;
+}
+int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out);
+int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y);
 
 // ---- device helpers --------------------------------------------------------------------------------
 

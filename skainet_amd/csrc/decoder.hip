@@ -409,7 +409,7 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
                 "skn_llama_create: hidden and ffn must be multiples of 256");
     SKN_REQUIRE(ctx, w->layers && w->tok_embd && w->out_norm && w->out_head, SKN_ERR_ARG,
                 "skn_llama_create: missing weights");
-    SKN_REQUIRE(ctx, (skn_is_quant(w->type_embd) || w->type_embd == SKN_TYPE_F32) && skn_is_quant(w->type_head),
+    SKN_REQUIRE(ctx, (skn_is_core_quant(w->type_embd) || w->type_embd == SKN_TYPE_F32) && skn_is_quant(w->type_head),
                 SKN_ERR_TYPE, "skn_llama_create: unsupported embedding / head type");
     for (int l = 0; l < cfg->n_layer; l++) {
         const skn_llama_layer& L = w->layers[l];

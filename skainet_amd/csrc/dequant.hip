@@ -96,8 +96,9 @@ extern "C" int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64
     if (n_elems == 0) return SKN_OK;
     SKN_REQUIRE(ctx, w_dev && out_dev, SKN_ERR_ARG, "skn_dequant: null pointer");
     SKN_REQUIRE(ctx, ((uintptr_t)out_dev & 15) == 0, SKN_ERR_ARG, "skn_dequant: out must be 16-byte aligned");
-    SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : 1)) == 0, SKN_ERR_ARG,
-                "skn_dequant: weight pointer is misaligned for its block type");
+    SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : ggml_type == SKN_TYPE_F32 ? 3 : 1)) == 0,
+                SKN_ERR_ARG, "skn_dequant: weight pointer is misaligned for its block type");
+    if (!skn_is_core_quant(ggml_type)) return skn_dequant_other(ctx, ggml_type, (const uint8_t*)w_dev, n_elems, out_dev);
     int64_t n_quads = n_elems / 4;
     int64_t blocks = (n_quads + 255) / 256;
     SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_dequant: too many elements for one launch");

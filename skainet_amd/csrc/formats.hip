@@ -1,0 +1,260 @@
+// The further ggml formats of the reference's size table (gguf/.../Constants.kt:58-90) that the library
+// computes with: Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K and the dense F32 / F16 / BF16.  One decode function per
+// format -- four consecutive elements of a block at a time, every value the exact real of its formula rounded
+// once (explicitly rounded intrinsics, so no contraction can change a bit) -- serves a dequantization kernel
+// (one thread per four outputs, 16-byte stores) and a batch-1 matvec (one wavefront per row, the lane's four
+// weights against one aligned float4 of x, DPP reduction).  These are plain streaming kernels; the hand-tuned
+// ones are those of Q4_K, Q8_0 and Q6_K.
+#include "common.h"
+
+namespace {
+
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+
+__device__ __forceinline__ uint32_t ld32(const uint8_t* p) { return *reinterpret_cast<const u32_a2*>(p); }
+__device__ __forceinline__ float ldh(const uint8_t* p) { return h2f_bits(*reinterpret_cast<const uint16_t*>(p)); }
+
+template <int T>
+struct Fmt;
+
+// Q4_0, 18 B: f16 d @0, qs[16] @2.  Low nibbles are elements 0..15, high nibbles 16..31; y = d * (q - 8).
+template <>
+struct Fmt<SKN_TYPE_Q4_0> {
+    static constexpr int kElems = 32, kBytes = 18;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b);
+        uint32_t q = ld32(b + 2 + 4 * (g & 3));
+        if (g >= 4) q >>= 4;
+        float4 y;
+        y.x = __fmul_rn(d, (float)((int)(q & 0xF) - 8));
+        y.y = __fmul_rn(d, (float)((int)((q >> 8) & 0xF) - 8));
+        y.z = __fmul_rn(d, (float)((int)((q >> 16) & 0xF) - 8));
+        y.w = __fmul_rn(d, (float)((int)((q >> 24) & 0xF) - 8));
+        return y;
+    }
+};
+
+// Q4_1, 20 B: f16 d @0, f16 m @2, qs[16] @4.  y = d * q + m.
+template <>
+struct Fmt<SKN_TYPE_Q4_1> {
+    static constexpr int kElems = 32, kBytes = 20;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b), m = ldh(b + 2);
+        uint32_t q = ld32(b + 4 + 4 * (g & 3));
+        if (g >= 4) q >>= 4;
+        float4 y;
+        y.x = __fadd_rn(__fmul_rn(d, (float)(q & 0xF)), m);
+        y.y = __fadd_rn(__fmul_rn(d, (float)((q >> 8) & 0xF)), m);
+        y.z = __fadd_rn(__fmul_rn(d, (float)((q >> 16) & 0xF)), m);
+        y.w = __fadd_rn(__fmul_rn(d, (float)((q >> 24) & 0xF)), m);
+        return y;
+    }
+};
+
+// five-bit values of elements 4g .. 4g+3: nibbles of qs[4 (g % 4) ..] (low for g < 4) with bit (element) of qh
+__device__ __forceinline__ void q5_quad(uint32_t qs4, uint32_t qh, int g, int (&v)[4]) {
+    if (g >= 4) qs4 >>= 4;
+    const uint32_t hb = qh >> (4 * g);
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = (int)(((qs4 >> (8 * i)) & 0xF) | (((hb >> i) & 1u) << 4));
+}
+
+// Q5_0, 22 B: f16 d @0, u32 qh @2 (bit j = fifth bit of element j), qs[16] @6.  y = d * (q - 16).
+template <>
+struct Fmt<SKN_TYPE_Q5_0> {
+    static constexpr int kElems = 32, kBytes = 22;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b);
+        int v[4];
+        q5_quad(ld32(b + 6 + 4 * (g & 3)), ld32(b + 2), g, v);
+        return make_float4(__fmul_rn(d, (float)(v[0] - 16)), __fmul_rn(d, (float)(v[1] - 16)),
+                           __fmul_rn(d, (float)(v[2] - 16)), __fmul_rn(d, (float)(v[3] - 16)));
+    }
+};
+
+// Q5_1, 24 B: f16 d @0, f16 m @2, u32 qh @4, qs[16] @8.  y = d * q + m.
+template <>
+struct Fmt<SKN_TYPE_Q5_1> {
+    static constexpr int kElems = 32, kBytes = 24;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b), m = ldh(b + 2);
+        int v[4];
+        q5_quad(ld32(b + 8 + 4 * (g & 3)), ld32(b + 4), g, v);
+        return make_float4(__fadd_rn(__fmul_rn(d, (float)v[0]), m), __fadd_rn(__fmul_rn(d, (float)v[1]), m),
+                           __fadd_rn(__fmul_rn(d, (float)v[2]), m), __fadd_rn(__fmul_rn(d, (float)v[3]), m));
+    }
+};
+
+// Q2_K, 84 B: scales[16] @0 (low nibble scale, high nibble min), qs[64] @16, f16 d @80, f16 dmin @82.
+// Element e: half n = e / 128, bit pair j = (e % 128) / 32, l = e % 32: qs[32n + l] >> 2j, scale 8n + 2j + (l >= 16).
+template <>
+struct Fmt<SKN_TYPE_Q2_K> {
+    static constexpr int kElems = 256, kBytes = 84;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, n = e >> 7, j = (e & 127) >> 5, l = e & 31;
+        const uint32_t s = b[8 * n + 2 * j + (l >> 4)];
+        const float dl = __fmul_rn(ldh(b + 80), (float)(s & 0xF));
+        const float ml = __fmul_rn(ldh(b + 82), (float)(s >> 4));
+        const uint32_t q = ld32(b + 16 + 32 * n + l) >> (2 * j);
+        float4 y;
+        y.x = __fsub_rn(__fmul_rn(dl, (float)(q & 3)), ml);
+        y.y = __fsub_rn(__fmul_rn(dl, (float)((q >> 8) & 3)), ml);
+        y.z = __fsub_rn(__fmul_rn(dl, (float)((q >> 16) & 3)), ml);
+        y.w = __fsub_rn(__fmul_rn(dl, (float)((q >> 24) & 3)), ml);
+        return y;
+    }
+};
+
+// Q5_K, 176 B: f16 d @0, f16 dmin @2, scales[12] @4 (the Q4_K packing), qh[32] @16, qs[128] @48.
+// Element e: chunk c = e / 64, r = e % 64, sub-block 2c + (r >= 32); nibble of qs[32c + r % 32], fifth bit =
+// bit (sub-block) of qh[r % 32].
+template <>
+struct Fmt<SKN_TYPE_Q5_K> {
+    static constexpr int kElems = 256, kBytes = 176;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, c = e >> 6, r = e & 63, up = r >> 5, j = 2 * c + up, l = r & 31;
+        const uint8_t* s = b + 4;
+        int sc, m;
+        if (j < 4) {
+            sc = s[j] & 63;
+            m = s[j + 4] & 63;
+        } else {
+            sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+            m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+        }
+        const float d1 = __fmul_rn(ldh(b), (float)sc), m1 = __fmul_rn(ldh(b + 2), (float)m);
+        uint32_t q = ld32(b + 48 + 32 * c + l);
+        if (up) q >>= 4;
+        const uint32_t hb = ld32(b + 16 + l) >> j;
+        float4 y;
+        y.x = __fsub_rn(__fmul_rn(d1, (float)((q & 0xF) | ((hb & 1) << 4))), m1);
+        y.y = __fsub_rn(__fmul_rn(d1, (float)(((q >> 8) & 0xF) | (((hb >> 8) & 1) << 4))), m1);
+        y.z = __fsub_rn(__fmul_rn(d1, (float)(((q >> 16) & 0xF) | (((hb >> 16) & 1) << 4))), m1);
+        y.w = __fsub_rn(__fmul_rn(d1, (float)(((q >> 24) & 0xF) | (((hb >> 24) & 1) << 4))), m1);
+        return y;
+    }
+};
+
+// Dense rows, read a scalar at a time where a caller needs it and four at a time otherwise.
+template <int T>
+__device__ __forceinline__ float dense_at(const uint8_t* w, int64_t i) {
+    if (T == SKN_TYPE_F32) return reinterpret_cast<const float*>(w)[i];
+    const uint32_t bits = reinterpret_cast<const uint16_t*>(w)[i];
+    return T == SKN_TYPE_F16 ? h2f_bits(bits) : __uint_as_float(bits << 16);
+}
+
+template <int T>
+__global__ __launch_bounds__(256) void dequant_blocks_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                             int64_t n_quads) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_quads) return;
+    constexpr int QB = Fmt<T>::kElems / 4;  // quads per block
+    reinterpret_cast<float4*>(out)[t] = Fmt<T>::decode4(w + (t / QB) * Fmt<T>::kBytes, (int)(t % QB));
+}
+
+template <int T>
+__global__ __launch_bounds__(256) void convert_dense_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
+                                                            int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = dense_at<T>(w, i);
+}
+
+// one wavefront per row, four rows per workgroup; lane l takes quads l, l + 64, ...
+template <int T>
+__global__ __launch_bounds__(256) void matvec_blocks_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                            float* __restrict__ y, int n_rows, int k) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    constexpr int QB = Fmt<T>::kElems / 4;
+    const uint8_t* rowp = w + (size_t)row * (k / Fmt<T>::kElems) * Fmt<T>::kBytes;
+    float acc = 0.f;
+    for (int q = lane; q < (k >> 2); q += 64) {
+        const float4 wv = Fmt<T>::decode4(rowp + (size_t)(q / QB) * Fmt<T>::kBytes, q % QB);
+        const float4 xv = reinterpret_cast<const float4*>(x)[q];
+        acc = fmaf(wv.x, xv.x, acc);
+        acc = fmaf(wv.y, xv.y, acc);
+        acc = fmaf(wv.z, xv.z, acc);
+        acc = fmaf(wv.w, xv.w, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) y[row] = acc;
+}
+
+template <int T>
+__global__ __launch_bounds__(256) void matvec_dense_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                           float* __restrict__ y, int n_rows, int k) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const uint8_t* rowp = w + (size_t)row * k * (T == SKN_TYPE_F32 ? 4 : 2);
+    float acc = 0.f;
+    for (int i = lane; i < k; i += 64) acc = fmaf(dense_at<T>(rowp, i), x[i], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) y[row] = acc;
+}
+
+template <int T>
+int launch_dequant(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, float* out) {
+    const int64_t n_quads = n_elems / 4, blocks = (n_quads + 255) / 256;
+    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_dequant: too many elements for one launch");
+    skn_launch(ctx, dequant_blocks_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, out, n_quads);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int T>
+int launch_convert(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, float* out) {
+    const int64_t blocks = (n_elems + 255) / 256;
+    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_dequant: too many elements for one launch");
+    skn_launch(ctx, convert_dense_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, out, n_elems);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int T>
+int launch_matvec(skn_ctx* ctx, const uint8_t* w, int n, int k, const float* x, float* y) {
+    skn_launch(ctx, matvec_blocks_kernel<T>, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, w, x, y, n, k);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int T>
+int launch_matvec_dense(skn_ctx* ctx, const uint8_t* w, int n, int k, const float* x, float* y) {
+    skn_launch(ctx, matvec_dense_kernel<T>, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, w, x, y, n, k);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+}  // namespace
+
+// Called by skn_dequant / skn_matvec_q after their argument checks, for the types they do not handle themselves.
+int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out) {
+    switch (ggml_type) {
+        case SKN_TYPE_Q4_0: return launch_dequant<SKN_TYPE_Q4_0>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q4_1: return launch_dequant<SKN_TYPE_Q4_1>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q5_0: return launch_dequant<SKN_TYPE_Q5_0>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q5_1: return launch_dequant<SKN_TYPE_Q5_1>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q2_K: return launch_dequant<SKN_TYPE_Q2_K>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q5_K: return launch_dequant<SKN_TYPE_Q5_K>(ctx, w, n_elems, out);
+        case SKN_TYPE_F32: return launch_convert<SKN_TYPE_F32>(ctx, w, n_elems, out);
+        case SKN_TYPE_F16: return launch_convert<SKN_TYPE_F16>(ctx, w, n_elems, out);
+        case SKN_TYPE_BF16: return launch_convert<SKN_TYPE_BF16>(ctx, w, n_elems, out);
+        default: return skn_fail(ctx, SKN_ERR_TYPE, "skn_dequant: ggml type %d is not supported", ggml_type);
+    }
+}
+
+int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y) {
+    switch (ggml_type) {
+        case SKN_TYPE_Q4_0: return launch_matvec<SKN_TYPE_Q4_0>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q4_1: return launch_matvec<SKN_TYPE_Q4_1>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q5_0: return launch_matvec<SKN_TYPE_Q5_0>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q5_1: return launch_matvec<SKN_TYPE_Q5_1>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q2_K: return launch_matvec<SKN_TYPE_Q2_K>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q5_K: return launch_matvec<SKN_TYPE_Q5_K>(ctx, w, n, k, x, y);
+        case SKN_TYPE_F32: return launch_matvec_dense<SKN_TYPE_F32>(ctx, w, n, k, x, y);
+        case SKN_TYPE_F16: return launch_matvec_dense<SKN_TYPE_F16>(ctx, w, n, k, x, y);
+        case SKN_TYPE_BF16: return launch_matvec_dense<SKN_TYPE_BF16>(ctx, w, n, k, x, y);
+        default: return skn_fail(ctx, SKN_ERR_TYPE, "skn_matvec_q: ggml type %d is not supported", ggml_type);
+    }
+}

@@ -934,9 +934,10 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     if (k == 0) return skn_memset(ctx, y_dev, 0, (size_t)n * sizeof(float));
     SKN_REQUIRE(ctx, w_dev && x_dev, SKN_ERR_ARG, "skn_matvec_q: null pointer");
     SKN_REQUIRE(ctx, ((uintptr_t)x_dev & 15) == 0, SKN_ERR_ARG, "skn_matvec_q: x must be 16-byte aligned");
-    SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : 1)) == 0, SKN_ERR_ARG,
-                "skn_matvec_q: weight pointer is misaligned for its block type");
+    SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : ggml_type == SKN_TYPE_F32 ? 3 : 1)) == 0,
+                SKN_ERR_ARG, "skn_matvec_q: weight pointer is misaligned for its block type");
     const uint8_t* w = (const uint8_t*)w_dev;
+    if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     const int nb = k / be;
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;

@@ -16,7 +16,10 @@ from __future__ import annotations
 import numpy as np
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
-BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210)}
+F32, F16, BF16 = 0, 1, 30
+Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
+BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22),
+         Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176), F32: (1, 4), F16: (1, 2), BF16: (1, 2)}
 
 
 def _f16_bytes(values):
@@ -62,7 +65,34 @@ def q6_k_blocks(n_blocks, rng):
     return b.reshape(-1)
 
 
-_GEN = {Q8_0: q8_0_blocks, Q4_K: q4_k_blocks, Q6_K: q6_k_blocks}
+def _scaled_blocks(n_blocks, rng, nbytes, f16_at, scale=0.01):
+    """Uniform random payload bytes with |N(0,1)| * scale fp16 fields at the given byte offsets."""
+    b = rng.integers(0, 256, size=(n_blocks, nbytes), dtype=np.uint8)
+    for off in f16_at:
+        b[:, off:off + 2] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * scale)
+    return b.reshape(-1)
+
+
+def q5_k_blocks(n_blocks, rng):
+    b = rng.integers(0, 256, size=(n_blocks, 176), dtype=np.uint8)
+    b[:, 0:2] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.01)
+    b[:, 2:4] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.005)
+    b[:, 4:16] = pack_q4k_scales(rng.integers(0, 64, size=(n_blocks, 8), dtype=np.uint8),
+                                 rng.integers(0, 64, size=(n_blocks, 8), dtype=np.uint8))
+    return b.reshape(-1)
+
+
+_GEN = {
+    Q8_0: q8_0_blocks, Q4_K: q4_k_blocks, Q6_K: q6_k_blocks, Q5_K: q5_k_blocks,
+    Q4_0: lambda n, rng: _scaled_blocks(n, rng, 18, (0,)),
+    Q4_1: lambda n, rng: _scaled_blocks(n, rng, 20, (0, 2)),
+    Q5_0: lambda n, rng: _scaled_blocks(n, rng, 22, (0,)),
+    Q5_1: lambda n, rng: _scaled_blocks(n, rng, 24, (0, 2)),
+    Q2_K: lambda n, rng: _scaled_blocks(n, rng, 84, (80, 82)),
+    F32: lambda n, rng: rng.standard_normal(n, dtype=np.float32).view(np.uint8),
+    F16: lambda n, rng: rng.standard_normal(n, dtype=np.float32).astype(np.float16).view(np.uint8),
+    BF16: lambda n, rng: f32_to_bf16_bits(rng.standard_normal(n, dtype=np.float32)).view(np.uint8),
+}
 
 
 def weight(qtype, n_rows, k, seed):

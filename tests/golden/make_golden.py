@@ -181,7 +181,93 @@ def exact_q6_k(b):
     return out
 
 
+def _exact_affine(d, q, m, d_neg, m_bits=None):
+    """d * q + m (m = None: no offset) as an exactly rounded float32 with IEEE zero signs."""
+    v = d * q + (m if m is not None else 0)
+    if v != 0:
+        return _round_f32(v)
+    prod_negzero = (d * q == 0) and (d_neg ^ (q < 0))
+    if m is None:
+        return _zero(prod_negzero)
+    # x + y with an exact zero sum is +0 unless both are -0 (or x = -y != 0: +0)
+    m_negzero = (m == 0) and _neg(*m_bits)
+    return _zero(prod_negzero and m_negzero) if (d * q == 0 and m == 0) else _zero(False)
+
+
+def _nibbles32(qs16):
+    return [int(v) & 15 for v in qs16] + [int(v) >> 4 for v in qs16]
+
+
+def exact_q4_0(b):
+    d = _f16_exact(b[0], b[1])
+    return [_exact_affine(d, q - 8, None, _neg(b[0], b[1])) for q in _nibbles32(b[2:18])]
+
+
+def exact_q4_1(b):
+    d, m = _f16_exact(b[0], b[1]), _f16_exact(b[2], b[3])
+    return [_exact_affine(d, q, m, _neg(b[0], b[1]), (b[2], b[3])) for q in _nibbles32(b[4:20])]
+
+
+def _qh_bits(b4):
+    word = int(b4[0]) | (int(b4[1]) << 8) | (int(b4[2]) << 16) | (int(b4[3]) << 24)
+    return [(word >> j) & 1 for j in range(32)]
+
+
+def exact_q5_0(b):
+    d = _f16_exact(b[0], b[1])
+    q5 = [n | (h << 4) for n, h in zip(_nibbles32(b[6:22]), _qh_bits(b[2:6]))]
+    return [_exact_affine(d, q - 16, None, _neg(b[0], b[1])) for q in q5]
+
+
+def exact_q5_1(b):
+    d, m = _f16_exact(b[0], b[1]), _f16_exact(b[2], b[3])
+    q5 = [n | (h << 4) for n, h in zip(_nibbles32(b[8:24]), _qh_bits(b[4:8]))]
+    return [_exact_affine(d, q, m, _neg(b[0], b[1]), (b[2], b[3])) for q in q5]
+
+
+def _exact_scaled_minus(d, sc, q, dmin, m, d_bits, dmin_bits):
+    v = d * sc * q - dmin * m
+    if v != 0:
+        return _round_f32(v)
+    t1_negzero = (d * sc * q == 0) and _neg(*d_bits)
+    t2_poszero = (dmin * m == 0) and not _neg(*dmin_bits)
+    return _zero(t1_negzero and t2_poszero)
+
+
+def exact_q2_k(b):
+    d, dmin = _f16_exact(b[80], b[81]), _f16_exact(b[82], b[83])
+    out = []
+    for e in range(256):
+        n, rem = divmod(e, 128)
+        j, l = divmod(rem, 32)
+        s = int(b[8 * n + 2 * j + (1 if l >= 16 else 0)])
+        q = (int(b[16 + 32 * n + l]) >> (2 * j)) & 3
+        out.append(_exact_scaled_minus(d, s & 15, q, dmin, s >> 4, (b[80], b[81]), (b[82], b[83])))
+    return out
+
+
+def exact_q5_k(b):
+    d, dmin = _f16_exact(b[0], b[1]), _f16_exact(b[2], b[3])
+    s = [int(v) for v in b[4:16]]
+    out = []
+    for e in range(256):
+        j = e // 32
+        if j < 4:
+            sc, m = s[j] & 63, s[j + 4] & 63
+        else:
+            sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4)
+            m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+        byte = int(b[48 + 32 * (e // 64) + e % 32])
+        q = ((byte >> 4) if (e % 64) >= 32 else (byte & 15)) | (((int(b[16 + e % 32]) >> j) & 1) << 4)
+        out.append(_exact_scaled_minus(d, sc, q, dmin, m, (b[0], b[1]), (b[2], b[3])))
+    return out
+
+
 EXACT = {synth.Q8_0: exact_q8_0, synth.Q4_K: exact_q4_k, synth.Q6_K: exact_q6_k}
+EXACT_MORE = {synth.Q4_0: exact_q4_0, synth.Q4_1: exact_q4_1, synth.Q5_0: exact_q5_0, synth.Q5_1: exact_q5_1,
+              synth.Q2_K: exact_q2_k, synth.Q5_K: exact_q5_k}
+F16_FIELDS = {synth.Q4_0: (0,), synth.Q4_1: (0, 2), synth.Q5_0: (0,), synth.Q5_1: (0, 2), synth.Q2_K: (80, 82),
+              synth.Q5_K: (0, 2)}
 
 
 def adversarial_blocks(qtype, rng):
@@ -230,6 +316,37 @@ def make_quant_blocks():
     return {k: v.shape for k, v in out.items()}
 
 
+def make_more_quant_blocks():
+    """The further formats: seeded blocks plus blocks with extreme fp16 fields and uniform fill bytes, evaluated
+    exactly (rational arithmetic, rounded once); kept in their own fixture file."""
+    out = {}
+    rng = np.random.default_rng(20240611)
+    names = {synth.Q4_0: "q4_0", synth.Q4_1: "q4_1", synth.Q5_0: "q5_0", synth.Q5_1: "q5_1", synth.Q2_K: "q2_k",
+             synth.Q5_K: "q5_k"}
+    f16b = lambda bits: [bits & 0xFF, bits >> 8]  # noqa: E731
+    extremes = [f16b(0x0001), f16b(0x03FF), f16b(0x0400), f16b(0x7BFF), f16b(0xBC01), f16b(0x3C00), f16b(0x0000),
+                f16b(0x8000)]
+    for qtype, name in names.items():
+        be, bb = synth.BLOCK[qtype]
+        blocks = [synth.weight(qtype, 12 if be == 32 else 4, be, seed=2000 + qtype).reshape(-1, bb)]
+        for i, ext in enumerate(extremes):
+            b = rng.integers(0, 256, size=bb, dtype=np.uint8)
+            for n, off in enumerate(F16_FIELDS[qtype]):
+                b[off:off + 2] = extremes[(i + 3 * n) % len(extremes)]
+            blocks.append(b[None, :])
+        for fill in (0x00, 0xFF, 0x0F, 0xF0, 0x55, 0xAA):
+            b = np.full(bb, fill, dtype=np.uint8)
+            for n, off in enumerate(F16_FIELDS[qtype]):
+                b[off:off + 2] = np.array([0.25 / (n + 1)], dtype=np.float16).view(np.uint8)
+            blocks.append(b[None, :])
+        blocks = np.concatenate(blocks)
+        vals = np.array([EXACT_MORE[qtype](blk) for blk in blocks], dtype=np.float32).reshape(-1)
+        out[f"{name}_raw"] = blocks.reshape(-1)
+        out[f"{name}_f32_bits"] = vals.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "quant_blocks_more.npz"), **out)
+    return {k: v.shape for k, v in out.items()}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reference", default="/root/reference")
@@ -246,6 +363,7 @@ def main():
     else:
         print("reference checkout absent: keeping the committed reference-held fixtures")
     print("quant_blocks.npz:", make_quant_blocks())
+    print("quant_blocks_more.npz:", make_more_quant_blocks())
 
 
 if __name__ == "__main__":

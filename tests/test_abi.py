@@ -46,9 +46,24 @@ def test_format_table_matches_reference_constants():
         runtime.row_bytes(runtime.Q4_K, 4100)
     assert e.value.code == runtime.ERR_SHAPE
     assert "row size (4100) is not a multiple of block size (256)" in e.value.message
-    with pytest.raises(runtime.SknError) as e:
-        runtime.type_block(2)  # Q4_0: in the reference's table, not on this path
-    assert e.value.code == runtime.ERR_TYPE
+    # every row of the reference's table: id -> (elements, bytes), Constants.kt:14-46 and :58-90
+    qk = 256
+    table = {
+        0: (1, 4), 1: (1, 2), 2: (32, 2 + 16), 3: (32, 2 + 2 + 16), 6: (32, 2 + 4 + 16), 7: (32, 2 + 2 + 4 + 16),
+        8: (32, 2 + 32), 9: (32, 4 + 4 + 32), 10: (256, 2 + 2 + qk // 16 + qk // 4), 11: (256, 2 + qk // 4 + qk // 8 + 12),
+        12: (256, 2 + 2 + qk // 2 + 12), 13: (256, 2 + 2 + qk // 2 + qk // 8 + 12),
+        14: (256, 2 + qk // 2 + qk // 4 + qk // 16), 15: (256, 4 + qk + qk // 8), 16: (256, 2 + qk // 4),
+        17: (256, 2 + qk // 4 + qk // 32), 18: (256, 2 + qk // 4 + qk // 8), 19: (256, 2 + qk // 8 + qk // 16),
+        20: (32, 2 + 16), 21: (256, 2 + qk // 4 + qk // 8 + qk // 32 + 4), 22: (256, 2 + qk // 4 + qk // 16),
+        23: (256, 2 + 2 + qk // 2 + qk // 64), 24: (1, 1), 25: (1, 2), 26: (1, 4), 27: (1, 8), 28: (1, 8),
+        29: (256, qk // 8 + qk // 16 + qk // 32), 30: (1, 2), 34: (256, 2 + 4 * 13), 35: (256, 2 + 64),
+    }
+    for type_id, sizes in table.items():
+        assert runtime.type_block(type_id) == sizes, type_id
+    for type_id in (4, 5, 31, 32, 33, 36, -1):  # ids the reference's enum does not have
+        with pytest.raises(runtime.SknError) as e:
+            runtime.type_block(type_id)
+        assert e.value.code == runtime.ERR_TYPE
 
 
 def test_status_strings_and_version():

@@ -1,0 +1,87 @@
+"""GPU parity for the further ggml formats (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K, F16, BF16, F32) through the C ABI:
+dequantization bit for bit against the CPU oracle, matvec and GEMM within the 1e-3 criterion."""
+import numpy as np
+import pytest
+
+from oracle import oracle_c, oracle_np
+from skainet_amd import runtime, synth
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+MORE = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (1, "f16"), (30, "bf16"), (0, "f32")]
+
+
+@pytest.mark.parametrize("qtype,name", MORE)
+def test_dequant_bit_exact(hip, qtype, name):
+    be, bb = synth.BLOCK[qtype]
+    n, k = 37, 1536 if be > 1 else 1001
+    raw = synth.weight(qtype, n, k, seed=qtype + 50)
+    want = oracle_c.dequant(qtype, raw)
+    out = hip.alloc(4 * n * k)
+    hip.dequant(qtype, hip.to_device(raw), n * k, out)
+    got = out.download(np.float32, n * k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("qtype,name", [t for t in MORE if t[0] not in (0, 1, 30)])
+def test_dequant_random_bytes_bit_exact(hip, qtype, name):
+    """Uniform random payload bytes (all scale / min / bit patterns), finite fp16 fields."""
+    be, bb = synth.BLOCK[qtype]
+    raw = np.random.default_rng(qtype).integers(0, 256, size=4096 * bb, dtype=np.uint8)
+    for off in {2: (0,), 3: (0, 2), 6: (0,), 7: (0, 2), 10: (80, 82), 13: (0, 2)}[qtype]:
+        raw.reshape(-1, bb)[:, off + 1] &= 0x7B
+    want = oracle_c.dequant(qtype, raw)
+    out = hip.alloc(4 * want.size)
+    hip.dequant(qtype, hip.to_device(raw), want.size, out)
+    got = out.download(np.float32, want.size)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("qtype,name", [t for t in MORE if t[0] not in (0, 1, 30)])
+def test_dequant_golden_blocks(hip, golden_dir, qtype, name):
+    import os
+    g = np.load(os.path.join(golden_dir, "quant_blocks_more.npz"))
+    raw, want = g[f"{name}_raw"], g[f"{name}_f32_bits"]
+    out = hip.alloc(4 * want.size)
+    hip.dequant(qtype, hip.to_device(raw), want.size, out)
+    assert np.array_equal(out.download(np.float32, want.size).view(np.uint32), want)
+
+
+@pytest.mark.parametrize("qtype,name", MORE)
+@pytest.mark.parametrize("n,k", [(64, 4096), (5, 768), (1, 256)])
+def test_matvec_vs_oracle(hip, qtype, name, n, k):
+    raw = synth.weight(qtype, n, k, seed=n + k + qtype)
+    x = synth.activation_f32(k, seed=k)
+    got = hip.matvec_q_host(qtype, raw, n, k, x)
+    want = oracle_c.matvec_q(qtype, raw, n, k, x)
+    assert oracle_np.rel_err(got, want) <= TOL
+
+
+def test_dense_matvec_odd_row_length(hip):
+    for qtype in (0, 1, 30):
+        n, k = 9, 333  # no block structure: any row length
+        raw = synth.weight(qtype, n, k, seed=5)
+        x = synth.activation_f32(k, seed=6)
+        got = hip.matvec_q_host(qtype, raw, n, k, x)
+        assert oracle_np.rel_err(got, oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
+
+
+@pytest.mark.parametrize("qtype,name", MORE)
+def test_gemm_vs_oracle(hip, qtype, name):
+    m, n, k = 48, 96, 1024
+    raw = synth.weight(qtype, n, k, seed=qtype + 7)
+    a = synth.activation_bf16((m, k), seed=8)
+    got = hip.gemm_q_host(qtype, raw, n, k, a, m)
+    want = oracle_c.gemm_q(qtype, raw, n, k, a, m)
+    assert oracle_np.rel_err(got, want) <= TOL
+
+
+def test_unknown_types_are_rejected(hip):
+    buf = hip.alloc(4096)
+    for qtype in (9, 11, 15, 16, 4):  # in the size table but not computed with / not in the table at all
+        with pytest.raises(runtime.SknError) as e:
+            hip.matvec_q(qtype, buf, 1, 256, buf, buf)
+        assert e.value.code == runtime.ERR_TYPE
+        with pytest.raises(runtime.SknError) as e:
+            hip.dequant(qtype, buf, 256, buf)
+        assert e.value.code == runtime.ERR_TYPE
