@@ -254,6 +254,12 @@ def main():
             extra[name] = {key: (round(r[key], 3) if isinstance(r[key], float) else r[key])
                            for key in ("kernel_us", "kernel_gbs", "hot_kernel_us", "hot_kernel_gbs", "wall_gbs")}
             extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
+        # the further formats (plain streaming kernels): 4096 x 4096 matvec, kernel GB/s
+        other = {}
+        for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q5_k", 13), ("f16", 1)):
+            r = bench_matvec(ctx, qt, 4096, 4096, 200, 20, copies=24, seed=7000 + qt)
+            other[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
+        extra["other_formats_4096x4096"] = other
         att = bench_attention(ctx, min(args.steps, 200), 10)
         extra["attention_8x32x128_ctx4096"] = {key: round(val, 4) for key, val in att.items()}
         extra["prefill_gemm"] = {f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
