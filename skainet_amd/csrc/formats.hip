@@ -189,7 +189,26 @@ __global__ __launch_bounds__(256) void matvec_dense_kernel(const uint8_t* __rest
     if (row >= n_rows) return;
     const uint8_t* rowp = w + (size_t)row * k * (T == SKN_TYPE_F32 ? 4 : 2);
     float acc = 0.f;
-    for (int i = lane; i < k; i += 64) acc = fmaf(dense_at<T>(rowp, i), x[i], acc);
+    int done = 0;
+    if (T != SKN_TYPE_F32 && (k & 7) == 0 && ((uintptr_t)w & 15) == 0) {
+        // eight 16-bit weights per 128-bit load (rows are 16-byte aligned when k is a multiple of 8)
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        for (int o = lane; o < (k >> 3); o += 64) {
+            const u32x4 v = reinterpret_cast<const u32x4*>(rowp)[o];
+            const float4 x0 = reinterpret_cast<const float4*>(x)[2 * o], x1 = reinterpret_cast<const float4*>(x)[2 * o + 1];
+            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+            const float xs8[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float lo = T == SKN_TYPE_F16 ? h2f_bits(d[i] & 0xFFFF) : __uint_as_float(d[i] << 16);
+                const float hi = T == SKN_TYPE_F16 ? h2f_bits(d[i] >> 16) : __uint_as_float(d[i] & 0xFFFF0000u);
+                acc = fmaf(lo, xs8[2 * i], acc);
+                acc = fmaf(hi, xs8[2 * i + 1], acc);
+            }
+        }
+        done = k;
+    }
+    for (int i = done + lane; i < k; i += 64) acc = fmaf(dense_at<T>(rowp, i), x[i], acc);
     acc = wave_sum(acc);
     if (lane == 0) y[row] = acc;
 }
