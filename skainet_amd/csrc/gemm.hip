@@ -289,13 +289,22 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
         s.h = *reinterpret_cast<const u32x4*>(gw + (size_t)sbk * 144);
         s.q = *reinterpret_cast<const u32x2*>(gw + (size_t)sbk * 144 + 16 + 32 * cc + 8 * bq);
     };
-    auto stash = [&](int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
+    // The staging of one iteration, in four parts (two activation stores each; the unpacking of one nibble
+    // dword each for parts 2 and 3) so that the main loop can place one part behind each pair of matrix
+    // instructions: a wavefront issues in order, and the unpacking only overlaps the matrix pipe that way.
+    auto stash_part = [&](int part, int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
         _Float16* da = sa[cc & 1];
         _Float16* db = sb[cc & 1];
-        *reinterpret_cast<u32x4*>(da + srow * kRow + sch) = s.a0;
-        *reinterpret_cast<u32x4*>(da + (srow + 32) * kRow + sch) = s.a1;
-        *reinterpret_cast<u32x4*>(da + (srow + 64) * kRow + sch) = s.a2;
-        *reinterpret_cast<u32x4*>(da + (srow + 96) * kRow + sch) = s.a3;
+        if (part == 0) {
+            *reinterpret_cast<u32x4*>(da + srow * kRow + sch) = s.a0;
+            *reinterpret_cast<u32x4*>(da + (srow + 32) * kRow + sch) = s.a1;
+            return;
+        }
+        if (part == 1) {
+            *reinterpret_cast<u32x4*>(da + (srow + 64) * kRow + sch) = s.a2;
+            *reinterpret_cast<u32x4*>(da + (srow + 96) * kRow + sch) = s.a3;
+            return;
+        }
         // the whole loaded tuple counts as used here: a word that this chunk does not need (d | dmin outside
         // chunk 0) would otherwise be recycled as a temporary while its load is in flight, and writing it
         // would wait for that load
@@ -311,28 +320,29 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
         const _Float16 ml = (_Float16)(float)scale_of(2 * cc);
         const _Float16 mh = (_Float16)((float)scale_of(2 * cc + 1) * 0.0625f);
         const half2_t mul_lo = {ml, ml}, mul_hi = {mh, mh};
-        const uint32_t q2[2] = {s.q.x, s.q.y};
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const uint32_t q = q2[j], q8 = q >> 8;
-            const uint32_t l02 = q & 0x000F000Fu, h02 = q & 0x00F000F0u;
-            const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
-            u32x4 o;
-            o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo);
-            o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi);
-            o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo);
-            o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi);
-            *reinterpret_cast<u32x4*>(db + brow * kRow + 16 * bq + 8 * j) = o;
-        }
-        if (cc == 0 && bq == 0) {  // per superblock: the column's d * 2^24, dmin and the eight m_j
+        const int j = part - 2;
+        const uint32_t q = j == 0 ? s.q.x : s.q.y, q8 = q >> 8;
+        const uint32_t l02 = q & 0x000F000Fu, h02 = q & 0x00F000F0u;
+        const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
+        u32x4 o;
+        o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo);
+        o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi);
+        o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo);
+        o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi);
+        *reinterpret_cast<u32x4*>(db + brow * kRow + 16 * bq + 8 * j) = o;
+        if (part == 3 && cc == 0 && bq == 0) {  // per superblock: the column's d * 2^24, dmin and the eight m_j
             const half2_t dd = __builtin_bit_cast(half2_t, hw[0]);
             sd[sbk & 1][brow] = (float)dd.x * 16777216.0f;
             sdm[sbk & 1][brow] = (float)dd.y;
             half8_t mm;
 #pragma unroll
-            for (int j = 0; j < 8; j++) mm[j] = (_Float16)(float)min_of(j);
+            for (int jj = 0; jj < 8; jj++) mm[jj] = (_Float16)(float)min_of(jj);
             *reinterpret_cast<half8_t*>(smin[sbk & 1] + brow * 8) = mm;
         }
+    };
+    auto stash = [&](int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int part = 0; part < 4; part++) stash_part(part, sbk, cc, s);
     };
 
     float16_t tot0, tot1, par0, par1;
@@ -345,11 +355,12 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
     const size_t soff0 = (size_t)srow0 * nsub + 4 * (lane >> 5), soff1 = (size_t)srow1 * nsub + 4 * (lane >> 5);
     const int pfrag = (lane & 31) * kRow + (lane >> 5) * 8;
 
-    // (issue order pinned: oldest stage first, as in the loop, so that the wait for a stage never covers a
-    // younger one)
+    // Software pipeline: while the matrix instructions of iteration it run, the wavefront unpacks and stores
+    // iteration it+1 into the other LDS buffer; its global data was requested two iterations earlier.
     fetch(0, 0, st[0]);
     fetch(0, 1, st[1]);
     fetch(0, 2, st[2]);
+    stash(0, 0, st[0]);
     for (int sbk = 0; sbk < nb; sbk++) {
         half4_t sh0, sl0, sh1, sl1;
 #pragma unroll
@@ -363,20 +374,26 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
                 sh1 = *reinterpret_cast<const half4_t*>(sum_hi + soff1 + 8 * sbk);
                 sl1 = *reinterpret_cast<const half4_t*>(sum_lo + soff1 + 8 * sbk);
             }
-            {
-                stash(sbk, cc, st[cc]);
-                __syncthreads();  // buffer cc & 1 is complete; the other one is free once every wavefront is here
-                const _Float16* pa0 = sa[cc & 1] + wm * 64 * kRow + pfrag;
-                const _Float16* pa1 = pa0 + 32 * kRow;
-                const _Float16* pb = sb[cc & 1] + wn * 32 * kRow + pfrag;
+            __syncthreads();  // buffer cc & 1 is complete, and nobody reads the other one any more
+            const _Float16* pa0 = sa[cc & 1] + wm * 64 * kRow + pfrag;
+            const _Float16* pa1 = pa0 + 32 * kRow;
+            const _Float16* pb = sb[cc & 1] + wn * 32 * kRow + pfrag;
+            half8_t fa0[4], fa1[4], fb[4];
 #pragma unroll
-                for (int t = 0; t < kKC / 16; t++) {
-                    const half8_t fa0 = *reinterpret_cast<const half8_t*>(pa0 + 16 * t);
-                    const half8_t fa1 = *reinterpret_cast<const half8_t*>(pa1 + 16 * t);
-                    const half8_t fb = *reinterpret_cast<const half8_t*>(pb + 16 * t);
-                    par0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0, fb, par0, 0, 0, 0);
-                    par1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1, fb, par1, 0, 0, 0);
-                }
+            for (int t = 0; t < 4; t++) {
+                fa0[t] = *reinterpret_cast<const half8_t*>(pa0 + 16 * t);
+                fa1[t] = *reinterpret_cast<const half8_t*>(pa1 + 16 * t);
+                fb[t] = *reinterpret_cast<const half8_t*>(pb + 16 * t);
+            }
+            const bool more = cc < 3 || sbk + 1 < nb;
+            const int nsb = cc < 3 ? sbk : sbk + 1, ncc = (cc + 1) & 3;
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                par0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0[t], fb[t], par0, 0, 0, 0);
+                par1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1[t], fb[t], par1, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (more) stash_part(t, nsb, ncc, st[ncc]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // end of the superblock: fold the partial tiles into the totals
