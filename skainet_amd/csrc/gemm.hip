@@ -245,47 +245,47 @@ __global__ __launch_bounds__(256) void gemm_dense_hilo_kernel(const _Float16* __
 // the activation sub-block sums (fp16 hi + lo) and the integers m_j, folded in with dmin.
 // Workgroup tile 128 x 64, 64 k per iteration (one chunk of every weight row: 32 nibble bytes, a quarter per
 // thread, unpacked into 64 fp16).
+template <int MT>
 __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restrict__ a16,
                                                        const _Float16* __restrict__ sum_hi,
                                                        const _Float16* __restrict__ sum_lo,
                                                        const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
                                                        float* __restrict__ c, int m, int n, int k) {
-    // 2 x 2 wavefronts, each a 64 x 32 part of the tile.
+    // 2 x 2 wavefronts, each MT 32 x 32 tiles stacked along m: workgroup tile (64 * MT) x 64.  MT = 1 doubles the
+    // number of workgroups (two per compute unit, whose phases overlap) for outputs too small to fill the chip.
+    constexpr int BM = 64 * MT;
     // Two LDS buffers (one barrier per iteration) and a ring of four register stages: the global loads of
     // iterations it+1 .. it+3 are in flight while iteration it is multiplied.  Four iterations = one superblock,
     // so the position in the ring is also the chunk index within the superblock.  Every thread issues the same
     // loads every iteration (no load sits in a conditional block): the wait counters then say exactly which
     // stage is complete.
-    __shared__ __align__(16) _Float16 sa[2][kBM * kRow];
+    __shared__ __align__(16) _Float16 sa[2][BM * kRow];
     __shared__ __align__(16) _Float16 sb[2][kBN * kRow];
     __shared__ float sd[2][kBN], sdm[2][kBN];
     __shared__ __align__(8) _Float16 smin[2][kBN * 8];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * kBN;
     const int nb = k >> 8, nsub = k >> 5;
 
     struct Stage {
-        u32x4 a0, a1, a2, a3, h;
+        u32x4 a[2 * MT], h;
         u32x2 q;
     };
     Stage st[4];
-    // activation staging: 128 rows x 8 chunks of 16 bytes, four per thread
+    // activation staging: BM rows x 8 chunks of 16 bytes, 2 * MT per thread (rows srow, srow + 32, ...)
     const int srow = tid >> 3, sch = (tid & 7) * 8;
-    const _Float16* ga0 = a16 + (size_t)min(m0 + srow, m - 1) * k + sch;
-    const _Float16* ga1 = a16 + (size_t)min(m0 + srow + 32, m - 1) * k + sch;
-    const _Float16* ga2 = a16 + (size_t)min(m0 + srow + 64, m - 1) * k + sch;
-    const _Float16* ga3 = a16 + (size_t)min(m0 + srow + 96, m - 1) * k + sch;
+    const _Float16* ga[2 * MT];
+#pragma unroll
+    for (int i = 0; i < 2 * MT; i++) ga[i] = a16 + (size_t)min(m0 + srow + 32 * i, m - 1) * k + sch;
     // weight staging: thread t owns row t / 4 of the tile and quarter t % 4 of the 32 nibble bytes of a chunk
     const int brow = tid >> 2, bq = tid & 3;
     const uint8_t* gw = w + (size_t)min(n0 + brow, n - 1) * nb * 144;
 
     auto fetch = [&](int sbk, int cc, Stage& s) __attribute__((always_inline)) {
         const int k0 = (4 * sbk + cc) * kKC;
-        s.a0 = *reinterpret_cast<const u32x4*>(ga0 + k0);
-        s.a1 = *reinterpret_cast<const u32x4*>(ga1 + k0);
-        s.a2 = *reinterpret_cast<const u32x4*>(ga2 + k0);
-        s.a3 = *reinterpret_cast<const u32x4*>(ga3 + k0);
+#pragma unroll
+        for (int i = 0; i < 2 * MT; i++) s.a[i] = *reinterpret_cast<const u32x4*>(ga[i] + k0);
         s.h = *reinterpret_cast<const u32x4*>(gw + (size_t)sbk * 144);
         s.q = *reinterpret_cast<const u32x2*>(gw + (size_t)sbk * 144 + 16 + 32 * cc + 8 * bq);
     };
@@ -295,14 +295,10 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
     auto stash_part = [&](int part, int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
         _Float16* da = sa[cc & 1];
         _Float16* db = sb[cc & 1];
-        if (part == 0) {
-            *reinterpret_cast<u32x4*>(da + srow * kRow + sch) = s.a0;
-            *reinterpret_cast<u32x4*>(da + (srow + 32) * kRow + sch) = s.a1;
-            return;
-        }
-        if (part == 1) {
-            *reinterpret_cast<u32x4*>(da + (srow + 64) * kRow + sch) = s.a2;
-            *reinterpret_cast<u32x4*>(da + (srow + 96) * kRow + sch) = s.a3;
+        if (part < 2) {
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+                *reinterpret_cast<u32x4*>(da + (srow + 32 * (MT * part + i)) * kRow + sch) = s.a[MT * part + i];
             return;
         }
         // the whole loaded tuple counts as used here: a word that this chunk does not need (d | dmin outside
@@ -345,14 +341,18 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
         for (int part = 0; part < 4; part++) stash_part(part, sbk, cc, s);
     };
 
-    float16_t tot0, tot1, par0, par1;
+    float16_t tot[MT], par[MT];
 #pragma unroll
-    for (int r = 0; r < 16; r++) tot0[r] = tot1[r] = par0[r] = par1[r] = 0.f;
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) tot[i][r] = par[i][r] = 0.f;
 
     // activation sub-block sums of this wavefront's two row tiles: lane l holds row l % 32, sub-blocks
     // 4 * (l / 32) .. + 3 of the current superblock (the operand layout of the eight-deep matrix instruction)
-    const int srow0 = min(m0 + wm * 64 + (lane & 31), m - 1), srow1 = min(m0 + wm * 64 + 32 + (lane & 31), m - 1);
-    const size_t soff0 = (size_t)srow0 * nsub + 4 * (lane >> 5), soff1 = (size_t)srow1 * nsub + 4 * (lane >> 5);
+    size_t soff[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+        soff[i] = (size_t)min(m0 + wm * 32 * MT + 32 * i + (lane & 31), m - 1) * nsub + 4 * (lane >> 5);
     const int pfrag = (lane & 31) * kRow + (lane >> 5) * 8;
 
     // Software pipeline: while the matrix instructions of iteration it run, the wavefront unpacks and stores
@@ -362,35 +362,35 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
     fetch(0, 2, st[2]);
     stash(0, 0, st[0]);
     for (int sbk = 0; sbk < nb; sbk++) {
-        half4_t sh0, sl0, sh1, sl1;
+        half4_t sh[MT], sl[MT];
 #pragma unroll
         for (int cc = 0; cc < 4; cc++) {
             // the stage three iterations ahead
             if (cc == 0) fetch(sbk, 3, st[3]);
             else fetch(min(sbk + 1, nb - 1), cc - 1, st[cc - 1]);  // (past the end: repeats the last superblock, unused)
             if (cc == 0) {
-                sh0 = *reinterpret_cast<const half4_t*>(sum_hi + soff0 + 8 * sbk);
-                sl0 = *reinterpret_cast<const half4_t*>(sum_lo + soff0 + 8 * sbk);
-                sh1 = *reinterpret_cast<const half4_t*>(sum_hi + soff1 + 8 * sbk);
-                sl1 = *reinterpret_cast<const half4_t*>(sum_lo + soff1 + 8 * sbk);
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    sh[i] = *reinterpret_cast<const half4_t*>(sum_hi + soff[i] + 8 * sbk);
+                    sl[i] = *reinterpret_cast<const half4_t*>(sum_lo + soff[i] + 8 * sbk);
+                }
             }
             __syncthreads();  // buffer cc & 1 is complete, and nobody reads the other one any more
-            const _Float16* pa0 = sa[cc & 1] + wm * 64 * kRow + pfrag;
-            const _Float16* pa1 = pa0 + 32 * kRow;
+            const _Float16* pa = sa[cc & 1] + wm * 32 * MT * kRow + pfrag;
             const _Float16* pb = sb[cc & 1] + wn * 32 * kRow + pfrag;
-            half8_t fa0[4], fa1[4], fb[4];
+            half8_t fa[MT][4], fb[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                fa0[t] = *reinterpret_cast<const half8_t*>(pa0 + 16 * t);
-                fa1[t] = *reinterpret_cast<const half8_t*>(pa1 + 16 * t);
+#pragma unroll
+                for (int i = 0; i < MT; i++) fa[i][t] = *reinterpret_cast<const half8_t*>(pa + 32 * i * kRow + 16 * t);
                 fb[t] = *reinterpret_cast<const half8_t*>(pb + 16 * t);
             }
             const bool more = cc < 3 || sbk + 1 < nb;
             const int nsb = cc < 3 ? sbk : sbk + 1, ncc = (cc + 1) & 3;
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                par0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0[t], fb[t], par0, 0, 0, 0);
-                par1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1[t], fb[t], par1, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < MT; i++) par[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i][t], fb[t], par[i], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
                 if (more) stash_part(t, nsb, ncc, st[ncc]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -398,24 +398,25 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
         }
         // end of the superblock: fold the partial tiles into the totals
         const half4_t fm = *reinterpret_cast<const half4_t*>(smin[sbk & 1] + (wn * 32 + (lane & 31)) * 8 + 4 * (lane >> 5));
-        float16_t mn0, mn1;
-#pragma unroll
-        for (int r = 0; r < 16; r++) mn0[r] = mn1[r] = 0.f;
-        mn0 = __builtin_amdgcn_mfma_f32_32x32x8f16(sh0, fm, mn0, 0, 0, 0);
-        mn1 = __builtin_amdgcn_mfma_f32_32x32x8f16(sh1, fm, mn1, 0, 0, 0);
-        mn0 = __builtin_amdgcn_mfma_f32_32x32x8f16(sl0, fm, mn0, 0, 0, 0);
-        mn1 = __builtin_amdgcn_mfma_f32_32x32x8f16(sl1, fm, mn1, 0, 0, 0);
         const float ds = sd[sbk & 1][wn * 32 + (lane & 31)];
         const float dm = sdm[sbk & 1][wn * 32 + (lane & 31)];
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            tot0[r] = fmaf(ds, par0[r], fmaf(-dm, mn0[r], tot0[r]));
-            tot1[r] = fmaf(ds, par1[r], fmaf(-dm, mn1[r], tot1[r]));
-            par0[r] = par1[r] = 0.f;
+        for (int i = 0; i < MT; i++) {
+            float16_t mn;
+#pragma unroll
+            for (int r = 0; r < 16; r++) mn[r] = 0.f;
+            mn = __builtin_amdgcn_mfma_f32_32x32x8f16(sh[i], fm, mn, 0, 0, 0);
+            mn = __builtin_amdgcn_mfma_f32_32x32x8f16(sl[i], fm, mn, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                tot[i][r] = fmaf(ds, par[i][r], fmaf(-dm, mn[r], tot[i][r]));
+                par[i][r] = 0.f;
+            }
         }
     }
-    store_tile(tot0, c, n, m0 + wm * 64, n0 + wn * 32, m, n, inv_scale, lane);
-    store_tile(tot1, c, n, m0 + wm * 64 + 32, n0 + wn * 32, m, n, inv_scale, lane);
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+        store_tile(tot[i], c, n, m0 + wm * 32 * MT + 32 * i, n0 + wn * 32, m, n, inv_scale, lane);
 }
 
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
@@ -470,9 +471,17 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
                     "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
         skn_launch(ctx, prep_a_q4k_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, sum_hi, sum_lo, k);
         SKN_LAUNCH_CHECK(ctx);
-        dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
-        skn_launch(ctx, gemm_q4k_kernel, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
-                   (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
+        // 128-row tiles when they alone give every compute unit two workgroups, 64-row tiles otherwise
+        const int wide = ((n + kBN - 1) / kBN) * ((m + 127) / 128);
+        if (wide >= 2 * ctx->compute_units) {
+            dim3 grid((n + kBN - 1) / kBN, (m + 127) / 128);
+            skn_launch(ctx, gemm_q4k_kernel<2>, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
+                       (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
+        } else {
+            dim3 grid((n + kBN - 1) / kBN, (m + 63) / 64);
+            skn_launch(ctx, gemm_q4k_kernel<1>, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
+                       (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
+        }
         SKN_LAUNCH_CHECK(ctx);
         return SKN_OK;
     }
