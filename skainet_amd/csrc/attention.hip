@@ -84,6 +84,9 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     for (int j = 0; j < 8; j++) o[j] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* trow = table + (size_t)kv_seq * pages_per_seq;
+    // the first 64 page ids of the sequence ride in a register (lane i holds page i), fetched here together with
+    // the length and the query instead of once the token range is known: one dependent round trip less
+    const int my_page = trow[min(lane, pages_per_seq - 1)];
 
     for (int base = t_begin; base < t_end; base += NS * U) {
         u32x4 kk[U], vv[U];
@@ -96,7 +99,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
             const int tc = min(t, t_end - 1);  // past the end: a valid row, masked below
             const int pi = POW2 ? tc >> page_shift : tc / page_tokens;
             slot[u] = tc - pi * page_tokens;
-            page[u] = trow[pi];
+            page[u] = __shfl(my_page, pi & 63, 64);
+            if (pi >= 64) page[u] = trow[pi];
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
