@@ -159,6 +159,57 @@ def bench_gemm(ctx, qtype, m, n, k, reps=20):
             "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
+def bench_dequant(ctx, qtype, n, k, reps=20):
+    """Block dequantization to fp32: bytes read + bytes written per launch against the HBM peak."""
+    w = ctx.to_device(synth.weight(qtype, n, k, seed=17))
+    out = ctx.alloc(4 * n * k)
+    for _ in range(3):
+        ctx.dequant(qtype, w, n * k, out)
+    ctx.prof_start(reps)
+    for _ in range(reps):
+        ctx.dequant(qtype, w, n * k, out)
+    ms, launches = ctx.prof_stop()
+    be, bb = synth.BLOCK[qtype]
+    nbytes = n * (k // be) * bb + 4 * n * k
+    w.free()
+    out.free()
+    us = ms / launches * 1e3
+    return {"kernel_us": round(us, 1), "gbs": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def bench_kv(ctx, steps=200):
+    """Paged KV cache, 8 sequences x 32 heads x 128: appending one token per sequence (131 072 bytes written per
+    step) and gathering 4096 tokens of one sequence back (64 MiB moved)."""
+    n_seq, n_head, dim, n_ctx = 8, 32, 128, 4096
+    kv = ctx.kv_cache(n_seq, n_head, dim, 256, 8192)
+    k1 = ctx.to_device(synth.kv_f16((n_seq, n_head, dim), seed=90))
+    v1 = ctx.to_device(synth.kv_f16((n_seq, n_head, dim), seed=91))
+    seqs = list(range(n_seq))
+    for _ in range(20):
+        kv.append(k1, v1, seqs)
+    ctx.prof_start(4 * steps)
+    for _ in range(steps):
+        kv.append(k1, v1, seqs)
+    ms, launches = ctx.prof_stop()
+    append_us = ms / steps * 1e3
+    run_k = ctx.to_device(synth.kv_f16((n_ctx, n_head, dim), seed=92))
+    run_v = ctx.to_device(synth.kv_f16((n_ctx, n_head, dim), seed=93))
+    kv.reset(0)
+    kv.append_run(0, run_k, run_v, n_ctx)
+    gk, gv = ctx.alloc(n_ctx * n_head * dim * 2), ctx.alloc(n_ctx * n_head * dim * 2)
+    kv.gather(0, 0, n_ctx, gk, gv)
+    ctx.prof_start(40)
+    for _ in range(10):
+        kv.gather(0, 0, n_ctx, gk, gv)
+    gms, gl = ctx.prof_stop()
+    gather_us = gms / 10 * 1e3
+    moved = 2 * 2 * n_ctx * n_head * dim * 2  # K and V, read and written
+    kv.free()
+    return {"append_us_per_step": round(append_us, 2), "append_launches_per_step": launches / steps,
+            "append_bytes_per_step": 2 * n_seq * n_head * dim * 2, "gather_4096_tokens_us": round(gather_us, 1),
+            "gather_gbs": round(moved / gather_us / 1e3, 1)}
+
+
 def cpu_baseline(qtype, n, k, budget_s=10.0):
     """The CPU oracle (C, OpenMP over rows) on the headline workload; a bounded number of repetitions."""
     from oracle import oracle_c  # the checker, timed as the "port" CPU baseline -- never the product path
@@ -260,6 +311,9 @@ def main():
             r = bench_matvec(ctx, qt, 4096, 4096, 200, 20, copies=24, seed=7000 + qt)
             other[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
         extra["other_formats_4096x4096"] = other
+        extra["dequant_4096x4096"] = {name: bench_dequant(ctx, qt, 4096, 4096)
+                                      for name, qt in (("q8_0", Q8_0), ("q4_k", Q4_K), ("q6_k", Q6_K))}
+        extra["kv_cache_8x32x128"] = bench_kv(ctx)
         att = bench_attention(ctx, min(args.steps, 200), 10)
         extra["attention_8x32x128_ctx4096"] = {key: round(val, 4) for key, val in att.items()}
         extra["prefill_gemm"] = {f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
