@@ -351,8 +351,8 @@ def main():
             "unit": "GB/s",
             "frac": round(head["kernel_gbs"] / HBM_PEAK_GBS, 4),
             # HBM bytes of one launch from hardware counters (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, one run
-            # each, scaled by what the same counters read for a copy kernel of this size): 1.017 x algorithmic
-            "traffic": 25850432,
+            # each, scaled by what the same counters read for a copy kernel of this size): 1.015 x algorithmic
+            "traffic": 25813511,
             "kernel": "matvec_q4k_kernel",
             "kernel_us": round(head["kernel_us"], 3),
             "cache_hot_gbs": round(head["hot_kernel_gbs"], 2),
