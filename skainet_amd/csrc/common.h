@@ -105,6 +105,8 @@ static inline bool skn_is_quant(int t) {
 }
 int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out);
 int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y);
+int skn_dequant_hilo(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
+int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
 
 // ---- device helpers --------------------------------------------------------------------------------
 

@@ -152,6 +152,38 @@ __global__ __launch_bounds__(256) void dequant_blocks_kernel(const uint8_t* __re
     reinterpret_cast<float4*>(out)[t] = Fmt<T>::decode4(w + (t / QB) * Fmt<T>::kBytes, (int)(t % QB));
 }
 
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+// the same decode written as an fp16 pair hi = f16(w), lo = f16(w - hi) (for the GEMM)
+template <int T>
+__global__ __launch_bounds__(256) void dequant_blocks_hilo_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ hi,
+                                                                  _Float16* __restrict__ lo, int64_t n_quads) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_quads) return;
+    constexpr int QB = Fmt<T>::kElems / 4;
+    const float4 y = Fmt<T>::decode4(w + (t / QB) * Fmt<T>::kBytes, (int)(t % QB));
+    const float v[4] = {y.x, y.y, y.z, y.w};
+    half4_t h, l;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        h[i] = (_Float16)v[i];
+        l[i] = (_Float16)(v[i] - (float)h[i]);
+    }
+    reinterpret_cast<half4_t*>(hi)[t] = h;
+    reinterpret_cast<half4_t*>(lo)[t] = l;
+}
+
+template <int T>
+__global__ __launch_bounds__(256) void convert_dense_hilo_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ hi,
+                                                                 _Float16* __restrict__ lo, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = dense_at<T>(w, i);
+    const _Float16 h = (_Float16)v;
+    hi[i] = h;
+    lo[i] = (_Float16)(v - (float)h);
+}
+
 template <int T>
 __global__ __launch_bounds__(256) void convert_dense_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
                                                             int64_t n) {
@@ -245,6 +277,42 @@ int launch_matvec_dense(skn_ctx* ctx, const uint8_t* w, int n, int k, const floa
     return SKN_OK;
 }
 
+template <int T>
+int launch_hilo(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
+    const int64_t n_quads = n_elems / 4, blocks = (n_quads + 255) / 256;
+    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_gemm_q: too many weights for one launch");
+    skn_launch(ctx, dequant_blocks_hilo_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, hi, lo, n_quads);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int T>
+int launch_hilo_dense(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
+    const int64_t blocks = (n_elems + 255) / 256;
+    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_gemm_q: too many weights for one launch");
+    skn_launch(ctx, convert_dense_hilo_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, hi, lo, n_elems);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+}  // namespace
+
+int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
+    switch (ggml_type) {
+        case SKN_TYPE_Q4_0: return launch_hilo<SKN_TYPE_Q4_0>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q4_1: return launch_hilo<SKN_TYPE_Q4_1>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q5_0: return launch_hilo<SKN_TYPE_Q5_0>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q5_1: return launch_hilo<SKN_TYPE_Q5_1>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q2_K: return launch_hilo<SKN_TYPE_Q2_K>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q5_K: return launch_hilo<SKN_TYPE_Q5_K>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_F32: return launch_hilo_dense<SKN_TYPE_F32>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_F16: return launch_hilo_dense<SKN_TYPE_F16>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_BF16: return launch_hilo_dense<SKN_TYPE_BF16>(ctx, w, n_elems, hi, lo);
+        default: return skn_fail(ctx, SKN_ERR_TYPE, "skn_gemm_q: ggml type %d is not supported", ggml_type);
+    }
+}
+
+namespace {
 }  // namespace
 
 // Called by skn_dequant / skn_matvec_q after their argument checks, for the types they do not handle themselves.

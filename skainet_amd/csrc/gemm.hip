@@ -486,26 +486,21 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
         return SKN_OK;
     }
 
-    // workspace: fp16 activations + row scales, then (general path) fp32 weights and their fp16 pair
+    // workspace: fp16 activations + row scales, then (general path) the weights as an fp16 pair
     const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
-    const size_t wf_bytes = align_up((size_t)n * k * 4), wh_bytes = align_up((size_t)n * k * 2);
+    const size_t wh_bytes = align_up((size_t)n * k * 2);
     uint8_t* ws;
-    int rc = gemm_workspace(ctx, a16_bytes + sc_bytes + wf_bytes + 2 * wh_bytes, &ws);
+    int rc = gemm_workspace(ctx, a16_bytes + sc_bytes + 2 * wh_bytes, &ws);
     if (rc != SKN_OK) return rc;
     _Float16* a16 = (_Float16*)ws;
     float* inv_scale = (float*)(ws + a16_bytes);
-    float* wf = (float*)(ws + a16_bytes + sc_bytes);
-    _Float16* whi = (_Float16*)(ws + a16_bytes + sc_bytes + wf_bytes);
-    _Float16* wlo = (_Float16*)(ws + a16_bytes + sc_bytes + wf_bytes + wh_bytes);
+    _Float16* whi = (_Float16*)(ws + a16_bytes + sc_bytes);
+    _Float16* wlo = (_Float16*)(ws + a16_bytes + sc_bytes + wh_bytes);
 
     skn_launch(ctx, prep_a_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, k);
     SKN_LAUNCH_CHECK(ctx);
-    rc = skn_dequant(ctx, ggml_type, w_dev, (int64_t)n * k, wf);
+    rc = skn_dequant_hilo(ctx, ggml_type, (const uint8_t*)w_dev, (int64_t)n * k, whi, wlo);
     if (rc != SKN_OK) return rc;
-    const int64_t total = (int64_t)n * k;
-    skn_launch(ctx, split_hilo_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (const float*)wf, whi, wlo,
-               total);
-    SKN_LAUNCH_CHECK(ctx);
     dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
     skn_launch(ctx, gemm_dense_hilo_kernel, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)whi,
                (const _Float16*)wlo, (const float*)inv_scale, c_dev, m, n, k);
