@@ -307,7 +307,8 @@ def main():
             extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
         # the further formats (plain streaming kernels): 4096 x 4096 matvec, kernel GB/s
         other = {}
-        for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q5_k", 13), ("f16", 1)):
+        for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q3_k", 11), ("q5_k", 13),
+                         ("q8_k", 15), ("iq4_nl", 20), ("iq4_xs", 23), ("f16", 1)):
             r = bench_matvec(ctx, qt, 4096, 4096, 200, 20, copies=24, seed=7000 + qt)
             other[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
         extra["other_formats_4096x4096"] = other

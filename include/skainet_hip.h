@@ -48,9 +48,13 @@ extern "C" {
 #define SKN_TYPE_Q5_1 7
 #define SKN_TYPE_Q8_0 8
 #define SKN_TYPE_Q2_K 10
+#define SKN_TYPE_Q3_K 11
 #define SKN_TYPE_Q4_K 12
 #define SKN_TYPE_Q5_K 13
 #define SKN_TYPE_Q6_K 14
+#define SKN_TYPE_Q8_K 15
+#define SKN_TYPE_IQ4_NL 20
+#define SKN_TYPE_IQ4_XS 23
 #define SKN_TYPE_BF16 30
 
 typedef struct skn_ctx skn_ctx;

@@ -20,7 +20,7 @@
  *   orc_dequant_* ..................... unpinned by the reference (it has no dequantizer); pinned by hand-built
  *                                       single-block known answers, an independent NumPy restatement
  *                                       (oracle/oracle_np.py) and the fp64 closed form rounded once
- *   deq_q4_0/q4_1/q5_0/q5_1/q2_k/q5_k . the further formats of the reference's size table: unpinned by the reference
+ *   deq_q4_0 ... deq_iq4_xs ........... the further formats of the reference's size table: unpinned by the reference
  *                                       in the same way; pinned by hand-built tagged blocks (element order, fifth-bit
  *                                       positions, scale indices), the NumPy restatement and exact rational goldens
  *                                       (tests/golden/quant_blocks_more.npz)
@@ -44,7 +44,7 @@
 #define ORC_ERR_SHAPE (-3)
 
 enum { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8, T_Q2_K = 10, T_Q4_K = 12,
-       T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30 };
+       T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30, T_Q3_K = 11, T_Q8_K = 15, T_IQ4_NL = 20, T_IQ4_XS = 23 };
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -142,6 +142,10 @@ int orc_type_sizes(int type, int* block_elems, int* block_bytes) {
         case T_Q5_1: *block_elems = 32; *block_bytes = 2 + 2 + 4 + 16; return ORC_OK;
         case T_Q2_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 16 + 256 / 4; return ORC_OK;
         case T_Q5_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 256 / 8 + 12; return ORC_OK;
+        case T_Q3_K: *block_elems = 256; *block_bytes = 2 + 256 / 4 + 256 / 8 + 12; return ORC_OK;
+        case T_Q8_K: *block_elems = 256; *block_bytes = 4 + 256 + 256 / 8; return ORC_OK;
+        case T_IQ4_NL: *block_elems = 32; *block_bytes = 2 + 16; return ORC_OK;
+        case T_IQ4_XS: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 256 / 64; return ORC_OK;
         case T_Q8_0: *block_elems = 32; *block_bytes = 2 + 32; return ORC_OK;
         case T_Q4_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 12; return ORC_OK;
         case T_Q6_K: *block_elems = 256; *block_bytes = 2 + 256 / 2 + 256 / 4 + 256 / 16; return ORC_OK;
@@ -310,9 +314,63 @@ static void deq_q5_k_block(const uint8_t* b, float* y) {
     }
 }
 
+/* Q3_K: hmask u8[32] @0, qs u8[64] @32, scales u8[12] @96, d f16 @108.  Sixteen 6-bit scales (low nibbles of
+ * bytes 0..7 for scales 0..7, high nibbles for 8..15; two more bits each from bytes 8..11), stored with an
+ * offset of 32.  Element e: half n = e / 128, bit pair j = (e % 128) / 32, l = e % 32: two bits of qs[32n + l] at
+ * 2j, minus 4 unless bit 4n + j of hmask[l] is set; scale 8n + 2j + (l >= 16).  y = d * (sc - 32) * q. */
+static void deq_q3_k_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b + 108);
+    const uint8_t* s = b + 96;
+    for (int e = 0; e < 256; e++) {
+        const int n = e / 128, j = (e % 128) / 32, l = e % 32;
+        const int is = 8 * n + 2 * j + (l >= 16);
+        const int lo4 = is < 8 ? (s[is] & 0x0F) : (s[is - 8] >> 4);
+        const int hi2 = (s[8 + is % 4] >> (2 * (is / 4))) & 3;
+        const int sc = (lo4 | (hi2 << 4)) - 32;
+        const int q = (int)((b[32 + 32 * n + l] >> (2 * j)) & 3) - (((b[l] >> (4 * n + j)) & 1) ? 0 : 4);
+        y[e] = d * (float)sc * (float)q;
+    }
+}
+
+/* Q8_K: d f32 @0, qs i8[256] @4, bsums i16[16] @260 (sums of 16 quants each; not used by the values).  y = d * q. */
+static void deq_q8_k_block(const uint8_t* b, float* y) {
+    float d;
+    memcpy(&d, b, 4);
+    for (int e = 0; e < 256; e++) y[e] = d * (float)(int8_t)b[4 + e];
+}
+
+/* the sixteen values of the non-linear 4-bit formats */
+static const int8_t kIq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+/* IQ4_NL: d f16 @0, qs u8[16] @2.  Low nibbles are elements 0..15, high nibbles 16..31; y = d * table[q]. */
+static void deq_iq4_nl_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b);
+    for (int j = 0; j < 16; j++) {
+        y[j] = d * (float)kIq4nl[b[2 + j] & 0x0F];
+        y[j + 16] = d * (float)kIq4nl[b[2 + j] >> 4];
+    }
+}
+
+/* IQ4_XS: d f16 @0, scales_h u16 @2, scales_l u8[4] @4, qs u8[128] @8.  Eight sub-blocks of 32 with a 6-bit
+ * scale (low 4 bits in the nibbles of scales_l, high 2 bits in scales_h), offset 32; values as IQ4_NL. */
+static void deq_iq4_xs_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b);
+    const unsigned sh = (unsigned)b[2] | ((unsigned)b[3] << 8);
+    for (int ib = 0; ib < 8; ib++) {
+        const int ls = ((b[4 + ib / 2] >> (4 * (ib % 2))) & 0x0F) | (int)(((sh >> (2 * ib)) & 3u) << 4);
+        const float dl = d * (float)(ls - 32);
+        const uint8_t* qs = b + 8 + 16 * ib;
+        for (int j = 0; j < 16; j++) {
+            y[32 * ib + j] = dl * (float)kIq4nl[qs[j] & 0x0F];
+            y[32 * ib + j + 16] = dl * (float)kIq4nl[qs[j] >> 4];
+        }
+    }
+}
+
 static int is_block_type(int type) {
     return type == T_Q8_0 || type == T_Q4_K || type == T_Q6_K || type == T_Q4_0 || type == T_Q4_1 || type == T_Q5_0 ||
-           type == T_Q5_1 || type == T_Q2_K || type == T_Q5_K || type == T_F16 || type == T_BF16 || type == T_F32;
+           type == T_Q5_1 || type == T_Q2_K || type == T_Q5_K || type == T_F16 || type == T_BF16 || type == T_F32 ||
+           type == T_Q3_K || type == T_Q8_K || type == T_IQ4_NL || type == T_IQ4_XS;
 }
 
 static void deq_block(int type, const uint8_t* b, float* y) {
@@ -327,6 +385,10 @@ static void deq_block(int type, const uint8_t* b, float* y) {
         case T_Q5_1: deq_q5_1_block(b, y); break;
         case T_Q2_K: deq_q2_k_block(b, y); break;
         case T_Q5_K: deq_q5_k_block(b, y); break;
+        case T_Q3_K: deq_q3_k_block(b, y); break;
+        case T_Q8_K: deq_q8_k_block(b, y); break;
+        case T_IQ4_NL: deq_iq4_nl_block(b, y); break;
+        case T_IQ4_XS: deq_iq4_xs_block(b, y); break;
         case T_F16: memcpy(&h, b, 2); y[0] = orc_h2f(h); break;
         case T_BF16: memcpy(&h, b, 2); y[0] = orc_bf2f(h); break;
         default: memcpy(y, b, 4); break; /* F32 */

@@ -25,6 +25,7 @@ import numpy as np
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 F32, F16, BF16 = 0, 1, 30
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
+Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
 
 # Constants.kt:58-90 restricted to the types this library computes with: type -> (block elems, block bytes)
 QUANT_SIZES = {
@@ -40,9 +41,14 @@ QUANT_SIZES = {
     Q4_K: (256, 2 + 2 + 256 // 2 + 12),
     Q5_K: (256, 2 + 2 + 256 // 2 + 256 // 8 + 12),
     Q6_K: (256, 2 + 256 // 2 + 256 // 4 + 256 // 16),
+    Q3_K: (256, 2 + 256 // 4 + 256 // 8 + 12),
+    Q8_K: (256, 4 + 256 + 256 // 8),
+    IQ4_NL: (32, 2 + 16),
+    IQ4_XS: (256, 2 + 2 + 256 // 2 + 256 // 64),
 }
 TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", F32: "F32", F16: "F16", BF16: "BF16", Q4_0: "Q4_0",
-              Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q2_K: "Q2_K", Q5_K: "Q5_K"}
+              Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q2_K: "Q2_K", Q5_K: "Q5_K", Q3_K: "Q3_K", Q8_K: "Q8_K",
+              IQ4_NL: "IQ4_NL", IQ4_XS: "IQ4_XS"}
 
 
 def quant_shape_to_byte_shape(shape, qtype):
@@ -193,6 +199,54 @@ def dequant_q5_k(raw):
     return y.astype(np.float32).reshape(-1)
 
 
+def dequant_q3_k(raw):
+    b = _blocks(raw, Q3_K)
+    nb = b.shape[0]
+    hm = b[:, 0:32]
+    qs = b[:, 32:96].reshape(nb, 2, 1, 32)
+    s = b[:, 96:108].astype(np.int32)
+    low = np.concatenate([s[:, 0:8] & 0x0F, s[:, 0:8] >> 4], axis=1)                       # [nb,16]
+    idx = np.arange(16)
+    high = (s[:, 8 + idx % 4] >> (2 * (idx // 4))[None, :]) & 3                            # [nb,16]
+    sc = ((low | (high << 4)) - 32).reshape(nb, 2, 4, 2)                                   # [half][pair][first / second 16]
+    shifts = (2 * np.arange(4, dtype=np.uint8)).reshape(1, 1, 4, 1)
+    q2 = ((qs >> shifts) & 3).astype(np.int32)                                             # [nb,2,4,32]
+    bitpos = (4 * np.arange(2)[:, None] + np.arange(4)[None, :]).astype(np.uint8)          # [2,4]
+    hbit = (hm[:, None, None, :] >> bitpos[None, :, :, None]) & 1                          # [nb,2,4,32]
+    q = q2 - 4 * (1 - hbit.astype(np.int32))
+    scale = np.repeat(sc, 16, axis=3).astype(np.float64)                                   # [nb,2,4,32]
+    d = _f16(b[:, 108:110])[:, None, None, None]
+    return (d * scale * q).astype(np.float32).reshape(-1)
+
+
+def dequant_q8_k(raw):
+    b = _blocks(raw, Q8_K)
+    d = np.ascontiguousarray(b[:, 0:4]).view("<f4").astype(np.float64)                     # [nb,1]
+    q = b[:, 4:260].view(np.int8).astype(np.float64)
+    return (d * q).astype(np.float32).reshape(-1)
+
+
+IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float64)
+
+
+def dequant_iq4_nl(raw):
+    b = _blocks(raw, IQ4_NL)
+    return (_f16(b[:, 0:2])[:, None] * IQ4_VALUES[_nibbles32(b[:, 2:18])]).astype(np.float32).reshape(-1)
+
+
+def dequant_iq4_xs(raw):
+    b = _blocks(raw, IQ4_XS)
+    nb = b.shape[0]
+    sh = b[:, 2].astype(np.int32) | (b[:, 3].astype(np.int32) << 8)
+    ib = np.arange(8)
+    low = (b[:, 4 + ib // 2].astype(np.int32) >> (4 * (ib % 2))[None, :]) & 0x0F
+    high = (sh[:, None] >> (2 * ib)[None, :]) & 3
+    ls = ((low | (high << 4)) - 32).astype(np.float64)                                      # [nb,8]
+    qs = b[:, 8:136].reshape(nb, 8, 16)
+    vals = IQ4_VALUES[np.concatenate([qs & 0x0F, qs >> 4], axis=2).astype(np.int64)]       # [nb,8,32]
+    return ((_f16(b[:, 0:2])[:, None] * ls)[:, :, None] * vals).astype(np.float32).reshape(-1)
+
+
 def dequant_f16(raw):
     return np.frombuffer(np.ascontiguousarray(raw), dtype="<f2").astype(np.float32)
 
@@ -207,6 +261,7 @@ def dequant_f32(raw):
 
 _DEQ = {Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q6_K: dequant_q6_k, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1,
         Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q2_K: dequant_q2_k, Q5_K: dequant_q5_k, F16: dequant_f16,
+        Q3_K: dequant_q3_k, Q8_K: dequant_q8_k, IQ4_NL: dequant_iq4_nl, IQ4_XS: dequant_iq4_xs,
         BF16: dequant_bf16, F32: dequant_f32}
 
 

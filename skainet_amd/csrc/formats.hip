@@ -1,5 +1,5 @@
 // The further ggml formats of the reference's size table (gguf/.../Constants.kt:58-90) that the library
-// computes with: Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K and the dense F32 / F16 / BF16.  One decode function per
+// computes with: Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS and the dense F32 / F16 / BF16.  One decode function per
 // format -- four consecutive elements of a block at a time, every value the exact real of its formula rounded
 // once (explicitly rounded intrinsics, so no contraction can change a bit) -- serves a dequantization kernel
 // (one thread per four outputs, 16-byte stores) and a batch-1 matvec (one wavefront per row, the lane's four
@@ -132,6 +132,80 @@ struct Fmt<SKN_TYPE_Q5_K> {
         y.z = __fsub_rn(__fmul_rn(d1, (float)(((q >> 16) & 0xF) | (((hb >> 16) & 1) << 4))), m1);
         y.w = __fsub_rn(__fmul_rn(d1, (float)(((q >> 24) & 0xF) | (((hb >> 24) & 1) << 4))), m1);
         return y;
+    }
+};
+
+// Q3_K, 110 B: hmask[32] @0, qs[64] @32, scales[12] @96, f16 d @108.  Sixteen 6-bit scales stored with an offset
+// of 32: low nibbles of bytes 0..7 for scales 0..7, high nibbles for 8..15, two more bits each from bytes 8..11.
+// Element e: half n = e / 128, bit pair j = (e % 128) / 32, l = e % 32: two bits of qs[32n + l] at 2j, minus 4
+// unless bit 4n + j of hmask[l] is set; scale 8n + 2j + (l >= 16).
+template <>
+struct Fmt<SKN_TYPE_Q3_K> {
+    static constexpr int kElems = 256, kBytes = 110;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, n = e >> 7, j = (e & 127) >> 5, l = e & 31;
+        const int is = 8 * n + 2 * j + (l >> 4);
+        const uint8_t* s = b + 96;
+        const int lo4 = is < 8 ? (s[is] & 0x0F) : (s[is - 8] >> 4);
+        const int hi2 = (s[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+        const float dl = __fmul_rn(ldh(b + 108), (float)((lo4 | (hi2 << 4)) - 32));
+        const uint32_t q = ld32(b + 32 + 32 * n + l) >> (2 * j);
+        const uint32_t hb = ld32(b + l) >> (4 * n + j);
+        float4 y;
+        y.x = __fmul_rn(dl, (float)((int)(q & 3) - ((hb & 1) ? 0 : 4)));
+        y.y = __fmul_rn(dl, (float)((int)((q >> 8) & 3) - (((hb >> 8) & 1) ? 0 : 4)));
+        y.z = __fmul_rn(dl, (float)((int)((q >> 16) & 3) - (((hb >> 16) & 1) ? 0 : 4)));
+        y.w = __fmul_rn(dl, (float)((int)((q >> 24) & 3) - (((hb >> 24) & 1) ? 0 : 4)));
+        return y;
+    }
+};
+
+// Q8_K, 292 B: f32 d @0, int8 qs[256] @4, int16 block sums @260 (not part of the values).  y = d * q.
+template <>
+struct Fmt<SKN_TYPE_Q8_K> {
+    static constexpr int kElems = 256, kBytes = 292;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = __uint_as_float(ld32(b));
+        const uint32_t q = ld32(b + 4 + 4 * g);
+        return make_float4(__fmul_rn(d, (float)(int8_t)(q & 0xFF)), __fmul_rn(d, (float)(int8_t)((q >> 8) & 0xFF)),
+                           __fmul_rn(d, (float)(int8_t)((q >> 16) & 0xFF)), __fmul_rn(d, (float)(int8_t)(q >> 24)));
+    }
+};
+
+// the sixteen values of the non-linear 4-bit formats, packed four to a word (index = nibble)
+__device__ __forceinline__ float iq4_value(uint32_t nibble) {
+    const uint32_t tab[4] = {0xBFAD9881u, 0xF6EADDCFu, 0x26190D01u, 0x71594535u};  // -127,-104,-83,-65 | -49,-35,-22,-10 | 1,13,25,38 | 53,69,89,113
+    const uint32_t w = nibble < 8 ? (nibble < 4 ? tab[0] : tab[1]) : (nibble < 12 ? tab[2] : tab[3]);
+    return (float)(int8_t)((w >> (8 * (nibble & 3))) & 0xFF);
+}
+
+// IQ4_NL, 18 B: f16 d @0, qs[16] @2.  Low nibbles are elements 0..15, high nibbles 16..31; y = d * table[q].
+template <>
+struct Fmt<SKN_TYPE_IQ4_NL> {
+    static constexpr int kElems = 32, kBytes = 18;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b);
+        uint32_t q = ld32(b + 2 + 4 * (g & 3));
+        if (g >= 4) q >>= 4;
+        return make_float4(__fmul_rn(d, iq4_value(q & 0xF)), __fmul_rn(d, iq4_value((q >> 8) & 0xF)),
+                           __fmul_rn(d, iq4_value((q >> 16) & 0xF)), __fmul_rn(d, iq4_value((q >> 24) & 0xF)));
+    }
+};
+
+// IQ4_XS, 136 B: f16 d @0, u16 scales_h @2, scales_l[4] @4, qs[128] @8.  Eight sub-blocks of 32 with a 6-bit scale
+// (low 4 bits in the nibbles of scales_l, high 2 bits in scales_h) stored with an offset of 32; values as IQ4_NL.
+template <>
+struct Fmt<SKN_TYPE_IQ4_XS> {
+    static constexpr int kElems = 256, kBytes = 136;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int ib = g >> 3, gg = g & 7;
+        const uint32_t sh = *reinterpret_cast<const uint16_t*>(b + 2);
+        const int ls = (int)(((b[4 + (ib >> 1)] >> (4 * (ib & 1))) & 0x0F) | (((sh >> (2 * ib)) & 3u) << 4));
+        const float dl = __fmul_rn(ldh(b), (float)(ls - 32));
+        uint32_t q = ld32(b + 8 + 16 * ib + 4 * (gg & 3));
+        if (gg >= 4) q >>= 4;
+        return make_float4(__fmul_rn(dl, iq4_value(q & 0xF)), __fmul_rn(dl, iq4_value((q >> 8) & 0xF)),
+                           __fmul_rn(dl, iq4_value((q >> 16) & 0xF)), __fmul_rn(dl, iq4_value((q >> 24) & 0xF)));
     }
 };
 
@@ -305,6 +379,10 @@ int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_
         case SKN_TYPE_Q5_1: return launch_hilo<SKN_TYPE_Q5_1>(ctx, w, n_elems, hi, lo);
         case SKN_TYPE_Q2_K: return launch_hilo<SKN_TYPE_Q2_K>(ctx, w, n_elems, hi, lo);
         case SKN_TYPE_Q5_K: return launch_hilo<SKN_TYPE_Q5_K>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q3_K: return launch_hilo<SKN_TYPE_Q3_K>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q8_K: return launch_hilo<SKN_TYPE_Q8_K>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_IQ4_NL: return launch_hilo<SKN_TYPE_IQ4_NL>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_IQ4_XS: return launch_hilo<SKN_TYPE_IQ4_XS>(ctx, w, n_elems, hi, lo);
         case SKN_TYPE_F32: return launch_hilo_dense<SKN_TYPE_F32>(ctx, w, n_elems, hi, lo);
         case SKN_TYPE_F16: return launch_hilo_dense<SKN_TYPE_F16>(ctx, w, n_elems, hi, lo);
         case SKN_TYPE_BF16: return launch_hilo_dense<SKN_TYPE_BF16>(ctx, w, n_elems, hi, lo);
@@ -324,6 +402,10 @@ int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_e
         case SKN_TYPE_Q5_1: return launch_dequant<SKN_TYPE_Q5_1>(ctx, w, n_elems, out);
         case SKN_TYPE_Q2_K: return launch_dequant<SKN_TYPE_Q2_K>(ctx, w, n_elems, out);
         case SKN_TYPE_Q5_K: return launch_dequant<SKN_TYPE_Q5_K>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q3_K: return launch_dequant<SKN_TYPE_Q3_K>(ctx, w, n_elems, out);
+        case SKN_TYPE_Q8_K: return launch_dequant<SKN_TYPE_Q8_K>(ctx, w, n_elems, out);
+        case SKN_TYPE_IQ4_NL: return launch_dequant<SKN_TYPE_IQ4_NL>(ctx, w, n_elems, out);
+        case SKN_TYPE_IQ4_XS: return launch_dequant<SKN_TYPE_IQ4_XS>(ctx, w, n_elems, out);
         case SKN_TYPE_F32: return launch_convert<SKN_TYPE_F32>(ctx, w, n_elems, out);
         case SKN_TYPE_F16: return launch_convert<SKN_TYPE_F16>(ctx, w, n_elems, out);
         case SKN_TYPE_BF16: return launch_convert<SKN_TYPE_BF16>(ctx, w, n_elems, out);
@@ -339,6 +421,10 @@ int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k
         case SKN_TYPE_Q5_1: return launch_matvec<SKN_TYPE_Q5_1>(ctx, w, n, k, x, y);
         case SKN_TYPE_Q2_K: return launch_matvec<SKN_TYPE_Q2_K>(ctx, w, n, k, x, y);
         case SKN_TYPE_Q5_K: return launch_matvec<SKN_TYPE_Q5_K>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q3_K: return launch_matvec<SKN_TYPE_Q3_K>(ctx, w, n, k, x, y);
+        case SKN_TYPE_Q8_K: return launch_matvec<SKN_TYPE_Q8_K>(ctx, w, n, k, x, y);
+        case SKN_TYPE_IQ4_NL: return launch_matvec<SKN_TYPE_IQ4_NL>(ctx, w, n, k, x, y);
+        case SKN_TYPE_IQ4_XS: return launch_matvec<SKN_TYPE_IQ4_XS>(ctx, w, n, k, x, y);
         case SKN_TYPE_F32: return launch_matvec_dense<SKN_TYPE_F32>(ctx, w, n, k, x, y);
         case SKN_TYPE_F16: return launch_matvec_dense<SKN_TYPE_F16>(ctx, w, n, k, x, y);
         case SKN_TYPE_BF16: return launch_matvec_dense<SKN_TYPE_BF16>(ctx, w, n, k, x, y);

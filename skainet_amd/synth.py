@@ -18,8 +18,10 @@ import numpy as np
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 F32, F16, BF16 = 0, 1, 30
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
+Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
 BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22),
-         Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176), F32: (1, 4), F16: (1, 2), BF16: (1, 2)}
+         Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
+         Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136)}
 
 
 def _f16_bytes(values):
@@ -82,7 +84,19 @@ def q5_k_blocks(n_blocks, rng):
     return b.reshape(-1)
 
 
+def q8_k_blocks(n_blocks, rng):
+    b = rng.integers(0, 256, size=(n_blocks, 292), dtype=np.uint8)
+    b[:, 0:4] = (np.abs(rng.standard_normal(n_blocks)) * 0.01).astype(np.float32).view(np.uint8).reshape(-1, 4)
+    q = b[:, 4:260].view(np.int8).astype(np.int16).reshape(n_blocks, 16, 16)
+    b[:, 260:292] = q.sum(axis=2).astype("<i2").view(np.uint8).reshape(n_blocks, 32)  # the block sums ggml keeps
+    return b.reshape(-1)
+
+
 _GEN = {
+    Q3_K: lambda n, rng: _scaled_blocks(n, rng, 110, (108,)),
+    Q8_K: q8_k_blocks,
+    IQ4_NL: lambda n, rng: _scaled_blocks(n, rng, 18, (0,)),
+    IQ4_XS: lambda n, rng: _scaled_blocks(n, rng, 136, (0,)),
     Q8_0: q8_0_blocks, Q4_K: q4_k_blocks, Q6_K: q6_k_blocks, Q5_K: q5_k_blocks,
     Q4_0: lambda n, rng: _scaled_blocks(n, rng, 18, (0,)),
     Q4_1: lambda n, rng: _scaled_blocks(n, rng, 20, (0, 2)),

@@ -263,11 +263,75 @@ def exact_q5_k(b):
     return out
 
 
+def _exact_product(d, factors, d_neg):
+    """d times small integers as an exactly rounded float32; the zero keeps the xor of the operand signs."""
+    v, neg = d, d_neg
+    for f in factors:
+        v *= f
+        neg ^= f < 0
+    return _round_f32(v) if v != 0 else _zero(neg)
+
+
+def exact_q3_k(b):
+    d = _f16_exact(b[108], b[109])
+    s = [int(v) for v in b[96:108]]
+    out = []
+    for e in range(256):
+        n, rem = divmod(e, 128)
+        j, l = divmod(rem, 32)
+        i = 8 * n + 2 * j + (1 if l >= 16 else 0)  # which of the sixteen scales
+        lo4 = (s[i] & 15) if i < 8 else (s[i - 8] >> 4)
+        hi2 = (s[8 + i % 4] >> (2 * (i // 4))) & 3
+        q = (int(b[32 + 32 * n + l]) >> (2 * j)) & 3
+        if not (int(b[l]) >> (4 * n + j)) & 1:
+            q -= 4
+        out.append(_exact_product(d, [(lo4 | (hi2 << 4)) - 32, q], _neg(b[108], b[109])))
+    return out
+
+
+def _f32_exact(b4):
+    bits = int(b4[0]) | (int(b4[1]) << 8) | (int(b4[2]) << 16) | (int(b4[3]) << 24)
+    sign = -1 if bits >> 31 else 1
+    e, m = (bits >> 23) & 0xFF, bits & 0x7FFFFF
+    assert e != 255, "fixtures hold finite scales only"
+    if e == 0:
+        return sign * Fraction(m, 1 << 149)
+    return sign * Fraction((1 << 23) + m, 1 << 23) * (Fraction(2) ** (e - 127))
+
+
+def exact_q8_k(b):
+    d = _f32_exact(b[0:4])
+    qs = [int(v) - 256 if v > 127 else int(v) for v in b[4:260]]
+    return [_exact_product(d, [q], bool(int(b[3]) & 0x80)) for q in qs]
+
+
+IQ4 = [-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113]
+
+
+def exact_iq4_nl(b):
+    d = _f16_exact(b[0], b[1])
+    return [_exact_product(d, [IQ4[q]], _neg(b[0], b[1])) for q in _nibbles32(b[2:18])]
+
+
+def exact_iq4_xs(b):
+    d = _f16_exact(b[0], b[1])
+    sh = int(b[2]) | (int(b[3]) << 8)
+    out = []
+    for ib in range(8):
+        ls = ((int(b[4 + ib // 2]) >> (4 * (ib % 2))) & 15) | (((sh >> (2 * ib)) & 3) << 4)
+        out += [_exact_product(d, [ls - 32, IQ4[q]], _neg(b[0], b[1])) for q in _nibbles32(b[8 + 16 * ib:24 + 16 * ib])]
+    return out
+
+
 EXACT = {synth.Q8_0: exact_q8_0, synth.Q4_K: exact_q4_k, synth.Q6_K: exact_q6_k}
 EXACT_MORE = {synth.Q4_0: exact_q4_0, synth.Q4_1: exact_q4_1, synth.Q5_0: exact_q5_0, synth.Q5_1: exact_q5_1,
-              synth.Q2_K: exact_q2_k, synth.Q5_K: exact_q5_k}
+              synth.Q2_K: exact_q2_k, synth.Q5_K: exact_q5_k, synth.Q3_K: exact_q3_k, synth.Q8_K: exact_q8_k,
+              synth.IQ4_NL: exact_iq4_nl, synth.IQ4_XS: exact_iq4_xs}
 F16_FIELDS = {synth.Q4_0: (0,), synth.Q4_1: (0, 2), synth.Q5_0: (0,), synth.Q5_1: (0, 2), synth.Q2_K: (80, 82),
-              synth.Q5_K: (0, 2)}
+              synth.Q5_K: (0, 2), synth.Q3_K: (108,), synth.Q8_K: (), synth.IQ4_NL: (0,), synth.IQ4_XS: (0,)}
+# Q8_K keeps its scale as a float32: subnormal, smallest normal, the largest whose products stay finite, odd significands, signed zeros
+F32_EXTREMES = [0x00000001, 0x007FFFFF, 0x00800000, 0x7BFFFFFF, 0xBF800001, 0x3F800000, 0x00000000, 0x80000000,
+                0x3DCCCCCD, 0xC2F6E979]
 
 
 def adversarial_blocks(qtype, rng):
@@ -322,7 +386,8 @@ def make_more_quant_blocks():
     out = {}
     rng = np.random.default_rng(20240611)
     names = {synth.Q4_0: "q4_0", synth.Q4_1: "q4_1", synth.Q5_0: "q5_0", synth.Q5_1: "q5_1", synth.Q2_K: "q2_k",
-             synth.Q5_K: "q5_k"}
+             synth.Q5_K: "q5_k", synth.Q3_K: "q3_k", synth.Q8_K: "q8_k", synth.IQ4_NL: "iq4_nl",
+             synth.IQ4_XS: "iq4_xs"}
     f16b = lambda bits: [bits & 0xFF, bits >> 8]  # noqa: E731
     extremes = [f16b(0x0001), f16b(0x03FF), f16b(0x0400), f16b(0x7BFF), f16b(0xBC01), f16b(0x3C00), f16b(0x0000),
                 f16b(0x8000)]
@@ -333,11 +398,15 @@ def make_more_quant_blocks():
             b = rng.integers(0, 256, size=bb, dtype=np.uint8)
             for n, off in enumerate(F16_FIELDS[qtype]):
                 b[off:off + 2] = extremes[(i + 3 * n) % len(extremes)]
+            if qtype == synth.Q8_K:
+                b[0:4] = np.array([F32_EXTREMES[i]], dtype="<u4").view(np.uint8)
             blocks.append(b[None, :])
         for fill in (0x00, 0xFF, 0x0F, 0xF0, 0x55, 0xAA):
             b = np.full(bb, fill, dtype=np.uint8)
             for n, off in enumerate(F16_FIELDS[qtype]):
                 b[off:off + 2] = np.array([0.25 / (n + 1)], dtype=np.float16).view(np.uint8)
+            if qtype == synth.Q8_K:
+                b[0:4] = np.array([F32_EXTREMES[8 + (fill & 1)]], dtype="<u4").view(np.uint8)
             blocks.append(b[None, :])
         blocks = np.concatenate(blocks)
         vals = np.array([EXACT_MORE[qtype](blk) for blk in blocks], dtype=np.float32).reshape(-1)

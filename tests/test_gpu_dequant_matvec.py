@@ -49,7 +49,7 @@ def test_dequant_full_size_checksum(hip):
 def test_dequant_errors(hip):
     buf = hip.alloc(1024)
     with pytest.raises(runtime.SknError) as e:
-        hip.dequant(11, buf, 256, buf)  # Q3_K: in the size table, not computed with
+        hip.dequant(16, buf, 256, buf)  # IQ2_XXS: in the size table, not computed with
     assert e.value.code == runtime.ERR_TYPE
     with pytest.raises(runtime.SknError) as e:
         hip.dequant(Q4_K, buf, 100, buf)
@@ -126,7 +126,7 @@ def test_matvec_errors_and_empty(hip):
     assert e.value.code == runtime.ERR_SHAPE
     assert "is not a multiple of block size (256)" in e.value.message
     with pytest.raises(runtime.SknError) as e:
-        hip.matvec_q(11, buf, 4, 256, buf, buf)
+        hip.matvec_q(16, buf, 4, 256, buf, buf)
     assert e.value.code == runtime.ERR_TYPE
     with pytest.raises(runtime.SknError) as e:
         hip.matvec_q(Q4_K, buf, 4, 256, None, buf)

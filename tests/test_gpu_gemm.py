@@ -121,7 +121,7 @@ def test_gemm_errors(hip):
         hip.gemm_q(Q4_K, buf, 4, 200, buf, 2, buf)
     assert e.value.code == runtime.ERR_SHAPE
     with pytest.raises(runtime.SknError) as e:
-        hip.gemm_q(11, buf, 4, 256, buf, 2, buf)
+        hip.gemm_q(16, buf, 4, 256, buf, 2, buf)
     assert e.value.code == runtime.ERR_TYPE
     with pytest.raises(runtime.SknError) as e:
         hip.gemm_q(Q4_K, None, 4, 256, buf, 2, buf)

@@ -1,4 +1,4 @@
-"""GPU parity for the further ggml formats (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K, F16, BF16, F32) through the C ABI:
+"""GPU parity for the further ggml formats (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, F16, BF16, F32) through the C ABI:
 dequantization bit for bit against the CPU oracle, matvec and GEMM within the 1e-3 criterion."""
 import numpy as np
 import pytest
@@ -8,7 +8,8 @@ from skainet_amd import runtime, synth
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
-MORE = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (1, "f16"), (30, "bf16"), (0, "f32")]
+MORE = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (11, "q3_k"), (15, "q8_k"),
+        (20, "iq4_nl"), (23, "iq4_xs"), (1, "f16"), (30, "bf16"), (0, "f32")]
 
 
 @pytest.mark.parametrize("qtype,name", MORE)
@@ -28,8 +29,9 @@ def test_dequant_random_bytes_bit_exact(hip, qtype, name):
     """Uniform random payload bytes (all scale / min / bit patterns), finite fp16 fields."""
     be, bb = synth.BLOCK[qtype]
     raw = np.random.default_rng(qtype).integers(0, 256, size=4096 * bb, dtype=np.uint8)
-    for off in {2: (0,), 3: (0, 2), 6: (0,), 7: (0, 2), 10: (80, 82), 13: (0, 2)}[qtype]:
-        raw.reshape(-1, bb)[:, off + 1] &= 0x7B
+    for off in {2: (0,), 3: (0, 2), 6: (0,), 7: (0, 2), 10: (80, 82), 13: (0, 2), 11: (108,), 15: (2,), 20: (0,),
+                23: (0,)}[qtype]:
+        raw.reshape(-1, bb)[:, off + 1] &= 0x7B  # (Q8_K: the top byte of its float32 scale)
     want = oracle_c.dequant(qtype, raw)
     out = hip.alloc(4 * want.size)
     hip.dequant(qtype, hip.to_device(raw), want.size, out)
@@ -78,7 +80,7 @@ def test_gemm_vs_oracle(hip, qtype, name):
 
 def test_unknown_types_are_rejected(hip):
     buf = hip.alloc(4096)
-    for qtype in (9, 11, 15, 16, 4):  # in the size table but not computed with / not in the table at all
+    for qtype in (9, 16, 22, 4, 36):  # in the size table but not computed with / not in the table at all
         with pytest.raises(runtime.SknError) as e:
             hip.matvec_q(qtype, buf, 1, 256, buf, buf)
         assert e.value.code == runtime.ERR_TYPE

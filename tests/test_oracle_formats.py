@@ -183,11 +183,11 @@ def test_q8_0_known_answers():
 
 def test_dequant_rejects_bad_arguments():
     with pytest.raises(ValueError):
-        oracle_c.dequant(11, np.zeros(110, dtype=np.uint8), 256)  # Q3_K: in the size table, not computed with
+        oracle_c.dequant(16, np.zeros(66, dtype=np.uint8), 256)  # IQ2_XXS: in the size table, not computed with
     with pytest.raises(ValueError):
         oracle_c.dequant(Q4_K, np.zeros(144, dtype=np.uint8), 100)
     with pytest.raises(ValueError):
-        oracle_np.dequant(11, np.zeros(110, dtype=np.uint8))
+        oracle_np.dequant(16, np.zeros(66, dtype=np.uint8))
 
 
 def test_synthetic_generator_statistics():

@@ -1,5 +1,5 @@
 """CPU: the further ggml block formats of the reference's size table (Constants.kt:58-90) -- Q4_0, Q4_1, Q5_0, Q5_1,
-Q2_K, Q5_K, F16, BF16.  The reference holds only their sizes; the packing is the published ggml definition
+Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, F16, BF16.  The reference holds only their sizes; the packing is the published ggml definition
 (parity unpinned by the reference).  Pinned here by hand-built single blocks whose answers are known in closed
 form (every field tagged so that a wrong element order, bit position or scale index shows), and by bit-for-bit
 agreement of the two independently written oracles on random bytes."""
@@ -10,9 +10,12 @@ from oracle import oracle_c, oracle_np
 from skainet_amd import synth
 
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
+Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
 F32, F16, BF16 = 0, 1, 30
 MORE = [(Q4_0, "q4_0"), (Q4_1, "q4_1"), (Q5_0, "q5_0"), (Q5_1, "q5_1"), (Q2_K, "q2_k"), (Q5_K, "q5_k"),
+        (Q3_K, "q3_k"), (Q8_K, "q8_k"), (IQ4_NL, "iq4_nl"), (IQ4_XS, "iq4_xs"),
         (F16, "f16"), (BF16, "bf16"), (F32, "f32")]
+IQ4 = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float64)
 
 
 def f16b(v):
@@ -38,8 +41,9 @@ def test_oracles_match_golden_blocks(golden_dir, qtype, name):
 
 
 def test_sizes_match_reference_table():
-    # literal numbers of reference gguf/.../Constants.kt:60-68,70 and the enum ids :16-19,23,26
+    # literal numbers of reference gguf/.../Constants.kt:60-90 and the enum ids :16-48
     want = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176),
+            Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136),
             F16: (1, 2), BF16: (1, 2), F32: (1, 4)}
     for t, sz in want.items():
         assert oracle_c.type_sizes(t) == sz
@@ -56,8 +60,9 @@ def test_oracles_agree_bitwise_on_random_blocks(qtype, name):
         raw = synth.weight(qtype, 4, 64, seed=3)
     else:
         # keep the fp16 fields finite (exponent field 31 is inf / nan)
-        for off in {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q2_K: (80, 82), Q5_K: (0, 2)}[qtype]:
-            raw.reshape(-1, bb)[:, off + 1] &= 0x7B
+        for off in {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q2_K: (80, 82), Q5_K: (0, 2), Q3_K: (108,),
+                    Q8_K: (2,), IQ4_NL: (0,), IQ4_XS: (0,)}[qtype]:
+            raw.reshape(-1, bb)[:, off + 1] &= 0x7B  # (Q8_K: the top byte of its float32 scale)
     both(qtype, raw)
 
 
@@ -132,6 +137,86 @@ def test_q5_k_fifth_bit_and_layout():
     y = both(Q5_K, np.concatenate([f16b(2.0), f16b(1.0), synth.pack_q4k_scales(sc, mn)[0], np.zeros(32, np.uint8),
                                    np.full(128, 0x11, np.uint8)]))
     assert np.array_equal(y.reshape(8, 32)[:, 0], 2.0 * sc[0] * 1.0 - 1.0 * mn[0])
+
+
+def _q3k_block(scales6, hmask, qs, d):
+    """Pack sixteen 6-bit scale codes the way ggml stores them in twelve bytes."""
+    s = np.zeros(12, dtype=np.uint8)
+    for i, v in enumerate(scales6):
+        if i < 8:
+            s[i] |= v & 15
+        else:
+            s[i - 8] |= (v & 15) << 4
+        s[8 + i % 4] |= (v >> 4) << (2 * (i // 4))
+    return np.concatenate([hmask, qs, s, f16b(d)]).astype(np.uint8)
+
+
+def test_q3_k_scales_high_bit_and_layout():
+    e = np.arange(256)
+    n, j, l = e // 128, (e % 128) // 32, e % 32
+    group = 8 * n + 2 * j + (l >= 16)
+    # every scale code distinct and above 32 (so both the low nibble and the two high bits matter); q = 1 with the
+    # high-bit mask all set: y = d * (code - 32)
+    codes = np.array([33, 47, 48, 63, 34, 50, 35, 62, 36, 44, 49, 61, 37, 40, 52, 60])
+    y = both(Q3_K, _q3k_block(codes, np.full(32, 0xFF, np.uint8), np.full(64, 0x55, np.uint8), 0.5))
+    assert np.array_equal(y, 0.5 * (codes[group] - 32))
+    # codes below 32 are negative scales
+    low = np.arange(16)
+    y = both(Q3_K, _q3k_block(low, np.full(32, 0xFF, np.uint8), np.full(64, 0x55, np.uint8), 1.0))
+    assert np.array_equal(y, (low[group] - 32.0))
+    # a cleared mask bit subtracts 4: bit (4n + j) of hmask[l]
+    for bit in range(8):
+        y = both(Q3_K, _q3k_block(np.full(16, 33), np.full(32, 1 << bit, np.uint8), np.full(64, 0xFF, np.uint8), 1.0))
+        assert np.array_equal(y, np.where(4 * n + j == bit, 3.0, -1.0)), bit
+    hm = np.zeros(32, np.uint8)
+    hm[9] = 0xFF
+    y = both(Q3_K, _q3k_block(np.full(16, 33), hm, np.zeros(64, np.uint8), 1.0))
+    assert np.array_equal(np.nonzero(y == 0.0)[0], np.arange(8) * 32 + 9)
+    # distinct quant bytes: element reads byte 32n + l, bit pair j
+    qs = (np.arange(64) * 7 % 256).astype(np.uint8)
+    y = both(Q3_K, _q3k_block(np.full(16, 33), np.full(32, 0xFF, np.uint8), qs, 1.0))
+    assert np.array_equal(y, (qs[32 * n + l] >> (2 * j)) & 3)
+
+
+def test_q8_k_float_scale_and_ignored_sums():
+    qs = np.arange(-128, 128, dtype=np.int8)
+    d = np.array([0.1], dtype=np.float32)  # not representable in fp16: the scale really is a float32
+    blk = np.concatenate([d.view(np.uint8), qs.view(np.uint8), np.zeros(32, np.uint8)])
+    y = both(Q8_K, blk)
+    assert np.array_equal(y, (d[0].astype(np.float64) * qs).astype(np.float32))
+    blk[260:292] = 0xFF  # the trailing block sums do not change the values
+    assert np.array_equal(both(Q8_K, blk), y)
+
+
+def test_iq4_table_and_element_order():
+    qs = np.array([j | ((15 - j) << 4) for j in range(16)], dtype=np.uint8)
+    y = both(IQ4_NL, np.concatenate([f16b(2.0), qs]))
+    assert np.array_equal(y[:16], 2.0 * IQ4)         # low nibbles first: the table in order
+    assert np.array_equal(y[16:], 2.0 * IQ4[::-1])   # then high nibbles
+    assert np.all(np.diff(IQ4) > 0) and IQ4.sum() == -94.0  # the published table: increasing, known checksum
+
+
+def test_iq4_xs_scales_and_layout():
+    # sub-block ib gets 6-bit code ls(ib): low nibble from scales_l, high two bits from scales_h
+    codes = np.array([33, 47, 0, 63, 32, 16, 50, 31])
+    sl = np.zeros(4, np.uint8)
+    sh = 0
+    for ib, v in enumerate(codes):
+        sl[ib // 2] |= (v & 15) << (4 * (ib % 2))
+        sh |= (v >> 4) << (2 * ib)
+    qs = np.tile(np.array([j | ((15 - j) << 4) for j in range(16)], dtype=np.uint8), 8)
+    blk = np.concatenate([f16b(0.25), np.array([sh & 0xFF, sh >> 8], np.uint8), sl, qs])
+    y = both(IQ4_XS, blk).reshape(8, 32)
+    for ib in range(8):
+        assert np.array_equal(y[ib, :16], 0.25 * (codes[ib] - 32) * IQ4), ib
+        assert np.array_equal(y[ib, 16:], 0.25 * (codes[ib] - 32) * IQ4[::-1]), ib
+    # distinct bytes: sub-block ib reads qs[16 ib .. 16 ib + 15]
+    qs = np.arange(128, dtype=np.uint8)
+    blk = np.concatenate([f16b(1.0), np.array([0, 0], np.uint8), np.full(4, 0x11, np.uint8), qs])
+    y = both(IQ4_XS, blk).reshape(8, 32)
+    for ib in range(8):
+        b = qs[16 * ib:16 * ib + 16]
+        assert np.array_equal(y[ib], -31.0 * np.concatenate([IQ4[b & 15], IQ4[b >> 4]])), ib
 
 
 def test_dense_types():
