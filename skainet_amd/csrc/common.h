@@ -28,7 +28,7 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_q4k = 0;
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
@@ -106,6 +106,14 @@ static inline bool skn_is_quant(int t) {
 }
 int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out);
 int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y);
+// Q4_K GEMM of one activation matrix [m, k] (bf16, or fp32 rounded to bf16 on the way in) against up to three
+// weight matrices [n_i, k] in one launch: c_i[m, n_i] = a * w_i^T.
+struct skn_gemm_seg {
+    const void* w;
+    int n;
+    float* c;
+};
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const void* a_dev, int a_is_f32, int m);
 int skn_dequant_hilo(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
 int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
 

@@ -507,34 +507,57 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
+        // Q4_K weights take the fp32 rows as they are (rounded to bf16 inside the GEMM's preparation pass)
+        const bool q4k_attn = L.type_attn == SKN_TYPE_Q4_K && H <= 16384 && ctx->opt_gemm_q4k != 1;
+        const bool q4k_ffn = L.type_ffn == SKN_TYPE_Q4_K && H <= 16384 && F <= 16384 && ctx->opt_gemm_q4k != 1;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
         skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
         SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wq, H, H, m->pb16, T, m->pq));
-        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wk, H, H, m->pb16, T, m->pk));
-        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wv, H, H, m->pb16, T, m->pv));
+        if (q4k_attn) {  // one activation preparation and one launch for the three projections
+            const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq}, {L.wk, H, m->pk}, {L.wv, H, m->pv}};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, m->pxn, 1, T));
+        } else {
+            SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
+            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wq, H, H, m->pb16, T, m->pq));
+            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wk, H, H, m->pb16, T, m->pk));
+            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wv, H, H, m->pb16, T, m->pv));
+        }
         skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
                    kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
                    kv->page_tokens, log2f(c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
         SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
-        SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
-        SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
+        if (q4k_attn) {
+            const skn_gemm_seg wo = {L.wo, H, m->pproj};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, &wo, 1, H, m->patt, 1, T));
+        } else {
+            SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
+            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
+        }
         skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
                    (int64_t)T * H);
         SKN_LAUNCH_CHECK(ctx);
         skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
         SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_gate, F, H, m->pb16, T, m->pgate));
-        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_up, F, H, m->pb16, T, m->pup));
+        if (q4k_ffn) {
+            const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pgate}, {L.w_up, F, m->pup}};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, m->pxn, 1, T));
+        } else {
+            SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
+            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_gate, F, H, m->pb16, T, m->pgate));
+            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_up, F, H, m->pb16, T, m->pup));
+        }
         skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
                    (const float*)m->pup, m->pmid, (int64_t)T * F);
         SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
-        SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_down, H, F, m->pb16, T, m->pproj));
+        if (q4k_ffn) {
+            const skn_gemm_seg down = {L.w_down, H, m->pproj};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, m->pmid, 1, T));
+        } else {
+            SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
+            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_down, H, F, m->pb16, T, m->pproj));
+        }
         skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
                    (int64_t)T * H);
         SKN_LAUNCH_CHECK(ctx);

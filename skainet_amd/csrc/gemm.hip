@@ -15,6 +15,8 @@
 //     applied to the fp32 partial sum of each superblock.
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -419,6 +421,393 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
         store_tile(tot[i], c, n, m0 + wm * 32 * MT + 32 * i, n0 + wn * 32, m, n, inv_scale, lane);
 }
 
+// ---- Q4_K path, second form: every wavefront loads its matrix-core operands itself ------------------------
+// Workgroup of eight wavefronts, tile (64 MT) x 64.  The tile is divided in two along m; along k it is not
+// divided spatially but by superblock: wavefront (mh, kq) computes rows [32 MT mh, 32 MT (mh + 1)) x all 64
+// columns for superblocks kq, kq + 4, ..., and the four partial tiles of each half are added through LDS at
+// the end.  The activations are prepared in "fragment order": for a block of 32 rows, a 64-element chunk and a
+// k-step s, the 64 x 16 bytes that the 64 lanes feed to one matrix instruction are contiguous (lane l = 32 h + r
+// holds row r and the eight elements that nibble dword 4 h + s of the chunk unpacks to), so a fragment is one
+// coalesced 1 KiB load and never passes through LDS.  The weights of four superblocks (576 contiguous bytes of
+// each of the 64 rows) are copied from global memory straight into LDS once per group of four superblocks --
+// the only barrier in the loop -- from where each lane picks the 16 bytes of its row and k-step quartet.
+// Operands are the exact integers of the first form.  One set of accumulators: see the kernel.
+constexpr int kWPitch = 576;  // LDS pitch of a weight row: the 144 bytes of four superblocks
+
+// Activations bf16 [m, k] -> fragment order.  One workgroup per R rows of the padded row count (rows >= m are
+// zero), one wavefront per row: the row's largest magnitude fixes its power-of-two scale, then the row is
+// converted 4096 elements at a time into LDS, laid out so that the copy to global memory writes runs of 16 R
+// bytes (the same sixteen bytes of R neighbouring rows).
+// afrag: [row block][chunk][k-step][lane] x 8 halves.  sfrag: [row block][superblock][lane] x 8 halves: the eight
+// sub-block sums of row r times 2^-12 as fp16 pairs, lanes 0..31 the "hi" parts, lanes 32..63 the "lo" parts.
+// IN = uint16_t: bf16 activations; IN = float: fp32 activations, rounded to bf16 (nearest even) on the way in.
+template <typename IN>
+__device__ __forceinline__ void load_bf16x4(const IN* p, uint32_t& lo, uint32_t& hi);
+template <>
+__device__ __forceinline__ void load_bf16x4<uint16_t>(const uint16_t* p, uint32_t& lo, uint32_t& hi) {
+    const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+    lo = v.x, hi = v.y;
+}
+template <>
+__device__ __forceinline__ void load_bf16x4<float>(const float* p, uint32_t& lo, uint32_t& hi) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(p);
+    auto rne = [](uint32_t u) { return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16; };
+    lo = rne(v.x) | (rne(v.y) << 16);
+    hi = rne(v.z) | (rne(v.w) << 16);
+}
+
+template <int R, typename IN>
+__global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const IN* __restrict__ a, _Float16* __restrict__ afrag,
+                                                            float* __restrict__ inv_scale, _Float16* __restrict__ sfrag,
+                                                            int m, int k) {
+    __shared__ __align__(16) u32x4 stage[512 * R];  // [chunk 64][k-step 4][half 2][row R] sixteen-byte pieces
+    const int tid = threadIdx.x, lane = tid & 63, r8 = tid >> 6;
+    const int row = blockIdx.x * R + r8;
+    const bool real = row < m;
+    const IN* ar = a + (size_t)(real ? row : 0) * k;
+    const int nch = k >> 6, nb = k >> 8;
+    auto widen = [](uint32_t pair, int which) { return __uint_as_float(which ? pair & 0xFFFF0000u : pair << 16); };
+
+    // pass 1: the row's largest finite magnitude
+    float mx = 0.f;
+    for (int i0 = 0; i0 < (k >> 3); i0 += 512) {  // eight loads in flight per lane
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const IN* src = ar + 8 * min(i0 + lane + 64 * j, (k >> 3) - 1);
+            uint32_t w0, w1, w2, w3;
+            load_bf16x4<IN>(src, w0, w1);
+            load_bf16x4<IN>(src + 4, w2, w3);
+            v[j] = u32x4{w0, w1, w2, w3};
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                const float f = fabsf(widen(v[j][x >> 1], x & 1));
+                if (f == f && f < INFINITY) mx = fmaxf(mx, f);
+            }
+    }
+    mx = wave_max(mx);
+    if (!real) mx = 0.f;
+    int e = 9;  // a zero row keeps scale 1
+    if (mx > 0.f) e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+    e = max(e, -100);  // (a subnormal maximum: exponent field 0)
+    const float scale = real ? __uint_as_float((uint32_t)(127 + 9 - e) << 23) : 0.f;
+    if (lane == 0 && real) inv_scale[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+    const int mb = row >> 5, r = row & 31;
+
+    // pass 2: slabs of 4096 elements = 64 chunks = 512 tasks (chunk c, nibble dword dw), eight per lane
+    for (int k0 = 0; k0 < k; k0 += 4096) {
+        const int tasks = min(4096, k - k0) >> 3;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int task = lane + 64 * j;
+            const int c = task >> 3, dw = task & 7;
+            uint2 lo = make_uint2(0u, 0u), hi = lo;
+            if (task < tasks) {
+                load_bf16x4<IN>(ar + k0 + 64 * c + 4 * dw, lo.x, lo.y);
+                load_bf16x4<IN>(ar + k0 + 64 * c + 32 + 4 * dw, hi.x, hi.y);
+            }
+            _Float16 l[4], u[4];
+            l[0] = (_Float16)(widen(lo.x, 0) * scale), l[1] = (_Float16)(widen(lo.x, 1) * scale);
+            l[2] = (_Float16)(widen(lo.y, 0) * scale), l[3] = (_Float16)(widen(lo.y, 1) * scale);
+            u[0] = (_Float16)(widen(hi.x, 0) * scale), u[1] = (_Float16)(widen(hi.x, 1) * scale);
+            u[2] = (_Float16)(widen(hi.y, 0) * scale), u[3] = (_Float16)(widen(hi.y, 1) * scale);
+            float sl = ((float)l[0] + (float)l[1]) + ((float)l[2] + (float)l[3]);
+            float su = ((float)u[0] + (float)u[1]) + ((float)u[2] + (float)u[3]);
+            // totals over the eight lanes of the chunk
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0xB1, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0xB1, 0xF, 0xF, true));
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x4E, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x4E, 0xF, 0xF, true));
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x141, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x141, 0xF, 0xF, true));
+            half8_t o;
+            o[0] = l[0], o[1] = l[2], o[2] = u[0], o[3] = u[2], o[4] = l[1], o[5] = l[3], o[6] = u[1], o[7] = u[3];
+            const int h = dw >> 2, s = dw & 3;
+            stage[((c * 4 + s) * 2 + h) * R + r8] = __builtin_bit_cast(u32x4, o);
+            if (dw == 0 && task < tasks) {
+                sl *= 0x1p-12f, su *= 0x1p-12f;
+                const _Float16 h0 = (_Float16)sl, h1 = (_Float16)su;
+                const int cg = (k0 >> 6) + c;
+                _Float16* sf = sfrag + ((size_t)mb * nb + (cg >> 2)) * 512 + 2 * (cg & 3);
+                half2_t vh = {h0, h1}, vl = {(_Float16)(sl - (float)h0), (_Float16)(su - (float)h1)};
+                *reinterpret_cast<half2_t*>(sf + r * 8) = vh;
+                *reinterpret_cast<half2_t*>(sf + (32 + r) * 8) = vl;
+            }
+        }
+        __syncthreads();
+        // piece i = ((c 4 + s) 2 + h) R + row: R consecutive lanes write 16 R contiguous bytes
+        u32x4* out = reinterpret_cast<u32x4*>(afrag) + ((size_t)mb * nch + (k0 >> 6)) * 256 + (blockIdx.x % (32 / R)) * R;
+#pragma unroll
+        for (int it = 0; it < 8; it++) {
+            const int i = tid + 64 * R * it, csh = i / R;
+            if (csh < tasks) out[(size_t)(csh >> 1) * 64 + (csh & 1) * 32 + (i % R)] = stage[i];
+        }
+        __syncthreads();
+    }
+}
+
+// up to three weight matrices [n_i, k] multiplied by the same activations in one launch
+struct Q4kFragSegs {
+    const uint8_t* w[3];
+    float* c[3];
+    int n[3];
+    int tile0[3];  // first column tile of each matrix (unused entries: n_tiles)
+    int n_tiles;
+};
+
+// Accumulators: acc holds the running sum of a column in units of cs = d * 2^24 of the latest superblock whose d
+// is not zero.  Entering a superblock it is rescaled by cs_old / cs_new (a relative error of 2^-23 per
+// superblock, against the 1e-3 asked of the op); the superblock's integer products then add to it as they come
+// out of the matrix core, and so does the "- dmin * m_j" term: one more sixteen-deep product per tile between
+// the activation sub-block sums (fp16 hi | lo) and -(dmin / cs) * m_j * 2^12, itself split into an fp16 pair.
+template <int MT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const Q4kFragSegs segs,
+                          const float* __restrict__ inv_scale, int m, int k) {
+    constexpr int kWBuf = kBN * kWPitch;
+    extern __shared__ __align__(16) uint8_t lds[];  // max(2 kWBuf, MT x 48 KiB) bytes
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kq = wave & 3, mh = wave >> 2;
+    const int h = lane >> 5, r = lane & 31;
+    const int nb = k >> 8, nch = k >> 6, groups = (nb + 3) >> 2;
+    // tile -> (row tile, weight matrix, column tile): the column tiles of up to three matrices sharing the
+    // activations are laid side by side
+    const int mt = blockIdx.x / segs.n_tiles, tn = blockIdx.x - mt * segs.n_tiles;
+    const int seg = tn >= segs.tile0[2] ? 2 : (tn >= segs.tile0[1] ? 1 : 0);
+    const uint8_t* __restrict__ w = segs.w[seg];
+    float* __restrict__ c = segs.c[seg];
+    const int n = segs.n[seg];
+    const int mb0 = (2 * mt + mh) * MT, n0 = (tn - segs.tile0[seg]) * kBN;
+
+    // Weight staging, global memory straight into LDS: a wavefront-wide load fills 64 sixteen-byte slots
+    // i * 64 + lane; slot P holds piece P % 36 of tile row P / 36 (36 pieces = the 576 bytes of four
+    // superblocks).  The 36 loads of a group are dealt round the eight wavefronts.  Completion is waited for
+    // with the vector-memory counter before the barrier that publishes the buffer.
+    auto wfetch = [&](int g, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int x = 0; x < 5; x++) {
+            const int i = wave + 8 * x;
+            if (i < 36) {
+                const int p = i * 64 + lane, row = p / 36, col = p - 36 * row;
+                const int off = min(g * 576 + col * 16, nb * 144 - 16);  // (a short last group repeats the row's last piece)
+                const uint8_t* src = w + (size_t)min(n0 + row, n - 1) * nb * 144 + off;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                                 (__attribute__((address_space(3))) void*)(lds + buf * kWBuf + i * 1024), 16, 0, 0);
+            }
+        }
+    };
+
+    const u32x4* ap[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) ap[i] = afrag + (size_t)(mb0 + i) * nch * 256 + lane;
+    // activation fragments: a ring of eight k-steps; the slot of step t is refilled with step t + 8 as soon as
+    // the matrix instructions of step t are issued
+    u32x4 a[8][MT];
+    auto afetch = [&](int step, int slot) __attribute__((always_inline)) {  // step: 16 per superblock, absolute
+#pragma unroll
+        for (int i = 0; i < MT; i++) a[slot][i] = ap[i][(size_t)step * 64];
+    };
+    float16_t acc[MT][2];
+    float cs[2] = {1.f, 1.f};
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
+
+    wfetch(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (kq < nb) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) afetch(16 * kq + s, s);
+    }
+    asm volatile("s_barrier" ::: "memory");
+
+    for (int g = 0; g < groups; g++) {
+        const int sb = 4 * g + kq;
+        if (g + 1 < groups) wfetch(g + 1, (g + 1) & 1);
+        if (sb < nb) {
+            // this lane's weight rows (one per 32-column tile): the 144 bytes of superblock sb
+            const uint8_t* wl = lds + (g & 1) * kWBuf + r * kWPitch + kq * 144;
+            constexpr int kTile = 32 * kWPitch;  // the lane's row of the second 32-column tile
+            u32x4 hd[2], sf[MT];
+#pragma unroll
+            for (int j = 0; j < 2; j++) hd[j] = *reinterpret_cast<const u32x4*>(wl + j * kTile);
+            auto sbyte = [&](int j, int i) { return (hd[j][1 + (i >> 2)] >> (8 * (i & 3))) & 0xFFu; };
+            auto scale_of = [&](int j, int s) {
+                return s < 4 ? (int)(sbyte(j, s) & 63) : (int)((sbyte(j, s + 4) & 0x0F) | ((sbyte(j, s - 4) >> 6) << 4));
+            };
+            auto min_of = [&](int j, int s) {
+                return s < 4 ? (int)(sbyte(j, s + 4) & 63) : (int)((sbyte(j, s + 4) >> 4) | ((sbyte(j, s) >> 6) << 4));
+            };
+            float min_unit[2], live[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const uint32_t dw0 = hd[j][0];
+                const half2_t dd = __builtin_bit_cast(half2_t, dw0);
+                const float ds = (float)dd.x * 16777216.0f;
+                live[j] = ds != 0.f ? 1.f : 0.f;  // (a zero d: the column keeps its unit and the products are zeroed)
+                const float cs_new = ds != 0.f ? ds : cs[j];
+                const float inv = 1.0f / cs_new, ratio = cs[j] * inv;
+                min_unit[j] = -(float)dd.y * inv * 4096.0f;
+                cs[j] = cs_new;
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio;
+            }
+            // Sixteen k-steps, software-pipelined: the weight fragments of step t + 1 are unpacked (vector ALU)
+            // while the matrix instructions of step t run.
+            u32x4 q[2], qn[2];
+            half2_t mul_lo[2], mul_hi[2];
+            half8_t fb[2], fbn[2];
+            auto load_q = [&](int cc, u32x4* dst) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) dst[j] = *reinterpret_cast<const u32x4*>(wl + j * kTile + 16 + 32 * cc + 16 * h);
+            };
+            auto scales = [&](int cc) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const _Float16 ml = (_Float16)((float)scale_of(j, 2 * cc) * live[j]);
+                    const _Float16 mh2 = (_Float16)((float)scale_of(j, 2 * cc + 1) * (0.0625f * live[j]));
+                    mul_lo[j] = half2_t{ml, ml};
+                    mul_hi[j] = half2_t{mh2, mh2};
+                }
+            };
+            auto decode = [&](int s, half8_t* dst) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const uint32_t qq = q[j][s], q8 = qq >> 8;
+                    const uint32_t l02 = qq & 0x000F000Fu, h02 = qq & 0x00F000F0u;
+                    const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
+                    u32x4 o;
+                    o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo[j]);
+                    o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi[j]);
+                    o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo[j]);
+                    o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi[j]);
+                    dst[j] = __builtin_bit_cast(half8_t, o);
+                }
+            };
+            load_q(0, q);
+            scales(0);
+            decode(0, fbn);
+            auto chunk = [&](auto cc_const) __attribute__((always_inline)) {
+                constexpr int cc = decltype(cc_const)::value;
+                if (cc == 2) {
+#pragma unroll
+                    for (int i = 0; i < MT; i++) sf[i] = sfrag[((size_t)(mb0 + i) * nb + sb) * 64 + lane];
+                }
+                if (cc < 3) load_q(cc + 1, qn);
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    fb[0] = fbn[0], fb[1] = fbn[1];
+                    if (s < 3) {
+                        decode(s + 1, fbn);
+                    } else if (cc < 3) {
+                        q[0] = qn[0], q[1] = qn[1];
+                        scales(cc + 1);
+                        decode(0, fbn);
+                    }
+                    const int step = 4 * cc + s, slot = step & 7;
+#pragma unroll
+                    for (int i = 0; i < MT; i++) {
+                        const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                        for (int j = 0; j < 2; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[j], acc[i][j], 0, 0, 0);
+                    }
+                    // refill the slot: eight steps ahead in this superblock, or the first half of superblock sb + 4
+                    // (past the end: a repeat of the last superblock, unused)
+                    afetch(step < 8 ? 16 * sb + step + 8 : 16 * min(sb + 4, nb - 1) + step - 8, slot);
+                }
+            };
+            chunk(std::integral_constant<int, 0>{});
+            chunk(std::integral_constant<int, 1>{});
+            chunk(std::integral_constant<int, 2>{});
+            chunk(std::integral_constant<int, 3>{});
+            // the "- dmin * m" term of the superblock
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                half8_t vh, vl;
+#pragma unroll
+                for (int s = 0; s < 8; s++) {
+                    const float v = fminf(fmaxf(min_unit[j] * (float)min_of(j, s), -60000.f), 60000.f);
+                    vh[s] = (_Float16)v;
+                    vl[s] = (_Float16)(v - (float)vh[s]);
+                }
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    const half8_t fs = __builtin_bit_cast(half8_t, sf[i]);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fs, vh, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fs, vl, acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+        // a bare barrier: a full __syncthreads() would also wait for the fragment loads in flight
+        // The next group's weights were requested before this superblock's 16 MT fragment loads, and loads
+        // complete in order: once all but the newest 8 MT have landed, so have they.
+        if (sb < nb) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * MT) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+    // back to true units
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[i][j][x] *= cs[j];
+
+    // add the four partial tiles of each half: tile t = 2 i + j belongs to wavefront kq = t % 4 of its half, the
+    // other three hand theirs over
+    float* red = reinterpret_cast<float*>(lds);
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = 2 * i + j, owner = t & 3;
+            if (kq != owner) {
+                float* dst = red + ((mh * 2 * MT + t) * 3 + ((kq - owner + 4) & 3) - 1) * 1024 + lane;
+#pragma unroll
+                for (int x = 0; x < 16; x++) dst[64 * x] = acc[i][j][x];
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = 2 * i + j;
+            if (kq == (t & 3)) {
+                float16_t sum = acc[i][j];
+#pragma unroll
+                for (int o = 0; o < 3; o++)
+#pragma unroll
+                    for (int x = 0; x < 16; x++) sum[x] += red[((mh * 2 * MT + t) * 3 + o) * 1024 + 64 * x + lane];
+                store_tile(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, inv_scale, lane);
+            }
+        }
+}
+
+// the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in once
+template <int MT>
+int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfrag, const Q4kFragSegs& segs, const float* isc,
+                int m, int k) {
+    constexpr int kLds = 2 * kBN * kWPitch > MT * 49152 ? 2 * kBN * kWPitch : MT * 49152;
+    static bool opted = false;
+    if (!opted) {
+        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        opted = true;
+    }
+    skn_launch(ctx, gemm_q4k_frag_kernel<MT>, dim3(m_tiles * segs.n_tiles), dim3(512), kLds, afrag, sfrag, segs, isc, m, k);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
 int gemm_workspace(skn_ctx* ctx, size_t bytes, uint8_t** out) {
     if (bytes > ctx->gemm_ws_bytes) {
@@ -441,6 +830,42 @@ inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
 
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const void* a_dev, int a_is_f32, int m) {
+    SKN_REQUIRE(ctx, nseg >= 1 && nseg <= 3 && m > 0 && k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_ARG,
+                "Q4_K GEMM: bad segment count or shape");
+    Q4kFragSegs fs;
+    int tiles = 0;
+    for (int i = 0; i < 3; i++) {
+        const skn_gemm_seg& s = segs[i < nseg ? i : nseg - 1];
+        SKN_REQUIRE(ctx, s.w && s.c && s.n > 0 && ((uintptr_t)s.w & 15) == 0, SKN_ERR_ARG,
+                    "Q4_K GEMM: weights must be non-null and 16-byte aligned");
+        fs.w[i] = (const uint8_t*)s.w, fs.c[i] = s.c, fs.n[i] = s.n, fs.tile0[i] = tiles;
+        if (i < nseg) tiles += (s.n + kBN - 1) / kBN;
+    }
+    for (int i = nseg; i < 3; i++) fs.tile0[i] = tiles;
+    fs.n_tiles = tiles;
+    SKN_REQUIRE(ctx, ((uintptr_t)a_dev & (a_is_f32 ? 15 : 7)) == 0, SKN_ERR_ARG, "Q4_K GEMM: activations are misaligned");
+    // fragment-order workspace: rows padded to whole tiles
+    const int mt_rows = m > 64 ? 128 : 64;
+    const int m_tiles = (m + mt_rows - 1) / mt_rows, m_pad = m_tiles * mt_rows;
+    const size_t af_bytes = align_up((size_t)m_pad * k * 2), sf_bytes = align_up((size_t)m_pad * (k / 256) * 16 * 2);
+    const size_t is_bytes = align_up((size_t)m_pad * 4);
+    uint8_t* ws;
+    int rc = gemm_workspace(ctx, af_bytes + sf_bytes + is_bytes, &ws);
+    if (rc != SKN_OK) return rc;
+    _Float16* afrag = (_Float16*)ws;
+    _Float16* sfrag = (_Float16*)(ws + af_bytes);
+    float* isc = (float*)(ws + af_bytes + sf_bytes);
+    if (a_is_f32)
+        skn_launch(ctx, prep_a_frag_kernel<4, float>, dim3(m_pad / 4), dim3(256), 0, (const float*)a_dev, afrag, isc, sfrag, m, k);
+    else
+        skn_launch(ctx, prep_a_frag_kernel<4, uint16_t>, dim3(m_pad / 4), dim3(256), 0, (const uint16_t*)a_dev, afrag, isc,
+                   sfrag, m, k);
+    SKN_LAUNCH_CHECK(ctx);
+    if (mt_rows == 128) return launch_frag<2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
+    return launch_frag<1>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
+}
+
 extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const uint16_t* a_bf16_dev,
                           int m, float* c_dev) {
     SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_gemm_q: ctx is null");
@@ -457,6 +882,12 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     SKN_REQUIRE(ctx, k % kKC == 0, SKN_ERR_SHAPE, "skn_gemm_q: k (%d) must be a multiple of %d", k, kKC);
 
     if (ggml_type == SKN_TYPE_Q4_K && k <= 16384) {
+        SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
+                    "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
+        if (ctx->opt_gemm_q4k != 1) {
+            const skn_gemm_seg seg = {w_dev, n, c_dev};
+            return skn_gemm_q4k_multi(ctx, &seg, 1, k, a_bf16_dev, 0, m);
+        }
         // workspace: permuted fp16 activations, row scales, sub-block sums (hi, lo)
         const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
         const size_t sum_bytes = align_up((size_t)m * (k / 32) * 2);
@@ -467,8 +898,6 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
         float* inv_scale = (float*)(ws + a16_bytes);
         _Float16* sum_hi = (_Float16*)(ws + a16_bytes + sc_bytes);
         _Float16* sum_lo = (_Float16*)(ws + a16_bytes + sc_bytes + sum_bytes);
-        SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
-                    "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
         skn_launch(ctx, prep_a_q4k_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, sum_hi, sum_lo, k);
         SKN_LAUNCH_CHECK(ctx);
         // 128-row tiles when they alone give every compute unit two workgroups, 64-row tiles otherwise
