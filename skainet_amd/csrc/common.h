@@ -28,7 +28,7 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_q4k = 0;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1;
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
@@ -95,6 +95,17 @@ inline void skn_launch(skn_ctx* ctx, F kernel, dim3 grid, dim3 block, size_t lds
         hipLaunchKernelGGL(kernel, grid, block, (unsigned)lds, ctx->stream, args...);
     }
 }
+
+#ifdef __HIPCC__
+// v as an fp16 pair: hi = f16(v), lo = f16(v - hi).  v is first hidden from the optimizer: when it can see the
+// product that made v, it fuses that product into each conversion separately (a fused convert rounds once, a
+// plain one twice) and the hi that lo was taken against is then not always the hi that is stored.
+__device__ __forceinline__ void skn_split_hilo(float v, _Float16& hi, _Float16& lo) {
+    asm("" : "+v"(v));
+    hi = (_Float16)v;
+    lo = (_Float16)(v - (float)hi);
+}
+#endif
 
 // the three formats with tuned kernels (and the only ones the decoder's embedding lookup reads)
 static inline bool skn_is_core_quant(int t) { return t == SKN_TYPE_Q8_0 || t == SKN_TYPE_Q4_K || t == SKN_TYPE_Q6_K; }

@@ -508,8 +508,8 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
         // Q4_K weights take the fp32 rows as they are (rounded to bf16 inside the GEMM's preparation pass)
-        const bool q4k_attn = L.type_attn == SKN_TYPE_Q4_K && H <= 16384 && ctx->opt_gemm_q4k != 1;
-        const bool q4k_ffn = L.type_ffn == SKN_TYPE_Q4_K && H <= 16384 && F <= 16384 && ctx->opt_gemm_q4k != 1;
+        const bool q4k_attn = L.type_attn == SKN_TYPE_Q4_K && H <= 16384;
+        const bool q4k_ffn = L.type_ffn == SKN_TYPE_Q4_K && H <= 16384 && F <= 16384;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
         skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
         SKN_LAUNCH_CHECK(ctx);

@@ -23,8 +23,9 @@ __device__ __forceinline__ void put4(float* __restrict__ out, _Float16* __restri
         half4_t h, l;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            h[i] = (_Float16)v[i];
-            l[i] = (_Float16)(v[i] - (float)h[i]);
+            _Float16 a, b;
+            skn_split_hilo(v[i], a, b);
+            h[i] = a, l[i] = b;
         }
         reinterpret_cast<half4_t*>(hi)[t] = h;
         reinterpret_cast<half4_t*>(lo)[t] = l;

@@ -240,8 +240,9 @@ __global__ __launch_bounds__(256) void dequant_blocks_hilo_kernel(const uint8_t*
     half4_t h, l;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        h[i] = (_Float16)v[i];
-        l[i] = (_Float16)(v[i] - (float)h[i]);
+        _Float16 a, b;
+        skn_split_hilo(v[i], a, b);
+        h[i] = a, l[i] = b;
     }
     reinterpret_cast<half4_t*>(hi)[t] = h;
     reinterpret_cast<half4_t*>(lo)[t] = l;
@@ -252,10 +253,10 @@ __global__ __launch_bounds__(256) void convert_dense_hilo_kernel(const uint8_t* 
                                                                  _Float16* __restrict__ lo, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float v = dense_at<T>(w, i);
-    const _Float16 h = (_Float16)v;
+    _Float16 h, l;
+    skn_split_hilo(dense_at<T>(w, i), h, l);
     hi[i] = h;
-    lo[i] = (_Float16)(v - (float)h);
+    lo[i] = l;
 }
 
 template <int T>

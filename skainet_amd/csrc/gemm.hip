@@ -8,11 +8,11 @@
 //   * Activations: bf16 -> fp16 is exact for every value whose magnitude is within fp16's normal range; each
 //     row is first scaled by a power of two that puts its largest magnitude just below 2^14 (2^10 on the Q4_K
 //     path) and the scale is undone in the epilogue.  Products and sums are fp32 inside the MFMA.
-//   * Weights, general path (Q8_0, Q6_K): W is dequantized once into a workspace as an fp16 pair
+//   * Weights, general path (every format but Q4_K): W is dequantized once into a workspace as an fp16 pair
 //     hi = f16(w), lo = f16(w - hi) (w_hi + w_lo = w to 2^-22 relative) and each k-step issues two MFMAs.
-//   * Weights, Q4_K path: see gemm_q4k_kernel -- the 4-bit quants times their 6-bit sub-block scale are
-//     integers below 2^10, exact in fp16, so one MFMA per k-step suffices and the f16 superblock scale d is
-//     applied to the fp32 partial sum of each superblock.
+//   * Weights, Q4_K path: see gemm_q4k_frag_kernel -- the 4-bit quants times their 6-bit sub-block scale are
+//     integers below 2^10, exact in fp16, so one MFMA per k-step suffices; the f16 superblock scale d is the
+//     unit in which a column's accumulators are kept.
 #include "common.h"
 
 #include <type_traits>
@@ -55,95 +55,6 @@ __global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict_
     if (threadIdx.x == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 - 13 + e) << 23);
     _Float16* out = a16 + (size_t)m * k;
     for (int i = threadIdx.x; i < k; i += 256) out[i] = (_Float16)(__uint_as_float((uint32_t)ar[i] << 16) * scale);
-}
-
-// Q4_K path.  The row is scaled by a power of two so that its largest magnitude lies in [2^9, 2^10): the
-// conversion to fp16 is exact down to 2^-24 (34 binades below the row maximum) and the sum of a 32-element
-// sub-block (needed for the "- dmin * m" term) stays below the fp16 maximum; each sum is kept as an fp16 pair
-// (hi, lo).  The row is written in the element order in which the Q4_K kernel unpacks weights: task (c, dw) =
-// (64-element chunk, dword of its 32 nibble bytes) gathers elements 4*dw + {0,1,2,3} of the chunk's lower and
-// upper half and writes them as [lo0, lo2, hi0, hi2, lo1, lo3, hi1, hi3] at 64*c + 8*dw.
-// One workgroup per row, eight tasks at most per thread (k <= 16384); eight consecutive lanes share a chunk.
-__global__ __launch_bounds__(256) void prep_a_q4k_kernel(const uint16_t* __restrict__ a, _Float16* __restrict__ a16,
-                                                         float* __restrict__ inv_scale, _Float16* __restrict__ sum_hi,
-                                                         _Float16* __restrict__ sum_lo, int k) {
-    __shared__ float red[4];
-    const int m = blockIdx.x, tid = threadIdx.x;
-    const uint16_t* ar = a + (size_t)m * k;
-    const int tasks = k >> 3;
-    uint2 lo[8], hi[8];
-    float mx = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const int task = min(tid + 256 * j, tasks - 1);
-        const int c = task >> 3, dw = task & 7;
-        lo[j] = *reinterpret_cast<const uint2*>(ar + 64 * c + 4 * dw);
-        hi[j] = *reinterpret_cast<const uint2*>(ar + 64 * c + 32 + 4 * dw);
-    }
-    auto widen = [](uint32_t pair, int which) { return __uint_as_float(which ? pair & 0xFFFF0000u : pair << 16); };
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const uint32_t w4[4] = {lo[j].x, lo[j].y, hi[j].x, hi[j].y};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float v = fabsf(widen(w4[i >> 1], i & 1));
-            if (v == v && v < INFINITY) mx = fmaxf(mx, v);
-        }
-    }
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red[tid >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    int e = 9;  // a zero row keeps scale 1
-    if (mx > 0.f) e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
-    e = max(e, -100);  // (a subnormal maximum: exponent field 0)
-    const float scale = __uint_as_float((uint32_t)(127 + 9 - e) << 23);
-    if (tid == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
-    _Float16* out = a16 + (size_t)m * k;
-    const int nsub = k >> 5;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const int task = tid + 256 * j;
-        const int c = task >> 3, dw = task & 7;
-        _Float16 l[4], u[4];
-        l[0] = (_Float16)(widen(lo[j].x, 0) * scale), l[1] = (_Float16)(widen(lo[j].x, 1) * scale);
-        l[2] = (_Float16)(widen(lo[j].y, 0) * scale), l[3] = (_Float16)(widen(lo[j].y, 1) * scale);
-        u[0] = (_Float16)(widen(hi[j].x, 0) * scale), u[1] = (_Float16)(widen(hi[j].x, 1) * scale);
-        u[2] = (_Float16)(widen(hi[j].y, 0) * scale), u[3] = (_Float16)(widen(hi[j].y, 1) * scale);
-        float sl = ((float)l[0] + (float)l[1]) + ((float)l[2] + (float)l[3]);
-        float su = ((float)u[0] + (float)u[1]) + ((float)u[2] + (float)u[3]);
-        // totals over the eight lanes of the chunk (all lanes run the permutations; tail tasks are clamped copies)
-        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0xB1, 0xF, 0xF, true));
-        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0xB1, 0xF, 0xF, true));
-        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x4E, 0xF, 0xF, true));
-        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x4E, 0xF, 0xF, true));
-        sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x141, 0xF, 0xF, true));
-        su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x141, 0xF, 0xF, true));
-        if (task < tasks) {
-            half8_t o;
-            o[0] = l[0], o[1] = l[2], o[2] = u[0], o[3] = u[2], o[4] = l[1], o[5] = l[3], o[6] = u[1], o[7] = u[3];
-            *reinterpret_cast<half8_t*>(out + 64 * c + 8 * dw) = o;
-            if (dw == 0) {
-                const _Float16 h0 = (_Float16)sl, h1 = (_Float16)su;
-                sum_hi[(size_t)m * nsub + 2 * c] = h0;
-                sum_lo[(size_t)m * nsub + 2 * c] = (_Float16)(sl - (float)h0);
-                sum_hi[(size_t)m * nsub + 2 * c + 1] = h1;
-                sum_lo[(size_t)m * nsub + 2 * c + 1] = (_Float16)(su - (float)h1);
-            }
-        }
-    }
-}
-
-// fp32 [n] -> fp16 pair (hi, lo)
-__global__ void split_hilo_kernel(const float* __restrict__ w, _Float16* __restrict__ hi, _Float16* __restrict__ lo,
-                                  int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
-        const float v = w[i];
-        const _Float16 h = (_Float16)v;
-        hi[i] = h;
-        lo[i] = (_Float16)(v - (float)h);
-    }
 }
 
 // C tile store: acc register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile
@@ -238,190 +149,7 @@ __global__ __launch_bounds__(256) void gemm_dense_hilo_kernel(const _Float16* __
 #undef SKN_STASH
 }
 
-// ---- Q4_K path: weights unpacked in the kernel, one MFMA per k-step ----------------------------------------
-// w[n, 256 b + e] = d * (sc_j * q) - dmin * m_j  (j = sub-block of e).  sc_j * q is an integer below 2^10: the
-// nibble masked in place is the fp16 subnormal q * 2^-24 (or 16 q * 2^-24 for a high nibble) and one packed
-// fp16 multiply by sc_j (or sc_j / 16) gives sc_j * q * 2^-24 exactly -- an fp16 operand the matrix core takes
-// as is.  Per superblock the products are accumulated in a partial tile, which is then folded into the total
-// with the column's d * 2^24; the "- dmin * m_j" term is a second, eight-deep product per superblock between
-// the activation sub-block sums (fp16 hi + lo) and the integers m_j, folded in with dmin.
-// Workgroup tile 128 x 64, 64 k per iteration (one chunk of every weight row: 32 nibble bytes, a quarter per
-// thread, unpacked into 64 fp16).
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restrict__ a16,
-                                                       const _Float16* __restrict__ sum_hi,
-                                                       const _Float16* __restrict__ sum_lo,
-                                                       const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
-                                                       float* __restrict__ c, int m, int n, int k) {
-    // 2 x 2 wavefronts, each MT 32 x 32 tiles stacked along m: workgroup tile (64 * MT) x 64.  MT = 1 doubles the
-    // number of workgroups (two per compute unit, whose phases overlap) for outputs too small to fill the chip.
-    constexpr int BM = 64 * MT;
-    // Two LDS buffers (one barrier per iteration) and a ring of four register stages: the global loads of
-    // iterations it+1 .. it+3 are in flight while iteration it is multiplied.  Four iterations = one superblock,
-    // so the position in the ring is also the chunk index within the superblock.  Every thread issues the same
-    // loads every iteration (no load sits in a conditional block): the wait counters then say exactly which
-    // stage is complete.
-    __shared__ __align__(16) _Float16 sa[2][BM * kRow];
-    __shared__ __align__(16) _Float16 sb[2][kBN * kRow];
-    __shared__ float sd[2][kBN], sdm[2][kBN];
-    __shared__ __align__(8) _Float16 smin[2][kBN * 8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * kBN;
-    const int nb = k >> 8, nsub = k >> 5;
-
-    struct Stage {
-        u32x4 a[2 * MT], h;
-        u32x2 q;
-    };
-    Stage st[4];
-    // activation staging: BM rows x 8 chunks of 16 bytes, 2 * MT per thread (rows srow, srow + 32, ...)
-    const int srow = tid >> 3, sch = (tid & 7) * 8;
-    const _Float16* ga[2 * MT];
-#pragma unroll
-    for (int i = 0; i < 2 * MT; i++) ga[i] = a16 + (size_t)min(m0 + srow + 32 * i, m - 1) * k + sch;
-    // weight staging: thread t owns row t / 4 of the tile and quarter t % 4 of the 32 nibble bytes of a chunk
-    const int brow = tid >> 2, bq = tid & 3;
-    const uint8_t* gw = w + (size_t)min(n0 + brow, n - 1) * nb * 144;
-
-    auto fetch = [&](int sbk, int cc, Stage& s) __attribute__((always_inline)) {
-        const int k0 = (4 * sbk + cc) * kKC;
-#pragma unroll
-        for (int i = 0; i < 2 * MT; i++) s.a[i] = *reinterpret_cast<const u32x4*>(ga[i] + k0);
-        s.h = *reinterpret_cast<const u32x4*>(gw + (size_t)sbk * 144);
-        s.q = *reinterpret_cast<const u32x2*>(gw + (size_t)sbk * 144 + 16 + 32 * cc + 8 * bq);
-    };
-    // The staging of one iteration, in four parts (two activation stores each; the unpacking of one nibble
-    // dword each for parts 2 and 3) so that the main loop can place one part behind each pair of matrix
-    // instructions: a wavefront issues in order, and the unpacking only overlaps the matrix pipe that way.
-    auto stash_part = [&](int part, int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
-        _Float16* da = sa[cc & 1];
-        _Float16* db = sb[cc & 1];
-        if (part < 2) {
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-                *reinterpret_cast<u32x4*>(da + (srow + 32 * (MT * part + i)) * kRow + sch) = s.a[MT * part + i];
-            return;
-        }
-        // the whole loaded tuple counts as used here: a word that this chunk does not need (d | dmin outside
-        // chunk 0) would otherwise be recycled as a temporary while its load is in flight, and writing it
-        // would wait for that load
-        asm volatile("" ::"v"(s.h));
-        const uint32_t hw[4] = {s.h.x, s.h.y, s.h.z, s.h.w};
-        auto sbyte = [&](int i) { return (hw[1 + (i >> 2)] >> (8 * (i & 3))) & 0xFFu; };
-        auto scale_of = [&](int j) {
-            return j < 4 ? (int)(sbyte(j) & 63) : (int)((sbyte(j + 4) & 0x0F) | ((sbyte(j - 4) >> 6) << 4));
-        };
-        auto min_of = [&](int j) {
-            return j < 4 ? (int)(sbyte(j + 4) & 63) : (int)((sbyte(j + 4) >> 4) | ((sbyte(j) >> 6) << 4));
-        };
-        const _Float16 ml = (_Float16)(float)scale_of(2 * cc);
-        const _Float16 mh = (_Float16)((float)scale_of(2 * cc + 1) * 0.0625f);
-        const half2_t mul_lo = {ml, ml}, mul_hi = {mh, mh};
-        const int j = part - 2;
-        const uint32_t q = j == 0 ? s.q.x : s.q.y, q8 = q >> 8;
-        const uint32_t l02 = q & 0x000F000Fu, h02 = q & 0x00F000F0u;
-        const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
-        u32x4 o;
-        o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo);
-        o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi);
-        o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo);
-        o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi);
-        *reinterpret_cast<u32x4*>(db + brow * kRow + 16 * bq + 8 * j) = o;
-        if (part == 3 && cc == 0 && bq == 0) {  // per superblock: the column's d * 2^24, dmin and the eight m_j
-            const half2_t dd = __builtin_bit_cast(half2_t, hw[0]);
-            sd[sbk & 1][brow] = (float)dd.x * 16777216.0f;
-            sdm[sbk & 1][brow] = (float)dd.y;
-            half8_t mm;
-#pragma unroll
-            for (int jj = 0; jj < 8; jj++) mm[jj] = (_Float16)(float)min_of(jj);
-            *reinterpret_cast<half8_t*>(smin[sbk & 1] + brow * 8) = mm;
-        }
-    };
-    auto stash = [&](int sbk, int cc, const Stage& s) __attribute__((always_inline)) {
-#pragma unroll
-        for (int part = 0; part < 4; part++) stash_part(part, sbk, cc, s);
-    };
-
-    float16_t tot[MT], par[MT];
-#pragma unroll
-    for (int i = 0; i < MT; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) tot[i][r] = par[i][r] = 0.f;
-
-    // activation sub-block sums of this wavefront's two row tiles: lane l holds row l % 32, sub-blocks
-    // 4 * (l / 32) .. + 3 of the current superblock (the operand layout of the eight-deep matrix instruction)
-    size_t soff[MT];
-#pragma unroll
-    for (int i = 0; i < MT; i++)
-        soff[i] = (size_t)min(m0 + wm * 32 * MT + 32 * i + (lane & 31), m - 1) * nsub + 4 * (lane >> 5);
-    const int pfrag = (lane & 31) * kRow + (lane >> 5) * 8;
-
-    // Software pipeline: while the matrix instructions of iteration it run, the wavefront unpacks and stores
-    // iteration it+1 into the other LDS buffer; its global data was requested two iterations earlier.
-    fetch(0, 0, st[0]);
-    fetch(0, 1, st[1]);
-    fetch(0, 2, st[2]);
-    stash(0, 0, st[0]);
-    for (int sbk = 0; sbk < nb; sbk++) {
-        half4_t sh[MT], sl[MT];
-#pragma unroll
-        for (int cc = 0; cc < 4; cc++) {
-            // the stage three iterations ahead
-            if (cc == 0) fetch(sbk, 3, st[3]);
-            else fetch(min(sbk + 1, nb - 1), cc - 1, st[cc - 1]);  // (past the end: repeats the last superblock, unused)
-            if (cc == 0) {
-#pragma unroll
-                for (int i = 0; i < MT; i++) {
-                    sh[i] = *reinterpret_cast<const half4_t*>(sum_hi + soff[i] + 8 * sbk);
-                    sl[i] = *reinterpret_cast<const half4_t*>(sum_lo + soff[i] + 8 * sbk);
-                }
-            }
-            __syncthreads();  // buffer cc & 1 is complete, and nobody reads the other one any more
-            const _Float16* pa = sa[cc & 1] + wm * 32 * MT * kRow + pfrag;
-            const _Float16* pb = sb[cc & 1] + wn * 32 * kRow + pfrag;
-            half8_t fa[MT][4], fb[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-#pragma unroll
-                for (int i = 0; i < MT; i++) fa[i][t] = *reinterpret_cast<const half8_t*>(pa + 32 * i * kRow + 16 * t);
-                fb[t] = *reinterpret_cast<const half8_t*>(pb + 16 * t);
-            }
-            const bool more = cc < 3 || sbk + 1 < nb;
-            const int nsb = cc < 3 ? sbk : sbk + 1, ncc = (cc + 1) & 3;
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-#pragma unroll
-                for (int i = 0; i < MT; i++) par[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i][t], fb[t], par[i], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (more) stash_part(t, nsb, ncc, st[ncc]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        // end of the superblock: fold the partial tiles into the totals
-        const half4_t fm = *reinterpret_cast<const half4_t*>(smin[sbk & 1] + (wn * 32 + (lane & 31)) * 8 + 4 * (lane >> 5));
-        const float ds = sd[sbk & 1][wn * 32 + (lane & 31)];
-        const float dm = sdm[sbk & 1][wn * 32 + (lane & 31)];
-#pragma unroll
-        for (int i = 0; i < MT; i++) {
-            float16_t mn;
-#pragma unroll
-            for (int r = 0; r < 16; r++) mn[r] = 0.f;
-            mn = __builtin_amdgcn_mfma_f32_32x32x8f16(sh[i], fm, mn, 0, 0, 0);
-            mn = __builtin_amdgcn_mfma_f32_32x32x8f16(sl[i], fm, mn, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                tot[i][r] = fmaf(ds, par[i][r], fmaf(-dm, mn[r], tot[i][r]));
-                par[i][r] = 0.f;
-            }
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < MT; i++)
-        store_tile(tot[i], c, n, m0 + wm * 32 * MT + 32 * i, n0 + wn * 32, m, n, inv_scale, lane);
-}
-
-// ---- Q4_K path, second form: every wavefront loads its matrix-core operands itself ------------------------
+// ---- Q4_K path: weights unpacked in the kernel, one MFMA per k-step, operands loaded by the wavefronts ------
 // Workgroup of eight wavefronts, tile (64 MT) x 64.  The tile is divided in two along m; along k it is not
 // divided spatially but by superblock: wavefront (mh, kq) computes rows [32 MT mh, 32 MT (mh + 1)) x all 64
 // columns for superblocks kq, kq + 4, ..., and the four partial tiles of each half are added through LDS at
@@ -431,7 +159,10 @@ __global__ __launch_bounds__(256) void gemm_q4k_kernel(const _Float16* __restric
 // coalesced 1 KiB load and never passes through LDS.  The weights of four superblocks (576 contiguous bytes of
 // each of the 64 rows) are copied from global memory straight into LDS once per group of four superblocks --
 // the only barrier in the loop -- from where each lane picks the 16 bytes of its row and k-step quartet.
-// Operands are the exact integers of the first form.  One set of accumulators: see the kernel.
+// w[n, 256 b + e] = d * (sc_j * q) - dmin * m_j  (j = sub-block of e).  sc_j * q is an integer below 2^10: the
+// nibble masked in place is the fp16 subnormal q * 2^-24 (or 16 q * 2^-24 for a high nibble) and one packed
+// fp16 multiply by sc_j * 2^10 (or sc_j * 2^6) gives sc_j * q * 2^-14 exactly -- an fp16 operand the matrix
+// core takes as is.  One set of accumulators: see the kernel.
 constexpr int kWPitch = 576;  // LDS pitch of a weight row: the 144 bytes of four superblocks
 
 // Activations bf16 [m, k] -> fragment order.  One workgroup per R rows of the padded row count (rows >= m are
@@ -528,11 +259,12 @@ __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const IN* __restric
             const int h = dw >> 2, s = dw & 3;
             stage[((c * 4 + s) * 2 + h) * R + r8] = __builtin_bit_cast(u32x4, o);
             if (dw == 0 && task < tasks) {
-                sl *= 0x1p-12f, su *= 0x1p-12f;
-                const _Float16 h0 = (_Float16)sl, h1 = (_Float16)su;
+                _Float16 h0, h1, l0, l1;
+                skn_split_hilo(sl * 0x1p-12f, h0, l0);
+                skn_split_hilo(su * 0x1p-12f, h1, l1);
                 const int cg = (k0 >> 6) + c;
                 _Float16* sf = sfrag + ((size_t)mb * nb + (cg >> 2)) * 512 + 2 * (cg & 3);
-                half2_t vh = {h0, h1}, vl = {(_Float16)(sl - (float)h0), (_Float16)(su - (float)h1)};
+                half2_t vh = {h0, h1}, vl = {l0, l1};
                 *reinterpret_cast<half2_t*>(sf + r * 8) = vh;
                 *reinterpret_cast<half2_t*>(sf + (32 + r) * 8) = vl;
             }
@@ -558,13 +290,13 @@ struct Q4kFragSegs {
     int n_tiles;
 };
 
-// Accumulators: acc holds the running sum of a column in units of cs = d * 2^24 of the latest superblock whose d
+// Accumulators: acc holds the running sum of a column in units of cs = d * 2^14 of the latest superblock whose d
 // is not zero.  Entering a superblock it is rescaled by cs_old / cs_new (a relative error of 2^-23 per
 // superblock, against the 1e-3 asked of the op); the superblock's integer products then add to it as they come
 // out of the matrix core, and so does the "- dmin * m_j" term: one more sixteen-deep product per tile between
 // the activation sub-block sums (fp16 hi | lo) and -(dmin / cs) * m_j * 2^12, itself split into an fp16 pair.
-template <int MT>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int MT, int MH>
+__global__ __launch_bounds__(256 * MH) __attribute__((amdgpu_waves_per_eu(MH, MH)))
 void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const Q4kFragSegs segs,
                           const float* __restrict__ inv_scale, int m, int k) {
     constexpr int kWBuf = kBN * kWPitch;
@@ -580,7 +312,7 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     const uint8_t* __restrict__ w = segs.w[seg];
     float* __restrict__ c = segs.c[seg];
     const int n = segs.n[seg];
-    const int mb0 = (2 * mt + mh) * MT, n0 = (tn - segs.tile0[seg]) * kBN;
+    const int mb0 = (MH * mt + mh) * MT, n0 = (tn - segs.tile0[seg]) * kBN;
 
     // Weight staging, global memory straight into LDS: a wavefront-wide load fills 64 sixteen-byte slots
     // i * 64 + lane; slot P holds piece P % 36 of tile row P / 36 (36 pieces = the 576 bytes of four
@@ -588,8 +320,8 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     // with the vector-memory counter before the barrier that publishes the buffer.
     auto wfetch = [&](int g, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int x = 0; x < 5; x++) {
-            const int i = wave + 8 * x;
+        for (int x = 0; x < (36 + 4 * MH - 1) / (4 * MH); x++) {
+            const int i = wave + 4 * MH * x;
             if (i < 36) {
                 const int p = i * 64 + lane, row = p / 36, col = p - 36 * row;
                 const int off = min(g * 576 + col * 16, nb * 144 - 16);  // (a short last group repeats the row's last piece)
@@ -637,29 +369,38 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
             u32x4 hd[2], sf[MT];
 #pragma unroll
             for (int j = 0; j < 2; j++) hd[j] = *reinterpret_cast<const u32x4*>(wl + j * kTile);
-            auto sbyte = [&](int j, int i) { return (hd[j][1 + (i >> 2)] >> (8 * (i & 3))) & 0xFFu; };
-            auto scale_of = [&](int j, int s) {
-                return s < 4 ? (int)(sbyte(j, s) & 63) : (int)((sbyte(j, s + 4) & 0x0F) | ((sbyte(j, s - 4) >> 6) << 4));
-            };
-            auto min_of = [&](int j, int s) {
-                return s < 4 ? (int)(sbyte(j, s + 4) & 63) : (int)((sbyte(j, s + 4) >> 4) | ((sbyte(j, s) >> 6) << 4));
-            };
-            float min_unit[2], live[2];
+            // The eight 6-bit scales and mins of the superblock, four to a word: bytes 0..3 of the twelve hold the
+            // low scales, 4..7 the low mins, 8..11 the low nibbles of the high ones, whose top two bits sit in
+            // bits 6..7 of the first eight bytes.
+            uint32_t sc4[2][2], mn4[2][2];
+            float min_unit[2], sc_unit[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const uint32_t dw0 = hd[j][0];
+                const uint32_t dw0 = hd[j][0], s0 = hd[j][1], s1 = hd[j][2], s2 = hd[j][3];
                 const half2_t dd = __builtin_bit_cast(half2_t, dw0);
-                const float ds = (float)dd.x * 16777216.0f;
-                live[j] = ds != 0.f ? 1.f : 0.f;  // (a zero d: the column keeps its unit and the products are zeroed)
-                const float cs_new = ds != 0.f ? ds : cs[j];
+                const float d = (float)dd.x, dmin = (float)dd.y;
+                const bool live = d != 0.f;  // (a zero d: the column keeps its unit and the products are zeroed)
+                sc4[j][0] = live ? s0 & 0x3F3F3F3Fu : 0u;
+                sc4[j][1] = live ? (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u) : 0u;
+                mn4[j][0] = s1 & 0x3F3F3F3Fu;
+                mn4[j][1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+                // The unit is d * 2^(14 + p) and the weight operands are sc * q * 2^-(14 + p) -- exact in fp16 for
+                // p <= 10.  p = 0 unless |dmin / d| is so large (>= 2^11) that the min operands below would
+                // overflow fp16; beyond 2^21 they saturate.
+                const int e_d = (int)((__float_as_uint(d) >> 23) & 0xFFu), e_m = (int)((__float_as_uint(dmin) >> 23) & 0xFFu);
+                const int pw = live ? min(max(e_m - e_d - 10, 0), 10) : 0;
+                sc_unit[j] = __uint_as_float((uint32_t)(127 + 10 - pw) << 23);
+                const float cs_new = live ? d * __uint_as_float((uint32_t)(127 + 14 + pw) << 23) : cs[j];
                 const float inv = 1.0f / cs_new, ratio = cs[j] * inv;
-                min_unit[j] = -(float)dd.y * inv * 4096.0f;
+                // -(dmin / unit) * 2^12: times a min (< 64) it stays inside fp16
+                min_unit[j] = fminf(fmaxf(-dmin * inv * 4096.0f, -1023.f), 1023.f);
                 cs[j] = cs_new;
 #pragma unroll
                 for (int i = 0; i < MT; i++)
 #pragma unroll
                     for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio;
             }
+            auto byte_f = [](uint32_t word, int b) { return (float)((word >> (8 * b)) & 0xFFu); };
             // Sixteen k-steps, software-pipelined: the weight fragments of step t + 1 are unpacked (vector ALU)
             // while the matrix instructions of step t run.
             u32x4 q[2], qn[2];
@@ -669,13 +410,13 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
 #pragma unroll
                 for (int j = 0; j < 2; j++) dst[j] = *reinterpret_cast<const u32x4*>(wl + j * kTile + 16 + 32 * cc + 16 * h);
             };
-            auto scales = [&](int cc) __attribute__((always_inline)) {
+            auto scales = [&](int cc) __attribute__((always_inline)) {  // sub-blocks 2 cc (low nibbles), 2 cc + 1 (high)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    const _Float16 ml = (_Float16)((float)scale_of(j, 2 * cc) * live[j]);
-                    const _Float16 mh2 = (_Float16)((float)scale_of(j, 2 * cc + 1) * (0.0625f * live[j]));
-                    mul_lo[j] = half2_t{ml, ml};
-                    mul_hi[j] = half2_t{mh2, mh2};
+                    const float fl = byte_f(sc4[j][cc >> 1], 2 * (cc & 1)) * sc_unit[j];
+                    const float fh = byte_f(sc4[j][cc >> 1], 2 * (cc & 1) + 1) * (sc_unit[j] * 0.0625f);
+                    mul_lo[j] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(fl, fl));  // (six bits times a power of two: exact)
+                    mul_hi[j] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(fh, fh));
                 }
             };
             auto decode = [&](int s, half8_t* dst) __attribute__((always_inline)) {
@@ -735,9 +476,9 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 half8_t vh, vl;
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
-                    const float v = fminf(fmaxf(min_unit[j] * (float)min_of(j, s), -60000.f), 60000.f);
-                    vh[s] = (_Float16)v;
-                    vl[s] = (_Float16)(v - (float)vh[s]);
+                    _Float16 a, b;
+                    skn_split_hilo(min_unit[j] * byte_f(mn4[j][s >> 2], s & 3), a, b);
+                    vh[s] = a, vl[s] = b;
                 }
 #pragma unroll
                 for (int i = 0; i < MT; i++) {
@@ -794,16 +535,16 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
 }
 
 // the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in once
-template <int MT>
+template <int MT, int MH>
 int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfrag, const Q4kFragSegs& segs, const float* isc,
                 int m, int k) {
-    constexpr int kLds = 2 * kBN * kWPitch > MT * 49152 ? 2 * kBN * kWPitch : MT * 49152;
+    constexpr int kLds = 2 * kBN * kWPitch > MT * MH * 24576 ? 2 * kBN * kWPitch : MT * MH * 24576;
     static bool opted = false;
     if (!opted) {
-        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<MT>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<MT, MH>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
         opted = true;
     }
-    skn_launch(ctx, gemm_q4k_frag_kernel<MT>, dim3(m_tiles * segs.n_tiles), dim3(512), kLds, afrag, sfrag, segs, isc, m, k);
+    skn_launch(ctx, gemm_q4k_frag_kernel<MT, MH>, dim3(m_tiles * segs.n_tiles), dim3(256 * MH), kLds, afrag, sfrag, segs, isc, m, k);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
@@ -862,8 +603,8 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
         skn_launch(ctx, prep_a_frag_kernel<4, uint16_t>, dim3(m_pad / 4), dim3(256), 0, (const uint16_t*)a_dev, afrag, isc,
                    sfrag, m, k);
     SKN_LAUNCH_CHECK(ctx);
-    if (mt_rows == 128) return launch_frag<2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
-    return launch_frag<1>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
+    if (mt_rows == 128) return launch_frag<2, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
+    return launch_frag<1, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
 }
 
 extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const uint16_t* a_bf16_dev,
@@ -884,35 +625,8 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     if (ggml_type == SKN_TYPE_Q4_K && k <= 16384) {
         SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
                     "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
-        if (ctx->opt_gemm_q4k != 1) {
-            const skn_gemm_seg seg = {w_dev, n, c_dev};
-            return skn_gemm_q4k_multi(ctx, &seg, 1, k, a_bf16_dev, 0, m);
-        }
-        // workspace: permuted fp16 activations, row scales, sub-block sums (hi, lo)
-        const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
-        const size_t sum_bytes = align_up((size_t)m * (k / 32) * 2);
-        uint8_t* ws;
-        int rc = gemm_workspace(ctx, a16_bytes + sc_bytes + 2 * sum_bytes, &ws);
-        if (rc != SKN_OK) return rc;
-        _Float16* a16 = (_Float16*)ws;
-        float* inv_scale = (float*)(ws + a16_bytes);
-        _Float16* sum_hi = (_Float16*)(ws + a16_bytes + sc_bytes);
-        _Float16* sum_lo = (_Float16*)(ws + a16_bytes + sc_bytes + sum_bytes);
-        skn_launch(ctx, prep_a_q4k_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, sum_hi, sum_lo, k);
-        SKN_LAUNCH_CHECK(ctx);
-        // 128-row tiles when they alone give every compute unit two workgroups, 64-row tiles otherwise
-        const int wide = ((n + kBN - 1) / kBN) * ((m + 127) / 128);
-        if (wide >= 2 * ctx->compute_units) {
-            dim3 grid((n + kBN - 1) / kBN, (m + 127) / 128);
-            skn_launch(ctx, gemm_q4k_kernel<2>, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
-                       (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
-        } else {
-            dim3 grid((n + kBN - 1) / kBN, (m + 63) / 64);
-            skn_launch(ctx, gemm_q4k_kernel<1>, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)sum_hi,
-                       (const _Float16*)sum_lo, (const uint8_t*)w_dev, (const float*)inv_scale, c_dev, m, n, k);
-        }
-        SKN_LAUNCH_CHECK(ctx);
-        return SKN_OK;
+        const skn_gemm_seg seg = {w_dev, n, c_dev};
+        return skn_gemm_q4k_multi(ctx, &seg, 1, k, a_bf16_dev, 0, m);
     }
 
     // workspace: fp16 activations + row scales, then (general path) the weights as an fp16 pair
