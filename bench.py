@@ -282,7 +282,7 @@ def main():
         print(json.dumps({"mode": "decode", **llama_bench.run(ctx, steps=min(args.steps, 128))}))
         ctx.close()
         return
-    gemm_shapes = [("q4_k", Q4_K, 512, 4096, 4096), ("q4_k", Q4_K, 512, 14336, 4096),
+    gemm_shapes = [("q4_k", Q4_K, 512, 4096, 4096), ("q4_k", Q4_K, 512, 14336, 4096), ("q4_k", Q4_K, 512, 4096, 11008),
                    ("q6_k", Q6_K, 512, 4096, 4096), ("q6_k", Q6_K, 512, 14336, 4096)]
     if args.mode == "attention":
         print(json.dumps({"mode": "attention", **bench_attention(ctx, min(args.steps, 200), 10)}))
