@@ -379,7 +379,7 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 const uint32_t dw0 = hd[j][0], s0 = hd[j][1], s1 = hd[j][2], s2 = hd[j][3];
                 const half2_t dd = __builtin_bit_cast(half2_t, dw0);
                 const float d = (float)dd.x, dmin = (float)dd.y;
-                const bool live = d != 0.f;  // (a zero d: the column keeps its unit and the products are zeroed)
+                const bool live = d != 0.f;  // (a zero d: the products are zeroed)
                 sc4[j][0] = live ? s0 & 0x3F3F3F3Fu : 0u;
                 sc4[j][1] = live ? (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u) : 0u;
                 mn4[j][0] = s1 & 0x3F3F3F3Fu;
@@ -390,7 +390,10 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 const int e_d = (int)((__float_as_uint(d) >> 23) & 0xFFu), e_m = (int)((__float_as_uint(dmin) >> 23) & 0xFFu);
                 const int pw = live ? min(max(e_m - e_d - 10, 0), 10) : 0;
                 sc_unit[j] = __uint_as_float((uint32_t)(127 + 10 - pw) << 23);
-                const float cs_new = live ? d * __uint_as_float((uint32_t)(127 + 14 + pw) << 23) : cs[j];
+                // (no live weights: the unit is free, and taken from dmin so that the min operands are well inside
+                // fp16 -- the unit inherited from the last live superblock can be orders of magnitude off)
+                const float cs_new = live ? d * __uint_as_float((uint32_t)(127 + 14 + pw) << 23)
+                                          : (dmin != 0.f ? fabsf(dmin) * 512.0f : cs[j]);
                 const float inv = 1.0f / cs_new, ratio = cs[j] * inv;
                 // -(dmin / unit) * 2^12: times a min (< 64) it stays inside fp16
                 min_unit[j] = fminf(fmaxf(-dmin * inv * 4096.0f, -1023.f), 1023.f);

@@ -88,6 +88,45 @@ def test_gemm_extreme_rows(hip, qtype):
         assert oracle_np.rel_err(got[r], want[r]) <= TOL, r
 
 
+def test_gemm_q4k_superblock_scale_extremes(hip):
+    """The Q4_K kernel keeps a column's accumulators in units of the current superblock's d: superblocks with
+    d = 0, negative d or dmin, dmin = 0, d a subnormal, |dmin / d| from 2^-20 to 2^20, and d jumping by 2^20
+    between neighbouring superblocks must all come out right."""
+    m, n, k = 40, 64, 4096
+    nb = k // 256
+    raw = synth.weight(Q4_K, n, k, seed=91).reshape(n, nb, 144).copy()
+    f16 = lambda v: np.array([v], dtype=np.float16).view(np.uint8)  # noqa: E731
+    cases = [(0.0, 0.01), (0.0, 0.0), (-0.02, 0.01), (0.02, -0.01), (0.01, 0.0), (6e-8, 1e-7), (1e-5, 10.0),
+             (1e-6, 1.0), (10.0, 1e-5), (500.0, 0.5), (3e-5, 0.03), (0.03, 3e-5), (-1e-4, -20.0), (2e-7, 0.2)]
+    rng = np.random.default_rng(92)
+    for col in range(n):
+        for sb in range(nb):
+            if col < 8 and sb % 3 == 1:
+                continue  # a few ordinary superblocks in between
+            d, dmin = cases[rng.integers(len(cases))] if col < 48 else cases[(col + sb) % len(cases)]
+            raw[col, sb, 0:2] = f16(d)
+            raw[col, sb, 2:4] = f16(dmin)
+    raw[48] = raw[48, 0]  # every superblock the same
+    raw[49, :, 0:2] = f16(0.0)  # a column with no live superblock at all
+    raw = raw.reshape(-1)
+    a = synth.activation_bf16((m, k), seed=93)
+    got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    want = oracle_c.gemm_q(Q4_K, raw, n, k, a, m)
+    assert np.all(np.isfinite(got))
+    for col in range(n):  # column by column: their magnitudes differ by many orders
+        assert oracle_np.rel_err(got[:, col], want[:, col]) <= TOL, col
+
+
+def test_gemm_q4k_several_row_tiles_and_ragged_columns(hip):
+    """Three 128-row tiles (the last one partial) and a column count that is not a multiple of the 64-column tile."""
+    m, n, k = 300, 200, 1280
+    raw = synth.weight(Q4_K, n, k, seed=95)
+    a = synth.activation_bf16((m, k), seed=96)
+    got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    want = oracle_c.gemm_q(Q4_K, raw, n, k, a, m)
+    assert oracle_np.rel_err(got, want) <= TOL
+
+
 @pytest.mark.parametrize("n", [4096, 14336])
 def test_gemm_benchmark_shapes_q6k(hip, n):
     """M=512, K=4096 with Q6_K weights (the mixed-precision prefill case), sampled columns."""
