@@ -117,14 +117,24 @@ static inline bool skn_is_quant(int t) {
 }
 int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out);
 int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y);
-// Q4_K GEMM of one activation matrix [m, k] (bf16, or fp32 rounded to bf16 on the way in) against up to three
-// weight matrices [n_i, k] in one launch: c_i[m, n_i] = a * w_i^T.
+// Q4_K GEMM of one activation matrix [m, k] against up to three weight matrices [n_i, k] in one launch:
+// c_i[m, n_i] (+)= a * w_i^T.  The activation rows are bf16 (as skn_gemm_q takes them), or fp32 that the GEMM's
+// preparation pass rounds to bf16 itself -- optionally after the RMSNorm (weights b) that precedes the GEMM in
+// a transformer block, with the arithmetic of the separate row-wise kernel.
+enum { SKN_SRC_BF16 = 0, SKN_SRC_F32 = 1, SKN_SRC_RMSNORM = 2 };
+struct skn_gemm_src {
+    int kind;
+    const void* a;
+    const void* b;
+    float eps;  // SKN_SRC_RMSNORM
+};
 struct skn_gemm_seg {
     const void* w;
     int n;
     float* c;
+    int accumulate;  // c += instead of c =
 };
-int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const void* a_dev, int a_is_f32, int m);
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m);
 int skn_dequant_hilo(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
 int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
 

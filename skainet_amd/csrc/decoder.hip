@@ -507,16 +507,17 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
-        // Q4_K weights take the fp32 rows as they are (rounded to bf16 inside the GEMM's preparation pass)
+        // Q4_K weights: the GEMM's preparation pass takes the fp32 rows and does the row-wise work before them
         const bool q4k_attn = L.type_attn == SKN_TYPE_Q4_K && H <= 16384;
         const bool q4k_ffn = L.type_ffn == SKN_TYPE_Q4_K && H <= 16384 && F <= 16384;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
-        skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
-        SKN_LAUNCH_CHECK(ctx);
-        if (q4k_attn) {  // one activation preparation and one launch for the three projections
-            const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq}, {L.wk, H, m->pk}, {L.wv, H, m->pv}};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, m->pxn, 1, T));
+        if (q4k_attn) {  // RMSNorm inside the activation pass, one launch for the three projections
+            const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq, 0}, {L.wk, H, m->pk, 0}, {L.wv, H, m->pv, 0}};
+            const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.attn_norm, c.rms_eps};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, src, T));
         } else {
+            skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
+            SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wq, H, H, m->pb16, T, m->pq));
             SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wk, H, H, m->pb16, T, m->pk));
@@ -528,39 +529,44 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
         SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
-        if (q4k_attn) {
-            const skn_gemm_seg wo = {L.wo, H, m->pproj};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, &wo, 1, H, m->patt, 1, T));
+        if (q4k_attn) {  // the residual is added by the GEMM's store
+            const skn_gemm_seg wo = {L.wo, H, m->px, 1};
+            const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, &wo, 1, H, src, T));
         } else {
             SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
+            skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
+                       (int64_t)T * H);
+            SKN_LAUNCH_CHECK(ctx);
         }
-        skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
-                   (int64_t)T * H);
-        SKN_LAUNCH_CHECK(ctx);
-        skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
-        SKN_LAUNCH_CHECK(ctx);
         if (q4k_ffn) {
-            const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pgate}, {L.w_up, F, m->pup}};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, m->pxn, 1, T));
+            const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pgate, 0}, {L.w_up, F, m->pup, 0}};
+            const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.ffn_norm, c.rms_eps};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, src, T));
+            // (SwiGLU stays a kernel of its own: inside the activation pass, which runs one wavefront per row,
+            // its exponentials cost more than the separate element-wise launch)
+            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                       (const float*)m->pup, m->pmid, (int64_t)T * F);
+            SKN_LAUNCH_CHECK(ctx);
+            const skn_gemm_seg down = {L.w_down, H, m->px, 1};  // residual added by the store
+            const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, mid, T));
         } else {
+            skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
+            SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_gate, F, H, m->pb16, T, m->pgate));
             SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_up, F, H, m->pb16, T, m->pup));
-        }
-        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
-                   (const float*)m->pup, m->pmid, (int64_t)T * F);
-        SKN_LAUNCH_CHECK(ctx);
-        if (q4k_ffn) {
-            const skn_gemm_seg down = {L.w_down, H, m->pproj};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, m->pmid, 1, T));
-        } else {
+            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                       (const float*)m->pup, m->pmid, (int64_t)T * F);
+            SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
             SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_down, H, F, m->pb16, T, m->pproj));
+            skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
+                       (int64_t)T * H);
+            SKN_LAUNCH_CHECK(ctx);
         }
-        skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
-                   (int64_t)T * H);
-        SKN_LAUNCH_CHECK(ctx);
         // the cache of this layer now holds pos0 + T tokens
         kv->len[0] = pos0 + T;
     }

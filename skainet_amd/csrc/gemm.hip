@@ -59,12 +59,16 @@ __global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict_
 
 // C tile store: acc register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile
 __device__ __forceinline__ void store_tile(const float16_t& acc, float* __restrict__ c, int ldc, int row0, int col0,
-                                           int m, int n, const float* __restrict__ inv_scale, int lane) {
+                                           int m, int n, const float* __restrict__ inv_scale, int lane,
+                                           bool accumulate = false) {
     const int col = col0 + (lane & 31);
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         const int row = row0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < m && col < n) c[(size_t)row * ldc + col] = acc[r] * inv_scale[row];
+        if (row < m && col < n) {
+            float* dst = c + (size_t)row * ldc + col;
+            *dst = accumulate ? *dst + acc[r] * inv_scale[row] : acc[r] * inv_scale[row];
+        }
     }
 }
 
@@ -171,31 +175,65 @@ constexpr int kWPitch = 576;  // LDS pitch of a weight row: the 144 bytes of fou
 // bytes (the same sixteen bytes of R neighbouring rows).
 // afrag: [row block][chunk][k-step][lane] x 8 halves.  sfrag: [row block][superblock][lane] x 8 halves: the eight
 // sub-block sums of row r times 2^-12 as fp16 pairs, lanes 0..31 the "hi" parts, lanes 32..63 the "lo" parts.
-// IN = uint16_t: bf16 activations; IN = float: fp32 activations, rounded to bf16 (nearest even) on the way in.
-template <typename IN>
-__device__ __forceinline__ void load_bf16x4(const IN* p, uint32_t& lo, uint32_t& hi);
-template <>
-__device__ __forceinline__ void load_bf16x4<uint16_t>(const uint16_t* p, uint32_t& lo, uint32_t& hi) {
-    const u32x2 v = *reinterpret_cast<const u32x2*>(p);
-    lo = v.x, hi = v.y;
-}
-template <>
-__device__ __forceinline__ void load_bf16x4<float>(const float* p, uint32_t& lo, uint32_t& hi) {
-    const u32x4 v = *reinterpret_cast<const u32x4*>(p);
-    auto rne = [](uint32_t u) { return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16; };
-    lo = rne(v.x) | (rne(v.y) << 16);
-    hi = rne(v.z) | (rne(v.w) << 16);
+// The rows come from a source (skn_gemm_src): bf16 as given; fp32 rounded to bf16 (nearest even) on the way in;
+// or fp32 RMS-normalized first (x * r * g, r = 1 / sqrt(mean(x^2) + eps)) -- the row-wise kernel that would
+// otherwise run before the GEMM.
+struct PrepRow {
+    const void* a;   // the row
+    const void* b;   // SKN_SRC_RMSNORM: the norm weights
+    float r;         // SKN_SRC_RMSNORM: 1 / sqrt(mean(x^2) + eps)
+};
+
+__device__ __forceinline__ uint32_t bf16_rne(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
 
-template <int R, typename IN>
-__global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const IN* __restrict__ a, _Float16* __restrict__ afrag,
+// elements [i, i + 4) of the row as four bf16 bit patterns in two words
+template <int SRC>
+__device__ __forceinline__ void load_bf16x4(const PrepRow& row, int i, uint32_t& lo, uint32_t& hi) {
+    if (SRC == SKN_SRC_BF16) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>((const uint16_t*)row.a + i);
+        lo = v.x, hi = v.y;
+        return;
+    }
+    const float4 x = *reinterpret_cast<const float4*>((const float*)row.a + i);
+    float y[4] = {x.x, x.y, x.z, x.w};
+    if (SRC == SKN_SRC_RMSNORM) {
+        const float4 g = *reinterpret_cast<const float4*>((const float*)row.b + i);
+        y[0] = x.x * row.r * g.x, y[1] = x.y * row.r * g.y, y[2] = x.z * row.r * g.z, y[3] = x.w * row.r * g.w;
+    }
+    lo = bf16_rne(y[0]) | (bf16_rne(y[1]) << 16);
+    hi = bf16_rne(y[2]) | (bf16_rne(y[3]) << 16);
+}
+
+template <int R, int SRC>
+__global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const skn_gemm_src src, _Float16* __restrict__ afrag,
                                                             float* __restrict__ inv_scale, _Float16* __restrict__ sfrag,
                                                             int m, int k) {
     __shared__ __align__(16) u32x4 stage[512 * R];  // [chunk 64][k-step 4][half 2][row R] sixteen-byte pieces
     const int tid = threadIdx.x, lane = tid & 63, r8 = tid >> 6;
     const int row = blockIdx.x * R + r8;
     const bool real = row < m;
-    const IN* ar = a + (size_t)(real ? row : 0) * k;
+    const size_t row_off = (size_t)(real ? row : 0) * k;
+    PrepRow ar;
+    ar.a = SRC == SKN_SRC_BF16 ? (const void*)((const uint16_t*)src.a + row_off) : (const void*)((const float*)src.a + row_off);
+    ar.b = src.b;
+    ar.r = 1.f;
+    if (SRC == SKN_SRC_RMSNORM) {
+        const float* xr = (const float*)ar.a;
+        float ss = 0.f;
+        for (int i0 = 0; i0 < (k >> 2); i0 += 512) {
+            float4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = reinterpret_cast<const float4*>(xr)[min(i0 + lane + 64 * j, (k >> 2) - 1)];
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (i0 + lane + 64 * j < (k >> 2)) ss += (v[j].x * v[j].x + v[j].y * v[j].y) + (v[j].z * v[j].z + v[j].w * v[j].w);
+        }
+        ss = wave_sum(ss);
+        ar.r = 1.0f / sqrtf(ss / (float)k + src.eps);
+    }
     const int nch = k >> 6, nb = k >> 8;
     auto widen = [](uint32_t pair, int which) { return __uint_as_float(which ? pair & 0xFFFF0000u : pair << 16); };
 
@@ -205,10 +243,10 @@ __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const IN* __restric
         u32x4 v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const IN* src = ar + 8 * min(i0 + lane + 64 * j, (k >> 3) - 1);
+            const int i = 8 * min(i0 + lane + 64 * j, (k >> 3) - 1);
             uint32_t w0, w1, w2, w3;
-            load_bf16x4<IN>(src, w0, w1);
-            load_bf16x4<IN>(src + 4, w2, w3);
+            load_bf16x4<SRC>(ar, i, w0, w1);
+            load_bf16x4<SRC>(ar, i + 4, w2, w3);
             v[j] = u32x4{w0, w1, w2, w3};
         }
 #pragma unroll
@@ -237,8 +275,8 @@ __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const IN* __restric
             const int c = task >> 3, dw = task & 7;
             uint2 lo = make_uint2(0u, 0u), hi = lo;
             if (task < tasks) {
-                load_bf16x4<IN>(ar + k0 + 64 * c + 4 * dw, lo.x, lo.y);
-                load_bf16x4<IN>(ar + k0 + 64 * c + 32 + 4 * dw, hi.x, hi.y);
+                load_bf16x4<SRC>(ar, k0 + 64 * c + 4 * dw, lo.x, lo.y);
+                load_bf16x4<SRC>(ar, k0 + 64 * c + 32 + 4 * dw, hi.x, hi.y);
             }
             _Float16 l[4], u[4];
             l[0] = (_Float16)(widen(lo.x, 0) * scale), l[1] = (_Float16)(widen(lo.x, 1) * scale);
@@ -286,7 +324,8 @@ struct Q4kFragSegs {
     const uint8_t* w[3];
     float* c[3];
     int n[3];
-    int tile0[3];  // first column tile of each matrix (unused entries: n_tiles)
+    int accumulate[3];  // add to c instead of overwriting it
+    int tile0[3];       // first column tile of each matrix (unused entries: n_tiles)
     int n_tiles;
 };
 
@@ -532,7 +571,7 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 for (int o = 0; o < 3; o++)
 #pragma unroll
                     for (int x = 0; x < 16; x++) sum[x] += red[((mh * 2 * MT + t) * 3 + o) * 1024 + 64 * x + lane];
-                store_tile(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, inv_scale, lane);
+                store_tile(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, inv_scale, lane, segs.accumulate[seg] != 0);
             }
         }
 }
@@ -574,7 +613,7 @@ inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
 
-int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const void* a_dev, int a_is_f32, int m) {
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m) {
     SKN_REQUIRE(ctx, nseg >= 1 && nseg <= 3 && m > 0 && k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_ARG,
                 "Q4_K GEMM: bad segment count or shape");
     Q4kFragSegs fs;
@@ -583,12 +622,15 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
         const skn_gemm_seg& s = segs[i < nseg ? i : nseg - 1];
         SKN_REQUIRE(ctx, s.w && s.c && s.n > 0 && ((uintptr_t)s.w & 15) == 0, SKN_ERR_ARG,
                     "Q4_K GEMM: weights must be non-null and 16-byte aligned");
-        fs.w[i] = (const uint8_t*)s.w, fs.c[i] = s.c, fs.n[i] = s.n, fs.tile0[i] = tiles;
+        fs.w[i] = (const uint8_t*)s.w, fs.c[i] = s.c, fs.n[i] = s.n, fs.accumulate[i] = s.accumulate, fs.tile0[i] = tiles;
         if (i < nseg) tiles += (s.n + kBN - 1) / kBN;
     }
     for (int i = nseg; i < 3; i++) fs.tile0[i] = tiles;
     fs.n_tiles = tiles;
-    SKN_REQUIRE(ctx, ((uintptr_t)a_dev & (a_is_f32 ? 15 : 7)) == 0, SKN_ERR_ARG, "Q4_K GEMM: activations are misaligned");
+    SKN_REQUIRE(ctx, src.a && ((uintptr_t)src.a & (src.kind == SKN_SRC_BF16 ? 7 : 15)) == 0, SKN_ERR_ARG,
+                "Q4_K GEMM: activations are null or misaligned");
+    SKN_REQUIRE(ctx, src.kind == SKN_SRC_BF16 || src.kind == SKN_SRC_F32 || (src.b && ((uintptr_t)src.b & 15) == 0),
+                SKN_ERR_ARG, "Q4_K GEMM: second activation operand is null or misaligned");
     // fragment-order workspace: rows padded to whole tiles
     const int mt_rows = m > 64 ? 128 : 64;
     const int m_tiles = (m + mt_rows - 1) / mt_rows, m_pad = m_tiles * mt_rows;
@@ -600,11 +642,13 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     _Float16* afrag = (_Float16*)ws;
     _Float16* sfrag = (_Float16*)(ws + af_bytes);
     float* isc = (float*)(ws + af_bytes + sf_bytes);
-    if (a_is_f32)
-        skn_launch(ctx, prep_a_frag_kernel<4, float>, dim3(m_pad / 4), dim3(256), 0, (const float*)a_dev, afrag, isc, sfrag, m, k);
-    else
-        skn_launch(ctx, prep_a_frag_kernel<4, uint16_t>, dim3(m_pad / 4), dim3(256), 0, (const uint16_t*)a_dev, afrag, isc,
-                   sfrag, m, k);
+    const dim3 pgrid(m_pad / 4), pblock(256);
+    switch (src.kind) {
+        case SKN_SRC_BF16: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_F32: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_F32>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_RMSNORM: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_RMSNORM>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        default: return skn_fail(ctx, SKN_ERR_ARG, "Q4_K GEMM: unknown activation source %d", src.kind);
+    }
     SKN_LAUNCH_CHECK(ctx);
     if (mt_rows == 128) return launch_frag<2, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
     return launch_frag<1, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
@@ -628,8 +672,9 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     if (ggml_type == SKN_TYPE_Q4_K && k <= 16384) {
         SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
                     "skn_gemm_q: Q4_K weights must be 16-byte aligned, activations 8-byte aligned");
-        const skn_gemm_seg seg = {w_dev, n, c_dev};
-        return skn_gemm_q4k_multi(ctx, &seg, 1, k, a_bf16_dev, 0, m);
+        const skn_gemm_seg seg = {w_dev, n, c_dev, 0};
+        const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
+        return skn_gemm_q4k_multi(ctx, &seg, 1, k, src, m);
     }
 
     // workspace: fp16 activations + row scales, then (general path) the weights as an fp16 pair
