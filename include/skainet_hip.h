@@ -152,6 +152,11 @@ int skn_kv_gather(skn_ctx* ctx, skn_kv* kv, int seq, int t0, int t1, uint16_t* k
  * q/out fp32 [n_seq][n_head][head_dim] on the device; n_ctx_host[s] = tokens to attend (NULL = all cached). */
 int skn_attn_decode(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* n_ctx_host, float scale,
                     float* out_dev);
+/* The same attention for the last n_queries tokens of one sequence at once (prompt processing), causal:
+ * out[t,h,:] = softmax(q[t,h,:] . K[0:m_t,h,:]^T * scale) . V[0:m_t,h,:] with m_t = len - n_queries + t + 1.
+ * q/out fp32 [n_queries][n_head][head_dim] on the device, 16-byte aligned; head_dim 64 or 128.  No reference
+ * counterpart, like the cache itself. */
+int skn_attn_prefill(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_queries, float scale, float* out_dev);
 
 /* ---- decoder glue (fp32, device pointers) ------------------------------------------------------------ */
 

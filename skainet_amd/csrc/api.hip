@@ -78,6 +78,7 @@ void skn_shutdown(skn_ctx* ctx) {
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     if (ctx->attn_counters) (void)hipFree(ctx->attn_counters);
     if (ctx->gemm_ws) (void)hipFree(ctx->gemm_ws);
+    if (ctx->prefill_ws) (void)hipFree(ctx->prefill_ws);
     for (hipEvent_t e : ctx->prof_events) (void)hipEventDestroy(e);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);

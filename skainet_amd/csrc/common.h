@@ -34,6 +34,9 @@ struct skn_ctx {
     size_t attn_scratch_bytes = 0;
     int* attn_counters = nullptr;  // one per (sequence, head): workgroups of a split attention count themselves in
     int attn_counters_cap = 0;
+    // prompt attention workspace (K and V of a sequence in matrix-core operand order), grown on demand
+    void* prefill_ws = nullptr;
+    size_t prefill_ws_bytes = 0;
     // GEMM workspace (fp16 activations, dequantized weight pairs), grown on demand
     void* gemm_ws = nullptr;
     size_t gemm_ws_bytes = 0;

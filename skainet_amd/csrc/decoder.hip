@@ -528,7 +528,10 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
                    kv->page_tokens, log2f(c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
+        if (D <= 128)
+            SKN_TRY(skn_attn_prefill_launch(ctx, kv, 0, m->pq, T, pos0 + 1, scale, m->patt));
+        else
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
         if (q4k_attn) {  // the residual is added by the GEMM's store
             const skn_gemm_seg wo = {L.wo, H, m->px, 1};
             const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};

@@ -27,3 +27,6 @@ int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t*
 int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
                        int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev);
 int skn_attn_splits(skn_ctx* ctx, int pairs, int max_ctx);
+// Causal attention of n_queries rows of one sequence: row t attends to its first first_ctx + t tokens (head_dim 64 / 128).
+int skn_attn_prefill_launch(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_queries, int first_ctx, float scale,
+                            float* out_dev);

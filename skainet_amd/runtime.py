@@ -86,6 +86,7 @@ _SIGNATURES = {
     "skn_kv_append_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]),
     "skn_kv_gather": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "skn_attn_decode": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_float, C.c_void_p]),
+    "skn_attn_prefill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_float, C.c_void_p]),
     "skn_rmsnorm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p]),
     "skn_rope": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
     "skn_swiglu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
@@ -216,6 +217,11 @@ class KVCache:
         if n_ctx is not None and len(n_ctx) != self.n_seq:
             raise ValueError("n_ctx needs one entry per sequence")
         self.ctx._check(self.ctx.lib.skn_attn_decode(self.ctx.handle, self.handle, _ptr(q_dev), arr, scale, _ptr(out_dev)))
+
+    def attn_prefill(self, seq, q_dev, n_queries, out_dev, scale):
+        """Causal attention of the last n_queries tokens of sequence seq (q/out fp32 [n_queries][n_head][head_dim])."""
+        self.ctx._check(self.ctx.lib.skn_attn_prefill(self.ctx.handle, self.handle, int(seq), _ptr(q_dev), int(n_queries),
+                                                      scale, _ptr(out_dev)))
 
     def free(self):
         if self.handle:

@@ -212,3 +212,71 @@ def test_attention_split_counts_and_repeated_launches(hip):
     finally:
         hip.set_option("attn.splits", 0)
     kv.free()
+
+
+@pytest.mark.parametrize(
+    "n_head,dim,page,cached,n_queries",
+    [
+        (4, 128, 256, 300, 300),   # a whole prompt: row t sees t + 1 tokens
+        (2, 64, 16, 70, 70),
+        (3, 128, 48, 130, 45),     # the last 45 tokens of 130 (pages of 48: tiles straddle pages)
+        (2, 128, 32, 33, 1),       # a single row = decode attention
+        (8, 64, 64, 257, 200),
+    ],
+)
+def test_prefill_attention_vs_oracle(hip, n_head, dim, page, cached, n_queries):
+    """skn_attn_prefill: causal attention of the last n_queries tokens of a sequence, against the oracle run
+    once per row with that row's context length."""
+    kv = hip.kv_cache(2, n_head, dim, page, max(cached, page) + page)
+    k, v = _fill(hip, kv, [5, cached], seed=51)   # sequence 1 is the one attended to; 0 holds something else
+    q = np.random.default_rng(8).standard_normal((n_queries, n_head, dim)).astype(np.float32) * 2.0
+    scale = 1.0 / np.sqrt(dim)
+    out = hip.alloc(q.nbytes)
+    out.upload(np.full(q.shape, np.nan, np.float32))
+    kv.attn_prefill(1, hip.to_device(q), n_queries, out, scale)
+    got = out.download(np.float32, q.size).reshape(q.shape)
+    ctx_len = [cached - n_queries + t + 1 for t in range(n_queries)]
+    kk = np.broadcast_to(k[1][None], (n_queries,) + k[1].shape)
+    vv = np.broadcast_to(v[1][None], (n_queries,) + v[1].shape)
+    want = oracle_c.attn_decode(q, np.ascontiguousarray(kk), np.ascontiguousarray(vv), ctx_len, scale)
+    for t in range(n_queries):
+        assert oracle_np.rel_err(got[t], want[t]) <= TOL, t
+    # the same rows through the decode kernel (sequence 1, explicit context of the last row)
+    if n_queries == 1:
+        out2 = hip.alloc(2 * n_head * dim * 4)
+        q2 = np.zeros((2, n_head, dim), np.float32)
+        q2[1] = q[0]
+        kv.attn_decode(hip.to_device(q2), out2, scale, n_ctx=[0, cached])
+        dec = out2.download(np.float32, 2 * n_head * dim).reshape(2, n_head, dim)[1]
+        assert oracle_np.rel_err(got[0], dec) <= TOL
+    kv.free()
+
+
+def test_prefill_attention_arguments_and_closed_form(hip):
+    n_head, dim, tok = 2, 128, 96
+    kv = hip.kv_cache(1, n_head, dim, 32, 128)
+    k = synth.kv_f16((1, tok, n_head, dim), seed=61)
+    v = synth.kv_f16((1, tok, n_head, dim), seed=62)
+    ku = np.broadcast_to(k[:, :1], k.shape).copy()  # identical keys: row t returns the mean of V[0 : t + 1]
+    kv.append_run(0, hip.to_device(ku[0]), hip.to_device(v[0]), tok)
+    q = np.random.default_rng(9).standard_normal((tok, n_head, dim)).astype(np.float32)
+    out = hip.alloc(q.nbytes)
+    kv.attn_prefill(0, hip.to_device(q), tok, out, 0.3)
+    got = out.download(np.float32, q.size).reshape(q.shape)
+    vf = v[0].view(np.float16).astype(np.float64)
+    means = np.cumsum(vf, axis=0) / np.arange(1, tok + 1)[:, None, None]
+    assert np.abs(got - means).max() <= 1e-3 * np.abs(means).max() * 1e-3 + 2e-6
+    with pytest.raises(runtime.SknError) as e:
+        kv.attn_prefill(0, hip.to_device(q), tok + 1, out, 0.3)  # more rows than cached tokens
+    assert e.value.code == runtime.ERR_RANGE
+    with pytest.raises(runtime.SknError) as e:
+        kv.attn_prefill(3, hip.to_device(q), 1, out, 0.3)
+    assert e.value.code == runtime.ERR_RANGE
+    kv.attn_prefill(0, hip.to_device(q), 0, out, 0.3)  # no rows: a no-op
+    kv256 = hip.kv_cache(1, 1, 256, 32, 64)
+    kv256.append_run(0, hip.alloc(256 * 2 * 4), hip.alloc(256 * 2 * 4), 4)
+    with pytest.raises(runtime.SknError) as e:
+        kv256.attn_prefill(0, hip.to_device(q), 2, out, 0.3)
+    assert e.value.code == runtime.ERR_SHAPE
+    kv256.free()
+    kv.free()
