@@ -335,7 +335,7 @@ struct Q4kFragSegs {
 // out of the matrix core, and so does the "- dmin * m_j" term: one more sixteen-deep product per tile between
 // the activation sub-block sums (fp16 hi | lo) and -(dmin / cs) * m_j * 2^12, itself split into an fp16 pair.
 template <int MT, int MH>
-__global__ __launch_bounds__(256 * MH) __attribute__((amdgpu_waves_per_eu(MH, MH)))
+__global__ __launch_bounds__(256 * MH) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const Q4kFragSegs segs,
                           const float* __restrict__ inv_scale, int m, int k) {
     constexpr int kWBuf = kBN * kWPitch;
@@ -632,7 +632,14 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     SKN_REQUIRE(ctx, src.kind == SKN_SRC_BF16 || src.kind == SKN_SRC_F32 || (src.b && ((uintptr_t)src.b & 15) == 0),
                 SKN_ERR_ARG, "Q4_K GEMM: second activation operand is null or misaligned");
     // fragment-order workspace: rows padded to whole tiles
-    const int mt_rows = m > 64 ? 128 : 64;
+    // Tile rows: 128 (eight wavefronts, one workgroup per compute unit) when that gives at most one tile per
+    // compute unit; otherwise 64 with four wavefronts, two independent workgroups per compute unit -- more weight
+    // staging per product, but the two wavefronts of a SIMD no longer meet at the same barriers (measured 4-11 %
+    // faster on grids of several rounds, 3 % slower on single-round grids).
+    const int n_tiles_all = [&] { int s = 0; for (int i = 0; i < nseg; i++) s += (segs[i].n + kBN - 1) / kBN; return s; }();
+    const bool small_tiles = ctx->opt_gemm_tile == 1 ||
+                             (ctx->opt_gemm_tile == 0 && (m <= 128 || ((m + 127) / 128) * n_tiles_all > ctx->compute_units));
+    const int mt_rows = small_tiles ? 64 : 128;
     const int m_tiles = (m + mt_rows - 1) / mt_rows, m_pad = m_tiles * mt_rows;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), sf_bytes = align_up((size_t)m_pad * (k / 256) * 16 * 2);
     const size_t is_bytes = align_up((size_t)m_pad * 4);
@@ -651,7 +658,7 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     }
     SKN_LAUNCH_CHECK(ctx);
     if (mt_rows == 128) return launch_frag<2, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
-    return launch_frag<1, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
+    return launch_frag<2, 1>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
 }
 
 extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const uint16_t* a_bf16_dev,
