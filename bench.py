@@ -138,6 +138,33 @@ def bench_attention(ctx, steps, warmup):
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
+def bench_attention_prefill(ctx, reps=20):
+    """Causal attention of a 512-token prompt, 32 heads x 128 dims: 4 * T^2 / 2 * heads * dim flops of the two
+    products (each done twice, on fp16 hi + lo pairs) against the dense fp16 matrix-core peak."""
+    n_tok, n_head, dim = 512, 32, 128
+    kv = ctx.kv_cache(1, n_head, dim, 256, 1024)
+    k = ctx.to_device(synth.kv_f16((n_tok, n_head, dim), seed=150))
+    v = ctx.to_device(synth.kv_f16((n_tok, n_head, dim), seed=170))
+    kv.append_run(0, k, v, n_tok)
+    q = ctx.to_device(np.random.default_rng(192).standard_normal((n_tok, n_head, dim)).astype(np.float32))
+    out = ctx.alloc(4 * n_tok * n_head * dim)
+    scale = 1.0 / np.sqrt(dim)
+    for _ in range(3):
+        kv.attn_prefill(0, q, n_tok, out, scale)
+    ctx.sync()
+    ctx.prof_start(4 * reps)
+    for _ in range(reps):
+        kv.attn_prefill(0, q, n_tok, out, scale)
+    ms, launches = ctx.prof_stop()
+    for buf in (k, v, q, out):
+        buf.free()
+    kv.free()
+    us = ms / reps * 1e3
+    flops = 4.0 * n_tok * (n_tok + 1) / 2 * n_head * dim
+    return {"us_per_call": round(us, 1), "launches_per_call": launches // reps, "tflops_useful": round(flops / us / 1e6, 1),
+            "frac_mfma_f16_peak": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
+
+
 def bench_gemm(ctx, qtype, m, n, k, reps=20):
     """Prefill GEMM C[m,n] = A[m,k] . deq(W)[n,k]^T (A bf16): summed kernel time of one call (activation
     preparation included), 2mnk flops against the dense fp16 matrix-core peak."""
@@ -317,6 +344,7 @@ def main():
         extra["kv_cache_8x32x128"] = bench_kv(ctx)
         att = bench_attention(ctx, min(args.steps, 200), 10)
         extra["attention_8x32x128_ctx4096"] = {key: round(val, 4) for key, val in att.items()}
+        extra["prompt_attention_512x32x128"] = bench_attention_prefill(ctx)
         extra["prefill_gemm"] = {f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
                                  for nm, qt, mm, nn, kk in gemm_shapes}
         try:
