@@ -6,8 +6,9 @@
 // order in which the matrix instructions take them: per head and tile of 32 tokens, the 64 lanes x 16 bytes of
 // every operand are contiguous (K as the row operand of K . Q^T, V transposed as the row operand of V^T . P^T),
 // so the attention kernel loads an operand with one coalesced 1 KiB load and uses neither LDS nor barriers.
-// (2) attn_prefill_kernel: one wavefront per (32 query rows, head) walks the key tiles up to its causal limit
-// with the online softmax: S^T = K Q^T (scores of a query sit in one lane column: its maximum and sum need no
+// (2) attn_prefill_kernel: one workgroup of four wavefronts per (32 query rows, head); wavefront w walks the key
+// tiles w, w + 4, ... up to the causal limit with the online softmax, and the four partial results are merged
+// through LDS: S^T = K Q^T (scores of a query sit in one lane column: its maximum and sum need no
 // cross-lane traffic beyond the two lane halves), P = exp2(S - max), O^T += V^T P^T.
 // Precision: K and V are the cached fp16 values; q (pre-multiplied by scale * log2 e) and P enter as fp16 pairs
 // hi + lo (two matrix instructions per step), products and sums are fp32.
@@ -67,15 +68,16 @@ __global__ __launch_bounds__(256) void attn_frag_kernel(const uint16_t* __restri
     }
 }
 
-// grid (query blocks of 32, heads), one wavefront each; the block with the most keys first.
+// grid (query blocks of 32, heads), four wavefronts each; the block with the most keys first.
 // q, out: fp32 [n_queries][n_head][D]; query row t attends to keys [0, first_ctx + t).
 template <int D>
-__global__ __launch_bounds__(64) void attn_prefill_kernel(const float* __restrict__ q, const u32x4* __restrict__ kfrag,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(const float* __restrict__ q, const u32x4* __restrict__ kfrag,
                                                           const u32x4* __restrict__ vfrag, float* __restrict__ out,
                                                           int n_queries, int n_head, int first_ctx, int n_tiles,
                                                           float scale_log2e) {
     constexpr int KS = D / 16, DB = D / 32;
-    const int lane = threadIdx.x, h = lane >> 5, n = lane & 31;
+    __shared__ float part[3][DB * 16 + 2][64];  // running maximum, sum and accumulators of wavefronts 1..3
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = lane >> 5, n = lane & 31;
     const int qb = (int)gridDim.x - 1 - (int)blockIdx.x, head = blockIdx.y;
     const int t = min(32 * qb + n, n_queries - 1);  // (rows past the end repeat the last one and are not stored)
     const int n_ctx = first_ctx + t;                // keys this lane's query sees
@@ -107,8 +109,8 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(const float* __restric
     const u32x4* vp = vfrag + (size_t)head * n_tiles * KS * 64 + lane;
     u32x4 kf[KS];
 #pragma unroll
-    for (int s = 0; s < KS; s++) kf[s] = kp[s * 64];
-    for (int tile = 0; tile <= last_tile; tile++) {
+    for (int s = 0; s < KS; s++) kf[s] = kp[((size_t)min(wave, last_tile) * KS + s) * 64];
+    for (int tile = wave; tile <= last_tile; tile += 4) {
         u32x4 vf[KS];
 #pragma unroll
         for (int s = 0; s < KS; s++) vf[s] = vp[((size_t)tile * KS + s) * 64];
@@ -123,7 +125,7 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(const float* __restric
             sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ql[s], sc, 0, 0, 0);
         }
         // the next tile's keys (past the end: the last tile again, unused)
-        const int nt = min(tile + 1, last_tile);
+        const int nt = min(tile + 4, last_tile);
 #pragma unroll
         for (int s = 0; s < KS; s++) kf[s] = kp[((size_t)nt * KS + s) * 64];
         // causal mask and the tile maximum of this query
@@ -135,14 +137,15 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(const float* __restric
             mt = fmaxf(mt, sc[x]);
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32));
-        const float mnew = fmaxf(mrun, mt);  // finite from the first tile on: key 0 is visible to every query
-        const float alpha = exp2f(mrun - mnew);
+        const float mnew = fmaxf(mrun, mt);
+        // (a wavefront that has not met a visible key of this query yet: everything stays zero)
+        const float alpha = mnew == -INFINITY ? 1.f : exp2f(mrun - mnew);
         mrun = mnew;
         float psum = 0.f;
         half8_t ph[2], pl[2];
 #pragma unroll
         for (int x = 0; x < 16; x++) {
-            const float p = exp2f(sc[x] - mnew);
+            const float p = mnew == -INFINITY ? 0.f : exp2f(sc[x] - mnew);
             psum += p;
             _Float16 a, b;
             skn_split_hilo(p, a, b);
@@ -164,6 +167,39 @@ __global__ __launch_bounds__(64) void attn_prefill_kernel(const float* __restric
                 o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ph[s], o[b], 0, 0, 0);
                 o[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pl[s], o[b], 0, 0, 0);
             }
+    }
+    // merge: wavefronts 1..3 hand their state to wavefront 0 (which owns tile 0, where key 0 is visible to every
+    // query: its maximum is finite)
+    if (wave > 0) {
+        part[wave - 1][0][lane] = mrun;
+        part[wave - 1][1][lane] = lrun;
+#pragma unroll
+        for (int b = 0; b < DB; b++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) part[wave - 1][2 + 16 * b + x][lane] = o[b][x];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    {
+        float mall = mrun;
+#pragma unroll
+        for (int w = 0; w < 3; w++) mall = fmaxf(mall, part[w][0][lane]);
+        const float f0 = exp2f(mrun - mall);
+        lrun *= f0;
+#pragma unroll
+        for (int b = 0; b < DB; b++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) o[b][x] *= f0;
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+            const float mw = part[w][0][lane];
+            const float f = mw == -INFINITY ? 0.f : exp2f(mw - mall);
+            lrun += part[w][1][lane] * f;
+#pragma unroll
+            for (int b = 0; b < DB; b++)
+#pragma unroll
+                for (int x = 0; x < 16; x++) o[b][x] += part[w][2 + 16 * b + x][lane] * f;
+        }
     }
     const float ltot = lrun + __shfl_xor(lrun, 32);
     const float inv = ltot > 0.f ? 1.0f / ltot : 0.f;
@@ -202,7 +238,7 @@ int launch_prefill(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_
                (const uint16_t*)kv->v_pool, (const int32_t*)(kv->page_table_dev + (size_t)seq * kv->pages_per_seq), kv->n_head,
                kv->page_tokens, n_tokens, n_tiles, kfrag, vfrag);
     SKN_LAUNCH_CHECK(ctx);
-    skn_launch(ctx, attn_prefill_kernel<D>, dim3((n_queries + 31) / 32, kv->n_head), dim3(64), 0, q_dev, (const u32x4*)kfrag,
+    skn_launch(ctx, attn_prefill_kernel<D>, dim3((n_queries + 31) / 32, kv->n_head), dim3(256), 0, q_dev, (const u32x4*)kfrag,
                (const u32x4*)vfrag, out_dev, n_queries, kv->n_head, first_ctx, n_tiles, scale * 1.4426950408889634f);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
