@@ -138,8 +138,7 @@ struct skn_gemm_seg {
     int accumulate;  // c += instead of c =
 };
 int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m);
-int skn_dequant_hilo(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
-int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo);
+int skn_weights_hilo_frag(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, void* bfrag);
 
 // ---- device helpers --------------------------------------------------------------------------------
 

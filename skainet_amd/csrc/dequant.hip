@@ -8,34 +8,8 @@
 
 namespace {
 
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-
-// Where a thread's four values go: fp32 (the dequantizer proper), or split into an fp16 pair hi = f16(w),
-// lo = f16(w - hi) for the matrix-core GEMM (w = hi + lo to 2^-22 relative), without an fp32 round trip
-// through memory.
-template <bool HILO>
-__device__ __forceinline__ void put4(float* __restrict__ out, _Float16* __restrict__ hi, _Float16* __restrict__ lo,
-                                     int64_t t, const float4& y) {
-    if (!HILO) {
-        reinterpret_cast<float4*>(out)[t] = y;
-    } else {
-        const float v[4] = {y.x, y.y, y.z, y.w};
-        half4_t h, l;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            _Float16 a, b;
-            skn_split_hilo(v[i], a, b);
-            h[i] = a, l[i] = b;
-        }
-        reinterpret_cast<half4_t*>(hi)[t] = h;
-        reinterpret_cast<half4_t*>(lo)[t] = l;
-    }
-}
-
 // Q8_0: 34-byte block = f16 d @0, int8 qs[32] @2.
-template <bool HILO>
 __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           _Float16* __restrict__ out_hi, _Float16* __restrict__ out_lo,
                                                            int64_t n_quads) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_quads) return;
@@ -49,13 +23,11 @@ __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t* __rest
     y.y = __fmul_rn(d, (float)(int8_t)((q >> 8) & 0xFF));
     y.z = __fmul_rn(d, (float)(int8_t)((q >> 16) & 0xFF));
     y.w = __fmul_rn(d, (float)(int8_t)(q >> 24));
-    put4<HILO>(out, out_hi, out_lo, t, y);
+    reinterpret_cast<float4*>(out)[t] = y;
 }
 
 // Q4_K: 144-byte superblock = f16 d @0, f16 dmin @2, 12 packed 6-bit scale/min bytes @4, 128 nibble bytes @16.
-template <bool HILO>
 __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           _Float16* __restrict__ out_hi, _Float16* __restrict__ out_lo,
                                                            int64_t n_quads) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_quads) return;
@@ -85,13 +57,11 @@ __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t* __rest
     y.y = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xF)), m1);
     y.z = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xF)), m1);
     y.w = __fsub_rn(__fmul_rn(d1, (float)((q >> 24) & 0xF)), m1);
-    put4<HILO>(out, out_hi, out_lo, t, y);
+    reinterpret_cast<float4*>(out)[t] = y;
 }
 
 // Q6_K: 210-byte superblock = ql[128] @0 (low nibbles), qh[64] @128 (high bit pairs), int8 scales[16] @192, f16 d @208.
-template <bool HILO>
 __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           _Float16* __restrict__ out_hi, _Float16* __restrict__ out_lo,
                                                            int64_t n_quads) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_quads) return;
@@ -111,7 +81,7 @@ __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t* __rest
     y.y = __fmul_rn(ds, (float)((int)(((lo >> 8) & 0xF) | (((hi >> 8) & 3) << 4)) - 32));
     y.z = __fmul_rn(ds, (float)((int)(((lo >> 16) & 0xF) | (((hi >> 16) & 3) << 4)) - 32));
     y.w = __fmul_rn(ds, (float)((int)(((lo >> 24) & 0xF) | (((hi >> 24) & 3) << 4)) - 32));
-    put4<HILO>(out, out_hi, out_lo, t, y);
+    reinterpret_cast<float4*>(out)[t] = y;
 }
 
 }  // namespace
@@ -134,31 +104,12 @@ extern "C" int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64
     SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_dequant: too many elements for one launch");
     const uint8_t* w = (const uint8_t*)w_dev;
     dim3 grid((unsigned)blocks), block(256);
-    _Float16* none = nullptr;
     if (ggml_type == SKN_TYPE_Q8_0)
-        skn_launch(ctx, dequant_q8_0_kernel<false>, grid, block, 0, w, out_dev, none, none, n_quads);
+        skn_launch(ctx, dequant_q8_0_kernel, grid, block, 0, w, out_dev, n_quads);
     else if (ggml_type == SKN_TYPE_Q4_K)
-        skn_launch(ctx, dequant_q4_k_kernel<false>, grid, block, 0, w, out_dev, none, none, n_quads);
+        skn_launch(ctx, dequant_q4_k_kernel, grid, block, 0, w, out_dev, n_quads);
     else
-        skn_launch(ctx, dequant_q6_k_kernel<false>, grid, block, 0, w, out_dev, none, none, n_quads);
-    SKN_LAUNCH_CHECK(ctx);
-    return SKN_OK;
-}
-
-// Internal: the same decode written as the fp16 pair the general GEMM path multiplies with (arguments already
-// checked by skn_gemm_q; n_elems is a multiple of 4).
-int skn_dequant_hilo(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
-    if (!skn_is_core_quant(ggml_type)) return skn_dequant_hilo_other(ctx, ggml_type, w, n_elems, hi, lo);
-    const int64_t n_quads = n_elems / 4, blocks = (n_quads + 255) / 256;
-    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_gemm_q: too many weights for one launch");
-    dim3 grid((unsigned)blocks), block(256);
-    float* none = nullptr;
-    if (ggml_type == SKN_TYPE_Q8_0)
-        skn_launch(ctx, dequant_q8_0_kernel<true>, grid, block, 0, w, none, hi, lo, n_quads);
-    else if (ggml_type == SKN_TYPE_Q4_K)
-        skn_launch(ctx, dequant_q4_k_kernel<true>, grid, block, 0, w, none, hi, lo, n_quads);
-    else
-        skn_launch(ctx, dequant_q6_k_kernel<true>, grid, block, 0, w, none, hi, lo, n_quads);
+        skn_launch(ctx, dequant_q6_k_kernel, grid, block, 0, w, out_dev, n_quads);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }

@@ -209,6 +209,62 @@ struct Fmt<SKN_TYPE_IQ4_XS> {
     }
 };
 
+// The three formats with tuned kernels of their own, decoded here as well for the GEMM's weight pass (same
+// arithmetic as the dequantization kernels: every value the exact real of its formula rounded once).
+// Q8_0, 34 B: f16 d @0, int8 qs[32] @2.
+template <>
+struct Fmt<SKN_TYPE_Q8_0> {
+    static constexpr int kElems = 32, kBytes = 34;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const float d = ldh(b);
+        const uint32_t q = ld32(b + 2 + 4 * g);
+        return make_float4(__fmul_rn(d, (float)(int8_t)(q & 0xFF)), __fmul_rn(d, (float)(int8_t)((q >> 8) & 0xFF)),
+                           __fmul_rn(d, (float)(int8_t)((q >> 16) & 0xFF)), __fmul_rn(d, (float)(int8_t)(q >> 24)));
+    }
+};
+
+// Q4_K, 144 B: f16 d @0, f16 dmin @2, 12 packed 6-bit scale / min bytes @4, 128 nibble bytes @16.
+template <>
+struct Fmt<SKN_TYPE_Q4_K> {
+    static constexpr int kElems = 256, kBytes = 144;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, c = e >> 6, r = e & 63, j = 2 * c + (r >= 32);
+        const float d = ldh(b), dmin = ldh(b + 2);
+        const uint8_t* s = b + 4;
+        int sc, m;
+        if (j < 4) {
+            sc = s[j] & 63;
+            m = s[j + 4] & 63;
+        } else {
+            sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
+            m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+        }
+        uint32_t q = ld32(b + 16 + 32 * c + (r & 31));
+        if (r >= 32) q >>= 4;
+        const float d1 = __fmul_rn(d, (float)sc), m1 = __fmul_rn(dmin, (float)m);
+        return make_float4(__fsub_rn(__fmul_rn(d1, (float)(q & 0xF)), m1), __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xF)), m1),
+                           __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xF)), m1),
+                           __fsub_rn(__fmul_rn(d1, (float)((q >> 24) & 0xF)), m1));
+    }
+};
+
+// Q6_K, 210 B: ql[128] @0 (low nibbles), qh[64] @128 (high bit pairs), int8 scales[16] @192, f16 d @208.
+template <>
+struct Fmt<SKN_TYPE_Q6_K> {
+    static constexpr int kElems = 256, kBytes = 210;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, n = e >> 7, r = e & 127, quarter = r >> 5, l = r & 31;
+        uint32_t lo = ld32(b + 64 * n + l + 32 * (quarter & 1));
+        if (quarter >= 2) lo >>= 4;
+        const uint32_t hi = ld32(b + 128 + 32 * n + l) >> (2 * quarter);
+        const float ds = __fmul_rn(ldh(b + 208), (float)(int8_t)b[192 + 8 * n + 2 * quarter + (l >> 4)]);
+        return make_float4(__fmul_rn(ds, (float)((int)((lo & 0xF) | ((hi & 3) << 4)) - 32)),
+                           __fmul_rn(ds, (float)((int)(((lo >> 8) & 0xF) | (((hi >> 8) & 3) << 4)) - 32)),
+                           __fmul_rn(ds, (float)((int)(((lo >> 16) & 0xF) | (((hi >> 16) & 3) << 4)) - 32)),
+                           __fmul_rn(ds, (float)((int)(((lo >> 24) & 0xF) | (((hi >> 24) & 3) << 4)) - 32)));
+    }
+};
+
 // Dense rows, read a scalar at a time where a caller needs it and four at a time otherwise.
 template <int T>
 __device__ __forceinline__ float dense_at(const uint8_t* w, int64_t i) {
@@ -226,37 +282,64 @@ __global__ __launch_bounds__(256) void dequant_blocks_kernel(const uint8_t* __re
     reinterpret_cast<float4*>(out)[t] = Fmt<T>::decode4(w + (t / QB) * Fmt<T>::kBytes, (int)(t % QB));
 }
 
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
-// the same decode written as an fp16 pair hi = f16(w), lo = f16(w - hi) (for the GEMM)
+// four consecutive elements 4q .. 4q + 3 of a weight row
 template <int T>
-__global__ __launch_bounds__(256) void dequant_blocks_hilo_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ hi,
-                                                                  _Float16* __restrict__ lo, int64_t n_quads) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n_quads) return;
-    constexpr int QB = Fmt<T>::kElems / 4;
-    const float4 y = Fmt<T>::decode4(w + (t / QB) * Fmt<T>::kBytes, (int)(t % QB));
-    const float v[4] = {y.x, y.y, y.z, y.w};
-    half4_t h, l;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        _Float16 a, b;
-        skn_split_hilo(v[i], a, b);
-        h[i] = a, l[i] = b;
+__device__ __forceinline__ float4 row_quad(const uint8_t* row, int q) {
+    if constexpr (T == SKN_TYPE_F32 || T == SKN_TYPE_F16 || T == SKN_TYPE_BF16) {
+        return make_float4(dense_at<T>(row, 4 * q), dense_at<T>(row, 4 * q + 1), dense_at<T>(row, 4 * q + 2),
+                           dense_at<T>(row, 4 * q + 3));
+    } else {
+        constexpr int QB = Fmt<T>::kElems / 4;
+        return Fmt<T>::decode4(row + (size_t)(q / QB) * Fmt<T>::kBytes, q % QB);
     }
-    reinterpret_cast<half4_t*>(hi)[t] = h;
-    reinterpret_cast<half4_t*>(lo)[t] = l;
 }
 
 template <int T>
-__global__ __launch_bounds__(256) void convert_dense_hilo_kernel(const uint8_t* __restrict__ w, _Float16* __restrict__ hi,
-                                                                 _Float16* __restrict__ lo, int64_t n) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    _Float16 h, l;
-    skn_split_hilo(dense_at<T>(w, i), h, l);
-    hi[i] = h;
-    lo[i] = l;
+__host__ __device__ constexpr size_t row_bytes_of(int k) {
+    if constexpr (T == SKN_TYPE_F32) return (size_t)k * 4;
+    else if constexpr (T == SKN_TYPE_F16 || T == SKN_TYPE_BF16) return (size_t)k * 2;
+    else return (size_t)(k / Fmt<T>::kElems) * Fmt<T>::kBytes;
+}
+
+// The GEMM's weight pass: W [n, k] of any format -> an fp16 pair (hi = f16(w), lo = f16((w - hi) * 2^11)) in the
+// order in which the matrix-core kernel consumes it.  For a block of 32 weight rows and a k-step t (sixteen
+// elements) the 64 x 16 bytes that the 64 lanes hand to one matrix instruction are contiguous, hi operand then lo
+// operand: piece ((cb * steps + t) * 2 + hl) * 64 + 32 h + r, where lane (h, r) holds row r and -- with
+// dw = 4 h + t % 4 inside the 64-element chunk t / 4 -- the elements 4 dw + {0, 2}, 32 + 4 dw + {0, 2},
+// 4 dw + {1, 3}, 32 + 4 dw + {1, 3}: the order of the activation fragments.  lo is kept times 2^11 so that it is
+// a normal fp16 number wherever hi is one (the kernel keeps its products in accumulators of their own).
+// One thread per (row, chunk, dw): eight neighbouring threads read 64 consecutive elements of a row and a
+// wavefront writes whole 128-byte lines (the same piece of eight neighbouring rows).  Rows beyond n repeat row
+// n - 1 (their products are never stored).
+constexpr int kFragChunks = 4;  // chunks per workgroup
+template <int T>
+__global__ __launch_bounds__(256) void weights_hilo_frag_kernel(const uint8_t* __restrict__ w, half8_t* __restrict__ bfrag,
+                                                                int n, int k) {
+    const int r = threadIdx.x >> 3, dw = threadIdx.x & 7;
+    const int cb = blockIdx.y, steps = k >> 4, nch = k >> 6;
+    const uint8_t* row = w + (size_t)min(cb * 32 + r, n - 1) * row_bytes_of<T>(k);
+    const int h = dw >> 2, s = dw & 3;
+#pragma unroll
+    for (int x = 0; x < kFragChunks; x++) {
+        const int c = blockIdx.x * kFragChunks + x;
+        if (c >= nch) break;
+        const float4 l = row_quad<T>(row, 16 * c + dw), u = row_quad<T>(row, 16 * c + dw + 8);
+        const float v[8] = {l.x, l.z, u.x, u.z, l.y, l.w, u.y, u.w};
+        half8_t vh, vl;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float f = v[i];
+            asm("" : "+v"(f));  // (keeps the two conversions of a fused product apart, see skn_split_hilo)
+            const _Float16 a = (_Float16)f;
+            vh[i] = a;
+            vl[i] = (_Float16)((f - (float)a) * 2048.0f);
+        }
+        half8_t* dst = bfrag + ((size_t)cb * steps + 4 * c + s) * 128 + 32 * h + r;
+        dst[0] = vh;
+        dst[64] = vl;
+    }
 }
 
 template <int T>
@@ -353,46 +436,39 @@ int launch_matvec_dense(skn_ctx* ctx, const uint8_t* w, int n, int k, const floa
 }
 
 template <int T>
-int launch_hilo(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
-    const int64_t n_quads = n_elems / 4, blocks = (n_quads + 255) / 256;
-    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_gemm_q: too many weights for one launch");
-    skn_launch(ctx, dequant_blocks_hilo_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, hi, lo, n_quads);
-    SKN_LAUNCH_CHECK(ctx);
-    return SKN_OK;
-}
-
-template <int T>
-int launch_hilo_dense(skn_ctx* ctx, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
-    const int64_t blocks = (n_elems + 255) / 256;
-    SKN_REQUIRE(ctx, blocks <= 0x7FFFFFFF, SKN_ERR_SHAPE, "skn_gemm_q: too many weights for one launch");
-    skn_launch(ctx, convert_dense_hilo_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, w, hi, lo, n_elems);
+int launch_hilo_frag(skn_ctx* ctx, const uint8_t* w, int n, int k, void* bfrag) {
+    const dim3 grid((unsigned)(((k >> 6) + kFragChunks - 1) / kFragChunks), (unsigned)((n + 63) / 64 * 2));
+    skn_launch(ctx, weights_hilo_frag_kernel<T>, grid, dim3(256), 0, w, (half8_t*)bfrag, n, k);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
 
 }  // namespace
 
-int skn_dequant_hilo_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, _Float16* hi, _Float16* lo) {
+// Internal (arguments already checked by skn_gemm_q; k is a multiple of 64): the weights as the fp16 pair the
+// general GEMM path multiplies with, in fragment order; bfrag holds ceil(n / 64) * 64 * k * 4 bytes.
+int skn_weights_hilo_frag(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, void* bfrag) {
     switch (ggml_type) {
-        case SKN_TYPE_Q4_0: return launch_hilo<SKN_TYPE_Q4_0>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q4_1: return launch_hilo<SKN_TYPE_Q4_1>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q5_0: return launch_hilo<SKN_TYPE_Q5_0>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q5_1: return launch_hilo<SKN_TYPE_Q5_1>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q2_K: return launch_hilo<SKN_TYPE_Q2_K>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q5_K: return launch_hilo<SKN_TYPE_Q5_K>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q3_K: return launch_hilo<SKN_TYPE_Q3_K>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_Q8_K: return launch_hilo<SKN_TYPE_Q8_K>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_IQ4_NL: return launch_hilo<SKN_TYPE_IQ4_NL>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_IQ4_XS: return launch_hilo<SKN_TYPE_IQ4_XS>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_F32: return launch_hilo_dense<SKN_TYPE_F32>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_F16: return launch_hilo_dense<SKN_TYPE_F16>(ctx, w, n_elems, hi, lo);
-        case SKN_TYPE_BF16: return launch_hilo_dense<SKN_TYPE_BF16>(ctx, w, n_elems, hi, lo);
+        case SKN_TYPE_Q8_0: return launch_hilo_frag<SKN_TYPE_Q8_0>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q4_K: return launch_hilo_frag<SKN_TYPE_Q4_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q6_K: return launch_hilo_frag<SKN_TYPE_Q6_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q4_0: return launch_hilo_frag<SKN_TYPE_Q4_0>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q4_1: return launch_hilo_frag<SKN_TYPE_Q4_1>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q5_0: return launch_hilo_frag<SKN_TYPE_Q5_0>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q5_1: return launch_hilo_frag<SKN_TYPE_Q5_1>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q2_K: return launch_hilo_frag<SKN_TYPE_Q2_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q5_K: return launch_hilo_frag<SKN_TYPE_Q5_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q3_K: return launch_hilo_frag<SKN_TYPE_Q3_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_Q8_K: return launch_hilo_frag<SKN_TYPE_Q8_K>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_IQ4_NL: return launch_hilo_frag<SKN_TYPE_IQ4_NL>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_IQ4_XS: return launch_hilo_frag<SKN_TYPE_IQ4_XS>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_F32: return launch_hilo_frag<SKN_TYPE_F32>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_F16: return launch_hilo_frag<SKN_TYPE_F16>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_BF16: return launch_hilo_frag<SKN_TYPE_BF16>(ctx, w, n, k, bfrag);
         default: return skn_fail(ctx, SKN_ERR_TYPE, "skn_gemm_q: ggml type %d is not supported", ggml_type);
     }
 }
 
-namespace {
-}  // namespace
 
 // Called by skn_dequant / skn_matvec_q after their argument checks, for the types they do not handle themselves.
 int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out) {

@@ -6,10 +6,13 @@
 // Both paths below therefore feed the MFMA with operands that are exact or exact to 2^-22:
 //
 //   * Activations: bf16 -> fp16 is exact for every value whose magnitude is within fp16's normal range; each
-//     row is first scaled by a power of two that puts its largest magnitude just below 2^14 (2^10 on the Q4_K
-//     path) and the scale is undone in the epilogue.  Products and sums are fp32 inside the MFMA.
+//     row is first scaled by a power of two that puts its largest magnitude just below 2^10 and the scale is
+//     undone in the epilogue.  Products and sums are fp32 inside the MFMA.  Both paths read them in "fragment
+//     order" (see prep_a_frag_kernel): a matrix-instruction operand is one coalesced 1 KiB load, no LDS.
 //   * Weights, general path (every format but Q4_K): W is dequantized once into a workspace as an fp16 pair
-//     hi = f16(w), lo = f16(w - hi) (w_hi + w_lo = w to 2^-22 relative) and each k-step issues two MFMAs.
+//     hi = f16(w), lo = f16((w - hi) * 2^11) (hi + lo * 2^-11 = w to 2^-22 relative, or 2^-36 absolute for
+//     weights in fp16's subnormal range), also in fragment order; each k-step issues two MFMAs per tile into two
+//     sets of accumulators that are combined at the end.
 //   * Weights, Q4_K path: see gemm_q4k_frag_kernel -- the 4-bit quants times their 6-bit sub-block scale are
 //     integers below 2^10, exact in fp16, so one MFMA per k-step suffices; the f16 superblock scale d is the
 //     unit in which a column's accumulators are kept.
@@ -26,36 +29,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int kBM = 128;  // workgroup tile rows (activations)
 constexpr int kBN = 64;   // workgroup tile columns (weight rows)
-constexpr int kKC = 64;   // k elements staged in LDS per iteration
-constexpr int kRow = kKC + 8;  // LDS row pitch in halves: 144 bytes keeps 128-bit reads of 16 rows conflict-free
-
-// ---- activation preparation: bf16 [m,k] -> fp16 [m,k] with a per-row power-of-two scale -------------------
-// One workgroup per row.
-__global__ __launch_bounds__(256) void prep_a_kernel(const uint16_t* __restrict__ a, _Float16* __restrict__ a16,
-                                                     float* __restrict__ inv_scale, int k) {
-    __shared__ float red[4];
-    const int m = blockIdx.x;
-    const uint16_t* ar = a + (size_t)m * k;
-    float mx = 0.f;
-    for (int i = threadIdx.x; i < k; i += 256) {
-        const float v = fabsf(__uint_as_float((uint32_t)ar[i] << 16));
-        if (v == v && v < INFINITY) mx = fmaxf(mx, v);
-    }
-    mx = wave_max(mx);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    // the row is scaled by a power of two so that its largest magnitude lies in [2^13, 2^14): large rows fit
-    // fp16 and tiny rows do not vanish in it (a zero row keeps scale 1)
-    int e = 13;
-    if (mx > 0.f) e = max((int)((__float_as_uint(mx) >> 23) & 0xFF) - 127, -100);
-    const float scale = __uint_as_float((uint32_t)(127 + 13 - e) << 23);
-    if (threadIdx.x == 0) inv_scale[m] = __uint_as_float((uint32_t)(127 - 13 + e) << 23);
-    _Float16* out = a16 + (size_t)m * k;
-    for (int i = threadIdx.x; i < k; i += 256) out[i] = (_Float16)(__uint_as_float((uint32_t)ar[i] << 16) * scale);
-}
 
 // C tile store: acc register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the 32x32 tile
 __device__ __forceinline__ void store_tile(const float16_t& acc, float* __restrict__ c, int ldc, int row0, int col0,
@@ -70,87 +44,6 @@ __device__ __forceinline__ void store_tile(const float16_t& acc, float* __restri
             *dst = accumulate ? *dst + acc[r] * inv_scale[row] : acc[r] * inv_scale[row];
         }
     }
-}
-
-// ---- general path: dense fp16 activations x (hi + lo) fp16 weights ----------------------------------------
-// Workgroup 256 threads = 2 x 2 wavefronts; workgroup tile 128 x 64; wavefront tile 64 x 32 = two 32x32 MFMA
-// tiles sharing one pair of weight fragments.  A, W_hi, W_lo tiles of 64 k go through LDS; the next tiles are
-// fetched into registers while the current ones are consumed.
-__global__ __launch_bounds__(256) void gemm_dense_hilo_kernel(const _Float16* __restrict__ a16,
-                                                              const _Float16* __restrict__ whi,
-                                                              const _Float16* __restrict__ wlo,
-                                                              const float* __restrict__ inv_scale, float* __restrict__ c,
-                                                              int m, int n, int k) {
-    __shared__ __align__(16) _Float16 sa[kBM * kRow];
-    __shared__ __align__(16) _Float16 sh[kBN * kRow];
-    __shared__ __align__(16) _Float16 sl[kBN * kRow];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * kBM, n0 = blockIdx.x * kBN;
-
-    // global -> register staging: A tile 128 rows x 8 chunks of 16 B = 1024 chunks (4 per thread),
-    // W tiles 64 rows x 8 chunks = 512 chunks each (2 per thread)
-    uint4 ra0, ra1, ra2, ra3, rh0, rh1, rl0, rl1;
-    const int srow = tid >> 3, sch = (tid & 7) * 8;  // this thread's row (+32 per slot) and column of the tiles
-    const _Float16* ga0 = a16 + (size_t)min(m0 + srow, m - 1) * k + sch;
-    const _Float16* ga1 = a16 + (size_t)min(m0 + srow + 32, m - 1) * k + sch;
-    const _Float16* ga2 = a16 + (size_t)min(m0 + srow + 64, m - 1) * k + sch;
-    const _Float16* ga3 = a16 + (size_t)min(m0 + srow + 96, m - 1) * k + sch;
-    const size_t gw0 = (size_t)min(n0 + srow, n - 1) * k + sch;
-    const size_t gw1 = (size_t)min(n0 + srow + 32, n - 1) * k + sch;
-#define SKN_FETCH(k0)                                              \
-    do {                                                           \
-        ra0 = *reinterpret_cast<const uint4*>(ga0 + (k0));         \
-        ra1 = *reinterpret_cast<const uint4*>(ga1 + (k0));         \
-        ra2 = *reinterpret_cast<const uint4*>(ga2 + (k0));         \
-        ra3 = *reinterpret_cast<const uint4*>(ga3 + (k0));         \
-        rh0 = *reinterpret_cast<const uint4*>(whi + gw0 + (k0));   \
-        rh1 = *reinterpret_cast<const uint4*>(whi + gw1 + (k0));   \
-        rl0 = *reinterpret_cast<const uint4*>(wlo + gw0 + (k0));   \
-        rl1 = *reinterpret_cast<const uint4*>(wlo + gw1 + (k0));   \
-    } while (0)
-#define SKN_STASH()                                                                  \
-    do {                                                                             \
-        *reinterpret_cast<uint4*>(sa + srow * kRow + sch) = ra0;                     \
-        *reinterpret_cast<uint4*>(sa + (srow + 32) * kRow + sch) = ra1;              \
-        *reinterpret_cast<uint4*>(sa + (srow + 64) * kRow + sch) = ra2;              \
-        *reinterpret_cast<uint4*>(sa + (srow + 96) * kRow + sch) = ra3;              \
-        *reinterpret_cast<uint4*>(sh + srow * kRow + sch) = rh0;                     \
-        *reinterpret_cast<uint4*>(sh + (srow + 32) * kRow + sch) = rh1;              \
-        *reinterpret_cast<uint4*>(sl + srow * kRow + sch) = rl0;                     \
-        *reinterpret_cast<uint4*>(sl + (srow + 32) * kRow + sch) = rl1;              \
-    } while (0)
-
-    float16_t acc0, acc1;
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc0[r] = acc1[r] = 0.f;
-
-    SKN_FETCH(0);
-    for (int k0 = 0; k0 < k; k0 += kKC) {
-        __syncthreads();  // everyone is done reading the previous tiles
-        SKN_STASH();
-        __syncthreads();
-        if (k0 + kKC < k) SKN_FETCH(k0 + kKC);
-        const _Float16* pa0 = sa + (wm * 64 + (lane & 31)) * kRow + (lane >> 5) * 8;
-        const _Float16* pa1 = pa0 + 32 * kRow;
-        const _Float16* ph = sh + (wn * 32 + (lane & 31)) * kRow + (lane >> 5) * 8;
-        const _Float16* pl = sl + (wn * 32 + (lane & 31)) * kRow + (lane >> 5) * 8;
-#pragma unroll
-        for (int t = 0; t < kKC / 16; t++) {
-            const half8_t fa0 = *reinterpret_cast<const half8_t*>(pa0 + 16 * t);
-            const half8_t fa1 = *reinterpret_cast<const half8_t*>(pa1 + 16 * t);
-            const half8_t fh = *reinterpret_cast<const half8_t*>(ph + 16 * t);
-            const half8_t fl = *reinterpret_cast<const half8_t*>(pl + 16 * t);
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0, fh, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1, fh, acc1, 0, 0, 0);
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa0, fl, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa1, fl, acc1, 0, 0, 0);
-        }
-    }
-    store_tile(acc0, c, n, m0 + wm * 64, n0 + wn * 32, m, n, inv_scale, lane);
-    store_tile(acc1, c, n, m0 + wm * 64 + 32, n0 + wn * 32, m, n, inv_scale, lane);
-#undef SKN_FETCH
-#undef SKN_STASH
 }
 
 // ---- Q4_K path: weights unpacked in the kernel, one MFMA per k-step, operands loaded by the wavefronts ------
@@ -174,7 +67,8 @@ constexpr int kWPitch = 576;  // LDS pitch of a weight row: the 144 bytes of fou
 // converted 4096 elements at a time into LDS, laid out so that the copy to global memory writes runs of 16 R
 // bytes (the same sixteen bytes of R neighbouring rows).
 // afrag: [row block][chunk][k-step][lane] x 8 halves.  sfrag: [row block][superblock][lane] x 8 halves: the eight
-// sub-block sums of row r times 2^-12 as fp16 pairs, lanes 0..31 the "hi" parts, lanes 32..63 the "lo" parts.
+// sub-block sums of row r times 2^-12 as fp16 pairs, lanes 0..31 the "hi" parts, lanes 32..63 the "lo" parts
+// (SUMS; k must then be a multiple of 256).
 // The rows come from a source (skn_gemm_src): bf16 as given; fp32 rounded to bf16 (nearest even) on the way in;
 // or fp32 RMS-normalized first (x * r * g, r = 1 / sqrt(mean(x^2) + eps)) -- the row-wise kernel that would
 // otherwise run before the GEMM.
@@ -207,7 +101,7 @@ __device__ __forceinline__ void load_bf16x4(const PrepRow& row, int i, uint32_t&
     hi = bf16_rne(y[2]) | (bf16_rne(y[3]) << 16);
 }
 
-template <int R, int SRC>
+template <int R, int SRC, bool SUMS>
 __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const skn_gemm_src src, _Float16* __restrict__ afrag,
                                                             float* __restrict__ inv_scale, _Float16* __restrict__ sfrag,
                                                             int m, int k) {
@@ -296,7 +190,7 @@ __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const skn_gemm_src 
             o[0] = l[0], o[1] = l[2], o[2] = u[0], o[3] = u[2], o[4] = l[1], o[5] = l[3], o[6] = u[1], o[7] = u[3];
             const int h = dw >> 2, s = dw & 3;
             stage[((c * 4 + s) * 2 + h) * R + r8] = __builtin_bit_cast(u32x4, o);
-            if (dw == 0 && task < tasks) {
+            if (SUMS && dw == 0 && task < tasks) {
                 _Float16 h0, h1, l0, l1;
                 skn_split_hilo(sl * 0x1p-12f, h0, l0);
                 skn_split_hilo(su * 0x1p-12f, h1, l1);
@@ -591,6 +485,130 @@ int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfra
     return SKN_OK;
 }
 
+// ---- general path: activations x (hi + lo * 2^-11) weights, both operands loaded in fragment order ---------
+// Workgroup of four wavefronts, one per SIMD, tile (32 MT) x 64.  The tile is not divided spatially: wavefront
+// kq computes all of it over a quarter of k (k is a multiple of 64, so the k-steps divide evenly) and the four
+// partial tiles are added through LDS at the end, so no operand is loaded twice inside a workgroup.  Per k-step
+// a wavefront loads MT activation fragments and four weight fragments (two column tiles, hi and lo) -- coalesced
+// 1 KiB loads straight into the registers the matrix instructions read, D steps ahead -- and issues 4 MT matrix
+// instructions.  Consecutive workgroups on an XCD (blockIdx / 8) are the row tiles of one column tile, so a
+// weight fragment comes from memory once and from that XCD's L2 for the other row tiles.
+template <int MT, int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_hilo_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ bfrag,
+                           const float* __restrict__ inv_scale, float* __restrict__ c, int m, int n, int steps,
+                           int m_tiles, int n_tiles) {
+    extern __shared__ __align__(16) float red[];  // 2 MT tiles x 3 copies x 1024 floats
+    const int lane = threadIdx.x & 63, kq = threadIdx.x >> 6;
+    const int slot_in_xcd = blockIdx.x >> 3;
+    const int mt = slot_in_xcd % m_tiles, tn = (slot_in_xcd / m_tiles) * 8 + (blockIdx.x & 7);
+    if (tn >= n_tiles) return;
+    const int U = steps >> 2, t0 = kq * U;  // this wavefront's k-steps [t0, t0 + U)
+    const u32x4* ap = afrag + ((size_t)mt * MT * steps + t0) * 64 + lane;   // + i * steps * 64 per row block
+    const u32x4* bp = bfrag + ((size_t)tn * 2 * steps + t0) * 128 + lane;   // + j * steps * 128 per column block
+
+    u32x4 ra[D][MT], rb[D][2][2];
+    auto fetch = [&](int u, int slot) __attribute__((always_inline)) {
+        u = min(u, U - 1);
+#pragma unroll
+        for (int i = 0; i < MT; i++) ra[slot][i] = ap[((size_t)i * steps + u) * 64];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            rb[slot][j][0] = bp[((size_t)j * steps + u) * 128];
+            rb[slot][j][1] = bp[((size_t)j * steps + u) * 128 + 64];
+        }
+    };
+    float16_t acc[MT][2], accl[MT][2];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[i][j][x] = accl[i][j][x] = 0.f;
+    auto mac = [&](int slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            const half8_t fa = __builtin_bit_cast(half8_t, ra[slot][i]);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, __builtin_bit_cast(half8_t, rb[slot][j][0]), acc[i][j], 0, 0, 0);
+                accl[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, __builtin_bit_cast(half8_t, rb[slot][j][1]), accl[i][j], 0, 0, 0);
+            }
+        }
+    };
+
+    // Ring of D slots, D - 1 steps ahead: while the matrix instructions of step u run, the slot of step u - 1 --
+    // whose registers are all free by then -- is refilled, one load after every second matrix instruction.
+    // (Measured: the depth does not matter from 3 to 6 -- the loop is bound by operand delivery, 2 MiB per
+    // compute unit and tile, not by its latency.)
+#pragma unroll
+    for (int x = 0; x < D - 1; x++) fetch(x, x);
+    int u0 = 0;
+    for (; u0 + D <= U; u0 += D) {
+#pragma unroll
+        for (int x = 0; x < D; x++) {
+            fetch(u0 + x + D - 1, (x + D - 1) % D);  // (past the end: a repeat of the last step, unused)
+            mac(x);
+#pragma unroll
+            for (int g = 0; g < MT + 4; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, (4 * MT) / (MT + 4), 0);  // matrix instructions
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                    // one load
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // the last U % D steps are already in slots 0 ..
+#pragma unroll
+    for (int x = 0; x < D - 1; x++)
+        if (u0 + x < U) mac(x);
+
+    // hi + lo * 2^-11, then the four partial tiles: tile t = 2 i + j belongs to wavefront t % 4, the other three
+    // hand theirs over
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[i][j][x] += accl[i][j][x] * 0x1p-11f;
+            const int t = 2 * i + j, owner = t & 3;
+            if (kq != owner) {
+                float* dst = red + (t * 3 + ((kq - owner + 4) & 3) - 1) * 1024 + lane;
+#pragma unroll
+                for (int x = 0; x < 16; x++) dst[64 * x] = acc[i][j][x];
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = 2 * i + j;
+            if (kq == (t & 3)) {
+                float16_t sum = acc[i][j];
+#pragma unroll
+                for (int o = 0; o < 3; o++)
+#pragma unroll
+                    for (int x = 0; x < 16; x++) sum[x] += red[(t * 3 + o) * 1024 + 64 * x + lane];
+                store_tile(sum, c, n, (mt * MT + i) * 32, tn * kBN + 32 * j, m, n, inv_scale, lane);
+            }
+        }
+}
+
+template <int MT, int D>
+int launch_hilo_gemm(skn_ctx* ctx, const u32x4* afrag, const u32x4* bfrag, const float* isc, float* c, int m, int n, int k) {
+    constexpr int kLds = 2 * MT * 3 * 4096;
+    static bool opted = false;
+    if (!opted) {
+        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<MT, D>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
+        opted = true;
+    }
+    const int m_tiles = (m + 32 * MT - 1) / (32 * MT), n_tiles = (n + kBN - 1) / kBN;
+    const unsigned grid = (unsigned)(((n_tiles + 7) / 8) * 8 * m_tiles);
+    skn_launch(ctx, gemm_hilo_frag_kernel<MT, D>, dim3(grid), dim3(256), kLds, afrag, bfrag, isc, c, m, n, k >> 4, m_tiles, n_tiles);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
 int gemm_workspace(skn_ctx* ctx, size_t bytes, uint8_t** out) {
     if (bytes > ctx->gemm_ws_bytes) {
@@ -651,9 +669,9 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     float* isc = (float*)(ws + af_bytes + sf_bytes);
     const dim3 pgrid(m_pad / 4), pblock(256);
     switch (src.kind) {
-        case SKN_SRC_BF16: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
-        case SKN_SRC_F32: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_F32>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
-        case SKN_SRC_RMSNORM: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_RMSNORM>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_BF16: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_F32: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_F32, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_RMSNORM: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_RMSNORM, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
         default: return skn_fail(ctx, SKN_ERR_ARG, "Q4_K GEMM: unknown activation source %d", src.kind);
     }
     SKN_LAUNCH_CHECK(ctx);
@@ -674,7 +692,7 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     SKN_REQUIRE(ctx, c_dev != nullptr, SKN_ERR_ARG, "skn_gemm_q: c is null");
     if (k == 0) return skn_memset(ctx, c_dev, 0, (size_t)m * n * sizeof(float));
     SKN_REQUIRE(ctx, w_dev && a_bf16_dev, SKN_ERR_ARG, "skn_gemm_q: null pointer");
-    SKN_REQUIRE(ctx, k % kKC == 0, SKN_ERR_SHAPE, "skn_gemm_q: k (%d) must be a multiple of %d", k, kKC);
+    SKN_REQUIRE(ctx, k % 64 == 0, SKN_ERR_SHAPE, "skn_gemm_q: k (%d) must be a multiple of %d", k, 64);
 
     if (ggml_type == SKN_TYPE_Q4_K && k <= 16384) {
         SKN_REQUIRE(ctx, ((uintptr_t)w_dev & 15) == 0 && ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG,
@@ -684,24 +702,25 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
         return skn_gemm_q4k_multi(ctx, &seg, 1, k, src, m);
     }
 
-    // workspace: fp16 activations + row scales, then (general path) the weights as an fp16 pair
-    const size_t a16_bytes = align_up((size_t)m * k * 2), sc_bytes = align_up((size_t)m * 4);
-    const size_t wh_bytes = align_up((size_t)n * k * 2);
+    // general path.  Workspace: activations in fragment order (rows padded to whole tiles) + row scales, then
+    // the weights as an fp16 pair in fragment order (rows padded to whole 64-column tiles)
+    SKN_REQUIRE(ctx, ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG, "skn_gemm_q: activations must be 8-byte aligned");
+    const int mt = m <= 32 ? 1 : (m <= 64 ? 2 : 4);
+    const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt), n_pad = (n + kBN - 1) / kBN * kBN;
+    const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
     uint8_t* ws;
-    int rc = gemm_workspace(ctx, a16_bytes + sc_bytes + 2 * wh_bytes, &ws);
+    int rc = gemm_workspace(ctx, af_bytes + is_bytes + (size_t)n_pad * k * 4, &ws);
     if (rc != SKN_OK) return rc;
-    _Float16* a16 = (_Float16*)ws;
-    float* inv_scale = (float*)(ws + a16_bytes);
-    _Float16* whi = (_Float16*)(ws + a16_bytes + sc_bytes);
-    _Float16* wlo = (_Float16*)(ws + a16_bytes + sc_bytes + wh_bytes);
-
-    skn_launch(ctx, prep_a_kernel, dim3(m), dim3(256), 0, a_bf16_dev, a16, inv_scale, k);
+    _Float16* afrag = (_Float16*)ws;
+    float* isc = (float*)(ws + af_bytes);
+    uint8_t* bfrag = ws + af_bytes + is_bytes;
+    const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
+    _Float16* no_sums = nullptr;
+    skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16, false>, dim3(m_pad / 4), dim3(256), 0, src, afrag, isc, no_sums, m, k);
     SKN_LAUNCH_CHECK(ctx);
-    rc = skn_dequant_hilo(ctx, ggml_type, (const uint8_t*)w_dev, (int64_t)n * k, whi, wlo);
+    rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;
-    dim3 grid((n + kBN - 1) / kBN, (m + kBM - 1) / kBM);
-    skn_launch(ctx, gemm_dense_hilo_kernel, grid, dim3(256), 0, (const _Float16*)a16, (const _Float16*)whi,
-               (const _Float16*)wlo, (const float*)inv_scale, c_dev, m, n, k);
-    SKN_LAUNCH_CHECK(ctx);
-    return SKN_OK;
+    if (mt == 1) return launch_hilo_gemm<1, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
+    if (mt == 2) return launch_hilo_gemm<2, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
+    return launch_hilo_gemm<4, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
 }

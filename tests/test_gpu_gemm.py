@@ -127,6 +127,50 @@ def test_gemm_q4k_several_row_tiles_and_ragged_columns(hip):
     assert oracle_np.rel_err(got, want) <= TOL
 
 
+@pytest.mark.parametrize(
+    "m,n,k",
+    [
+        (1, 1, 64),       # one k-step per wavefront
+        (32, 31, 192),    # fewer steps than the prefetch ring holds
+        (33, 65, 320),    # two row blocks, a second column tile of one column
+        (64, 100, 448),
+        (65, 64, 1088),   # the smallest shape on 128-row tiles; steps not a multiple of the ring depth
+        (129, 130, 2112),
+        (260, 96, 6400),
+    ],
+)
+def test_gemm_general_path_shapes(hip, m, n, k):
+    """Row counts on every tile height (32, 64, 128 rows), ragged columns, and row lengths whose k-steps per
+    wavefront are below, at and off multiples of the kernel's prefetch depth (Q8_0: k a multiple of 64)."""
+    raw = synth.weight(Q8_0, n, k, seed=n + k)
+    a = synth.activation_bf16((m, k), seed=m + k)
+    got = hip.gemm_q_host(Q8_0, raw, n, k, a, m)
+    want = oracle_c.gemm_q(Q8_0, raw, n, k, a, m)
+    assert oracle_np.rel_err(got, want) <= TOL
+
+
+def test_gemm_general_path_weight_magnitudes(hip):
+    """Dense fp32 weights from 1e-4 to 4e4 (rows of one magnitude each, and rows mixing them): the fp16 pair the
+    kernel multiplies with keeps a weight to 2^-22 relative or 2^-36 absolute, whichever is larger -- the same
+    precision from fp16's subnormal range to its largest finite value."""
+    F32 = 0
+    m, n, k = 48, 96, 1024
+    rng = np.random.default_rng(31)
+    w = rng.standard_normal((n, k)).astype(np.float32)
+    scales = np.array([3e-4, 1e-3, 0.02, 1.0, 37.0, 2.0e3, 4.0e4], dtype=np.float32)
+    for r in range(n):
+        if r < 64:
+            w[r] *= scales[r % len(scales)] / 4.0  # (|N(0,1)| stays below 6 here: nothing overflows fp16)
+        else:
+            w[r] *= scales[rng.integers(len(scales) - 1, size=k)]
+    a = synth.activation_bf16((m, k), seed=32)
+    got = hip.gemm_q_host(F32, w.view(np.uint8).reshape(-1), n, k, a, m)
+    want = oracle_c.gemm_q(F32, w.view(np.uint8).reshape(-1), n, k, a, m)
+    assert np.all(np.isfinite(got))
+    for col in range(n):  # column by column: their magnitudes differ by many orders
+        assert oracle_np.rel_err(got[:, col], want[:, col]) <= TOL, col
+
+
 @pytest.mark.parametrize("n", [4096, 14336])
 def test_gemm_benchmark_shapes_q6k(hip, n):
     """M=512, K=4096 with Q6_K weights (the mixed-precision prefill case), sampled columns."""
