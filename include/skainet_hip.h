@@ -56,6 +56,8 @@ extern "C" {
 #define SKN_TYPE_IQ4_NL 20
 #define SKN_TYPE_IQ4_XS 23
 #define SKN_TYPE_BF16 30
+#define SKN_TYPE_TQ1_0 34
+#define SKN_TYPE_TQ2_0 35
 
 typedef struct skn_ctx skn_ctx;
 typedef struct skn_kv skn_kv;

@@ -20,7 +20,7 @@
  *   orc_dequant_* ..................... unpinned by the reference (it has no dequantizer); pinned by hand-built
  *                                       single-block known answers, an independent NumPy restatement
  *                                       (oracle/oracle_np.py) and the fp64 closed form rounded once
- *   deq_q4_0 ... deq_iq4_xs ........... the further formats of the reference's size table: unpinned by the reference
+ *   deq_q4_0 ... deq_tq2_0 ............ the further formats of the reference's size table: unpinned by the reference
  *                                       in the same way; pinned by hand-built tagged blocks (element order, fifth-bit
  *                                       positions, scale indices), the NumPy restatement and exact rational goldens
  *                                       (tests/golden/quant_blocks_more.npz)
@@ -44,7 +44,7 @@
 #define ORC_ERR_SHAPE (-3)
 
 enum { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8, T_Q2_K = 10, T_Q4_K = 12,
-       T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30, T_Q3_K = 11, T_Q8_K = 15, T_IQ4_NL = 20, T_IQ4_XS = 23 };
+       T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30, T_Q3_K = 11, T_Q8_K = 15, T_IQ4_NL = 20, T_IQ4_XS = 23, T_TQ1_0 = 34, T_TQ2_0 = 35 };
 
 /* ---------------------------------------------------------------- scalars */
 
@@ -146,6 +146,8 @@ int orc_type_sizes(int type, int* block_elems, int* block_bytes) {
         case T_Q8_K: *block_elems = 256; *block_bytes = 4 + 256 + 256 / 8; return ORC_OK;
         case T_IQ4_NL: *block_elems = 32; *block_bytes = 2 + 16; return ORC_OK;
         case T_IQ4_XS: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 256 / 64; return ORC_OK;
+        case T_TQ1_0: *block_elems = 256; *block_bytes = 2 + 4 * 13; return ORC_OK;
+        case T_TQ2_0: *block_elems = 256; *block_bytes = 2 + 64; return ORC_OK;
         case T_Q8_0: *block_elems = 32; *block_bytes = 2 + 32; return ORC_OK;
         case T_Q4_K: *block_elems = 256; *block_bytes = 2 + 2 + 256 / 2 + 12; return ORC_OK;
         case T_Q6_K: *block_elems = 256; *block_bytes = 2 + 256 / 2 + 256 / 4 + 256 / 16; return ORC_OK;
@@ -367,10 +369,43 @@ static void deq_iq4_xs_block(const uint8_t* b, float* y) {
     }
 }
 
+/* TQ1_0 (ternary, 1.6875 bits per weight): qs u8[48] @0, qh u8[4] @48, d f16 @52.  A byte packs five trits
+ * (four in qh) as a base-3 fraction: byte = ceil(v * 256 / 243), v = sum t_n 3^(4-n); trit n comes back as
+ * ((byte * 3^n mod 256) * 3) >> 8.  Elements: trit n of bytes 0..31 at 32 n + m, then trit n of bytes 32..47 at
+ * 160 + 16 n + m, then trit n (n < 4) of qh byte j at 240 + 4 n + j.  y = d * (t - 1). */
+static void deq_tq1_0_block(const uint8_t* b, float* y) {
+    static const uint8_t pow3[5] = {1, 3, 9, 27, 81};
+    const float d = rd_h(b + 52);
+    for (int n = 0; n < 5; n++)
+        for (int m = 0; m < 32; m++) {
+            const uint8_t q = (uint8_t)(b[m] * pow3[n]);
+            y[32 * n + m] = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+        }
+    for (int n = 0; n < 5; n++)
+        for (int m = 0; m < 16; m++) {
+            const uint8_t q = (uint8_t)(b[32 + m] * pow3[n]);
+            y[160 + 16 * n + m] = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+        }
+    for (int n = 0; n < 4; n++)
+        for (int j = 0; j < 4; j++) {
+            const uint8_t q = (uint8_t)(b[48 + j] * pow3[n]);
+            y[240 + 4 * n + j] = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+        }
+}
+
+/* TQ2_0 (ternary, 2.0625 bits per weight): qs u8[64] @0, d f16 @64.  Element 128 g + 32 l + m is bits 2l..2l+1
+ * of byte 32 g + m; y = d * (q - 1). */
+static void deq_tq2_0_block(const uint8_t* b, float* y) {
+    const float d = rd_h(b + 64);
+    for (int g = 0; g < 2; g++)
+        for (int l = 0; l < 4; l++)
+            for (int m = 0; m < 32; m++) y[128 * g + 32 * l + m] = (float)((int)((b[32 * g + m] >> (2 * l)) & 3) - 1) * d;
+}
+
 static int is_block_type(int type) {
     return type == T_Q8_0 || type == T_Q4_K || type == T_Q6_K || type == T_Q4_0 || type == T_Q4_1 || type == T_Q5_0 ||
            type == T_Q5_1 || type == T_Q2_K || type == T_Q5_K || type == T_F16 || type == T_BF16 || type == T_F32 ||
-           type == T_Q3_K || type == T_Q8_K || type == T_IQ4_NL || type == T_IQ4_XS;
+           type == T_Q3_K || type == T_Q8_K || type == T_IQ4_NL || type == T_IQ4_XS || type == T_TQ1_0 || type == T_TQ2_0;
 }
 
 static void deq_block(int type, const uint8_t* b, float* y) {
@@ -389,6 +424,8 @@ static void deq_block(int type, const uint8_t* b, float* y) {
         case T_Q8_K: deq_q8_k_block(b, y); break;
         case T_IQ4_NL: deq_iq4_nl_block(b, y); break;
         case T_IQ4_XS: deq_iq4_xs_block(b, y); break;
+        case T_TQ1_0: deq_tq1_0_block(b, y); break;
+        case T_TQ2_0: deq_tq2_0_block(b, y); break;
         case T_F16: memcpy(&h, b, 2); y[0] = orc_h2f(h); break;
         case T_BF16: memcpy(&h, b, 2); y[0] = orc_bf2f(h); break;
         default: memcpy(y, b, 4); break; /* F32 */

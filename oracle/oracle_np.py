@@ -26,6 +26,7 @@ Q8_0, Q4_K, Q6_K = 8, 12, 14
 F32, F16, BF16 = 0, 1, 30
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
 Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
+TQ1_0, TQ2_0 = 34, 35
 
 # Constants.kt:58-90 restricted to the types this library computes with: type -> (block elems, block bytes)
 QUANT_SIZES = {
@@ -45,10 +46,12 @@ QUANT_SIZES = {
     Q8_K: (256, 4 + 256 + 256 // 8),
     IQ4_NL: (32, 2 + 16),
     IQ4_XS: (256, 2 + 2 + 256 // 2 + 256 // 64),
+    TQ1_0: (256, 2 + 4 * 13),
+    TQ2_0: (256, 2 + 64),
 }
 TYPE_NAMES = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", F32: "F32", F16: "F16", BF16: "BF16", Q4_0: "Q4_0",
               Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q2_K: "Q2_K", Q5_K: "Q5_K", Q3_K: "Q3_K", Q8_K: "Q8_K",
-              IQ4_NL: "IQ4_NL", IQ4_XS: "IQ4_XS"}
+              IQ4_NL: "IQ4_NL", IQ4_XS: "IQ4_XS", TQ1_0: "TQ1_0", TQ2_0: "TQ2_0"}
 
 
 def quant_shape_to_byte_shape(shape, qtype):
@@ -247,6 +250,30 @@ def dequant_iq4_xs(raw):
     return ((_f16(b[:, 0:2])[:, None] * ls)[:, :, None] * vals).astype(np.float32).reshape(-1)
 
 
+def dequant_tq1_0(raw):
+    """Five trits per byte (four in qh) as a base-3 fraction: trit n = ((byte * 3^n mod 256) * 3) >> 8."""
+    b = _blocks(raw, TQ1_0)
+    nb = b.shape[0]
+    d = _f16(b[:, 52:54])
+
+    def trits(bytes_, count):  # [nb, m] -> [nb, count, m]
+        p3 = np.array([1, 3, 9, 27, 81], dtype=np.int64)[:count]
+        q = (bytes_.astype(np.int64)[:, None, :] * p3[None, :, None]) & 0xFF
+        return (q * 3) >> 8
+
+    t = np.concatenate([trits(b[:, 0:32], 5).reshape(nb, 160), trits(b[:, 32:48], 5).reshape(nb, 80),
+                        trits(b[:, 48:52], 4).reshape(nb, 16)], axis=1)
+    return (d[:, None] * (t - 1).astype(np.float64)).astype(np.float32).reshape(-1)
+
+
+def dequant_tq2_0(raw):
+    b = _blocks(raw, TQ2_0)
+    nb = b.shape[0]
+    qs = b[:, 0:64].reshape(nb, 2, 1, 32).astype(np.int64)
+    q = (qs >> (2 * np.arange(4))[None, None, :, None]) & 3                                  # [nb,2,4,32]
+    return (_f16(b[:, 64:66])[:, None] * (q.reshape(nb, 256) - 1).astype(np.float64)).astype(np.float32).reshape(-1)
+
+
 def dequant_f16(raw):
     return np.frombuffer(np.ascontiguousarray(raw), dtype="<f2").astype(np.float32)
 
@@ -262,6 +289,7 @@ def dequant_f32(raw):
 _DEQ = {Q8_0: dequant_q8_0, Q4_K: dequant_q4_k, Q6_K: dequant_q6_k, Q4_0: dequant_q4_0, Q4_1: dequant_q4_1,
         Q5_0: dequant_q5_0, Q5_1: dequant_q5_1, Q2_K: dequant_q2_k, Q5_K: dequant_q5_k, F16: dequant_f16,
         Q3_K: dequant_q3_k, Q8_K: dequant_q8_k, IQ4_NL: dequant_iq4_nl, IQ4_XS: dequant_iq4_xs,
+        TQ1_0: dequant_tq1_0, TQ2_0: dequant_tq2_0,
         BF16: dequant_bf16, F32: dequant_f32}
 
 

@@ -116,7 +116,8 @@ static inline bool skn_is_core_quant(int t) { return t == SKN_TYPE_Q8_0 || t == 
 static inline bool skn_is_quant(int t) {
     return skn_is_core_quant(t) || t == SKN_TYPE_Q4_0 || t == SKN_TYPE_Q4_1 || t == SKN_TYPE_Q5_0 || t == SKN_TYPE_Q5_1 ||
            t == SKN_TYPE_Q2_K || t == SKN_TYPE_Q5_K || t == SKN_TYPE_F32 || t == SKN_TYPE_F16 || t == SKN_TYPE_BF16 ||
-           t == SKN_TYPE_Q3_K || t == SKN_TYPE_Q8_K || t == SKN_TYPE_IQ4_NL || t == SKN_TYPE_IQ4_XS;
+           t == SKN_TYPE_Q3_K || t == SKN_TYPE_Q8_K || t == SKN_TYPE_IQ4_NL || t == SKN_TYPE_IQ4_XS ||
+           t == SKN_TYPE_TQ1_0 || t == SKN_TYPE_TQ2_0;
 }
 int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_elems, float* out);
 int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, const float* x, float* y);

@@ -1,5 +1,6 @@
 // The further ggml formats of the reference's size table (gguf/.../Constants.kt:58-90) that the library
-// computes with: Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS and the dense F32 / F16 / BF16.  One decode function per
+// computes with: Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, TQ1_0, TQ2_0 and the dense
+// F32 / F16 / BF16.  One decode function per
 // format -- four consecutive elements of a block at a time, every value the exact real of its formula rounded
 // once (explicitly rounded intrinsics, so no contraction can change a bit) -- serves a dequantization kernel
 // (one thread per four outputs, 16-byte stores) and a batch-1 matvec (one wavefront per row, the lane's four
@@ -206,6 +207,46 @@ struct Fmt<SKN_TYPE_IQ4_XS> {
         if (gg >= 4) q >>= 4;
         return make_float4(__fmul_rn(dl, iq4_value(q & 0xF)), __fmul_rn(dl, iq4_value((q >> 8) & 0xF)),
                            __fmul_rn(dl, iq4_value((q >> 16) & 0xF)), __fmul_rn(dl, iq4_value((q >> 24) & 0xF)));
+    }
+};
+
+// TQ1_0 (ternary), 54 B: qs[48] @0, qh[4] @48, f16 d @52.  A byte packs five trits (four in qh) as a base-3
+// fraction, byte = ceil(v * 256 / 243) with v = sum t_n 3^(4-n); trit n is ((byte * 3^n mod 256) * 3) >> 8.
+// Elements: trit n of bytes 0..31 at 32 n + m; trit n of bytes 32..47 at 160 + 16 n + m; trit n (< 4) of qh byte
+// j at 240 + 4 n + j.  y = d * (t - 1).
+template <>
+struct Fmt<SKN_TYPE_TQ1_0> {
+    static constexpr int kElems = 256, kBytes = 54;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g;
+        int n, off;
+        if (e < 160) n = e >> 5, off = e & 31;
+        else if (e < 240) n = (e - 160) >> 4, off = 32 + ((e - 160) & 15);
+        else n = (e - 240) >> 2, off = 48;
+        const uint32_t p3 = n == 0 ? 1u : n == 1 ? 3u : n == 2 ? 9u : n == 3 ? 27u : 81u;
+        const uint32_t q = ld32(b + off);
+        const float d = ldh(b + 52);
+        float y[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t t = ((((q >> (8 * i)) & 0xFFu) * p3 & 0xFFu) * 3u) >> 8;
+            y[i] = __fmul_rn((float)((int)t - 1), d);
+        }
+        return make_float4(y[0], y[1], y[2], y[3]);
+    }
+};
+
+// TQ2_0 (ternary), 66 B: qs[64] @0, f16 d @64.  Element 128 g + 32 l + m is bits 2l..2l+1 of byte 32 g + m;
+// y = d * (q - 1).
+template <>
+struct Fmt<SKN_TYPE_TQ2_0> {
+    static constexpr int kElems = 256, kBytes = 66;
+    static __device__ __forceinline__ float4 decode4(const uint8_t* b, int g) {
+        const int e = 4 * g, l = (e >> 5) & 3;
+        const uint32_t q = ld32(b + 32 * (e >> 7) + (e & 31)) >> (2 * l);
+        const float d = ldh(b + 64);
+        return make_float4(__fmul_rn((float)((int)(q & 3) - 1), d), __fmul_rn((float)((int)((q >> 8) & 3) - 1), d),
+                           __fmul_rn((float)((int)((q >> 16) & 3) - 1), d), __fmul_rn((float)((int)((q >> 24) & 3) - 1), d));
     }
 };
 
@@ -462,6 +503,8 @@ int skn_weights_hilo_frag(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, 
         case SKN_TYPE_Q8_K: return launch_hilo_frag<SKN_TYPE_Q8_K>(ctx, w, n, k, bfrag);
         case SKN_TYPE_IQ4_NL: return launch_hilo_frag<SKN_TYPE_IQ4_NL>(ctx, w, n, k, bfrag);
         case SKN_TYPE_IQ4_XS: return launch_hilo_frag<SKN_TYPE_IQ4_XS>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_TQ1_0: return launch_hilo_frag<SKN_TYPE_TQ1_0>(ctx, w, n, k, bfrag);
+        case SKN_TYPE_TQ2_0: return launch_hilo_frag<SKN_TYPE_TQ2_0>(ctx, w, n, k, bfrag);
         case SKN_TYPE_F32: return launch_hilo_frag<SKN_TYPE_F32>(ctx, w, n, k, bfrag);
         case SKN_TYPE_F16: return launch_hilo_frag<SKN_TYPE_F16>(ctx, w, n, k, bfrag);
         case SKN_TYPE_BF16: return launch_hilo_frag<SKN_TYPE_BF16>(ctx, w, n, k, bfrag);
@@ -483,6 +526,8 @@ int skn_dequant_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int64_t n_e
         case SKN_TYPE_Q8_K: return launch_dequant<SKN_TYPE_Q8_K>(ctx, w, n_elems, out);
         case SKN_TYPE_IQ4_NL: return launch_dequant<SKN_TYPE_IQ4_NL>(ctx, w, n_elems, out);
         case SKN_TYPE_IQ4_XS: return launch_dequant<SKN_TYPE_IQ4_XS>(ctx, w, n_elems, out);
+        case SKN_TYPE_TQ1_0: return launch_dequant<SKN_TYPE_TQ1_0>(ctx, w, n_elems, out);
+        case SKN_TYPE_TQ2_0: return launch_dequant<SKN_TYPE_TQ2_0>(ctx, w, n_elems, out);
         case SKN_TYPE_F32: return launch_convert<SKN_TYPE_F32>(ctx, w, n_elems, out);
         case SKN_TYPE_F16: return launch_convert<SKN_TYPE_F16>(ctx, w, n_elems, out);
         case SKN_TYPE_BF16: return launch_convert<SKN_TYPE_BF16>(ctx, w, n_elems, out);
@@ -502,6 +547,8 @@ int skn_matvec_other(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k
         case SKN_TYPE_Q8_K: return launch_matvec<SKN_TYPE_Q8_K>(ctx, w, n, k, x, y);
         case SKN_TYPE_IQ4_NL: return launch_matvec<SKN_TYPE_IQ4_NL>(ctx, w, n, k, x, y);
         case SKN_TYPE_IQ4_XS: return launch_matvec<SKN_TYPE_IQ4_XS>(ctx, w, n, k, x, y);
+        case SKN_TYPE_TQ1_0: return launch_matvec<SKN_TYPE_TQ1_0>(ctx, w, n, k, x, y);
+        case SKN_TYPE_TQ2_0: return launch_matvec<SKN_TYPE_TQ2_0>(ctx, w, n, k, x, y);
         case SKN_TYPE_F32: return launch_matvec_dense<SKN_TYPE_F32>(ctx, w, n, k, x, y);
         case SKN_TYPE_F16: return launch_matvec_dense<SKN_TYPE_F16>(ctx, w, n, k, x, y);
         case SKN_TYPE_BF16: return launch_matvec_dense<SKN_TYPE_BF16>(ctx, w, n, k, x, y);

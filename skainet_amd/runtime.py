@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libskainet_hip.so")
 F32, F16, Q8_0, Q4_K, Q6_K = 0, 1, 8, 12, 14
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K, BF16 = 2, 3, 6, 7, 10, 13, 30
 Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
+TQ1_0, TQ2_0 = 34, 35
 
 OK = 0
 ERR_ARG, ERR_TYPE, ERR_SHAPE, ERR_OOM, ERR_HIP, ERR_RANGE, ERR_POOL, ERR_STATE = -1, -2, -3, -4, -5, -6, -7, -8

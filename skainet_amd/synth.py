@@ -19,9 +19,11 @@ Q8_0, Q4_K, Q6_K = 8, 12, 14
 F32, F16, BF16 = 0, 1, 30
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
 Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
+TQ1_0, TQ2_0 = 34, 35
 BLOCK = {Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22),
          Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
-         Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136)}
+         Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136), TQ1_0: (256, 54),
+         TQ2_0: (256, 66)}
 
 
 def _f16_bytes(values):
@@ -92,7 +94,27 @@ def q8_k_blocks(n_blocks, rng):
     return b.reshape(-1)
 
 
+def tq1_0_blocks(n_blocks, rng):
+    """Valid encodings only: a byte is ceil(v * 256 / 243) for a five-trit value v (qh: four trits, then a zero)."""
+    v = rng.integers(0, 243, size=(n_blocks, 52), dtype=np.int64)
+    v[:, 48:52] = rng.integers(0, 81, size=(n_blocks, 4), dtype=np.int64) * 3
+    b = np.empty((n_blocks, 54), dtype=np.uint8)
+    b[:, 0:52] = ((v * 256 + 242) // 243).astype(np.uint8)
+    b[:, 52:54] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.01)
+    return b.reshape(-1)
+
+
+def tq2_0_blocks(n_blocks, rng):
+    q = rng.integers(0, 3, size=(n_blocks, 64, 4), dtype=np.uint8)  # two-bit fields hold 0..2
+    b = np.empty((n_blocks, 66), dtype=np.uint8)
+    b[:, 0:64] = q[:, :, 0] | (q[:, :, 1] << 2) | (q[:, :, 2] << 4) | (q[:, :, 3] << 6)
+    b[:, 64:66] = _f16_bytes(np.abs(rng.standard_normal(n_blocks)) * 0.01)
+    return b.reshape(-1)
+
+
 _GEN = {
+    TQ1_0: tq1_0_blocks,
+    TQ2_0: tq2_0_blocks,
     Q3_K: lambda n, rng: _scaled_blocks(n, rng, 110, (108,)),
     Q8_K: q8_k_blocks,
     IQ4_NL: lambda n, rng: _scaled_blocks(n, rng, 18, (0,)),

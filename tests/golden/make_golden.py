@@ -323,12 +323,46 @@ def exact_iq4_xs(b):
     return out
 
 
+def exact_tq1_0(b):
+    """Independent of the multiply-and-shift decode: a byte is the base-3 fraction byte / 256, whose first five
+    digits are the digits of floor(byte * 243 / 256)."""
+    d = _f16_exact(b[52], b[53])
+    neg = _neg(b[52], b[53])
+
+    def trit(byte, n):
+        return (int(byte) * 243 // 256) // 3 ** (4 - n) % 3
+
+    out = [None] * 256
+    for n in range(5):
+        for m in range(32):
+            out[32 * n + m] = _exact_product(d, [trit(b[m], n) - 1], neg)
+        for m in range(16):
+            out[160 + 16 * n + m] = _exact_product(d, [trit(b[32 + m], n) - 1], neg)
+    for n in range(4):
+        for j in range(4):
+            out[240 + 4 * n + j] = _exact_product(d, [trit(b[48 + j], n) - 1], neg)
+    return out
+
+
+def exact_tq2_0(b):
+    d = _f16_exact(b[64], b[65])
+    neg = _neg(b[64], b[65])
+    out = []
+    for e in range(256):
+        g, rem = divmod(e, 128)
+        l, m = divmod(rem, 32)
+        out.append(_exact_product(d, [((int(b[32 * g + m]) >> (2 * l)) & 3) - 1], neg))
+    return out
+
+
 EXACT = {synth.Q8_0: exact_q8_0, synth.Q4_K: exact_q4_k, synth.Q6_K: exact_q6_k}
 EXACT_MORE = {synth.Q4_0: exact_q4_0, synth.Q4_1: exact_q4_1, synth.Q5_0: exact_q5_0, synth.Q5_1: exact_q5_1,
               synth.Q2_K: exact_q2_k, synth.Q5_K: exact_q5_k, synth.Q3_K: exact_q3_k, synth.Q8_K: exact_q8_k,
-              synth.IQ4_NL: exact_iq4_nl, synth.IQ4_XS: exact_iq4_xs}
+              synth.IQ4_NL: exact_iq4_nl, synth.IQ4_XS: exact_iq4_xs, synth.TQ1_0: exact_tq1_0,
+              synth.TQ2_0: exact_tq2_0}
 F16_FIELDS = {synth.Q4_0: (0,), synth.Q4_1: (0, 2), synth.Q5_0: (0,), synth.Q5_1: (0, 2), synth.Q2_K: (80, 82),
-              synth.Q5_K: (0, 2), synth.Q3_K: (108,), synth.Q8_K: (), synth.IQ4_NL: (0,), synth.IQ4_XS: (0,)}
+              synth.Q5_K: (0, 2), synth.Q3_K: (108,), synth.Q8_K: (), synth.IQ4_NL: (0,), synth.IQ4_XS: (0,),
+              synth.TQ1_0: (52,), synth.TQ2_0: (64,)}
 # Q8_K keeps its scale as a float32: subnormal, smallest normal, the largest whose products stay finite, odd significands, signed zeros
 F32_EXTREMES = [0x00000001, 0x007FFFFF, 0x00800000, 0x7BFFFFFF, 0xBF800001, 0x3F800000, 0x00000000, 0x80000000,
                 0x3DCCCCCD, 0xC2F6E979]
@@ -387,7 +421,7 @@ def make_more_quant_blocks():
     rng = np.random.default_rng(20240611)
     names = {synth.Q4_0: "q4_0", synth.Q4_1: "q4_1", synth.Q5_0: "q5_0", synth.Q5_1: "q5_1", synth.Q2_K: "q2_k",
              synth.Q5_K: "q5_k", synth.Q3_K: "q3_k", synth.Q8_K: "q8_k", synth.IQ4_NL: "iq4_nl",
-             synth.IQ4_XS: "iq4_xs"}
+             synth.IQ4_XS: "iq4_xs", synth.TQ1_0: "tq1_0", synth.TQ2_0: "tq2_0"}
     f16b = lambda bits: [bits & 0xFF, bits >> 8]  # noqa: E731
     extremes = [f16b(0x0001), f16b(0x03FF), f16b(0x0400), f16b(0x7BFF), f16b(0xBC01), f16b(0x3C00), f16b(0x0000),
                 f16b(0x8000)]

@@ -1,4 +1,5 @@
-"""GPU parity for the further ggml formats (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, F16, BF16, F32) through the C ABI:
+"""GPU parity for the further ggml formats (Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, TQ1_0,
+TQ2_0, F16, BF16, F32) through the C ABI:
 dequantization bit for bit against the CPU oracle, matvec and GEMM within the 1e-3 criterion."""
 import numpy as np
 import pytest
@@ -9,7 +10,7 @@ from skainet_amd import runtime, synth
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
 MORE = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (11, "q3_k"), (15, "q8_k"),
-        (20, "iq4_nl"), (23, "iq4_xs"), (1, "f16"), (30, "bf16"), (0, "f32")]
+        (20, "iq4_nl"), (23, "iq4_xs"), (34, "tq1_0"), (35, "tq2_0"), (1, "f16"), (30, "bf16"), (0, "f32")]
 
 
 @pytest.mark.parametrize("qtype,name", MORE)
@@ -30,7 +31,7 @@ def test_dequant_random_bytes_bit_exact(hip, qtype, name):
     be, bb = synth.BLOCK[qtype]
     raw = np.random.default_rng(qtype).integers(0, 256, size=4096 * bb, dtype=np.uint8)
     for off in {2: (0,), 3: (0, 2), 6: (0,), 7: (0, 2), 10: (80, 82), 13: (0, 2), 11: (108,), 15: (2,), 20: (0,),
-                23: (0,)}[qtype]:
+                23: (0,), 34: (52,), 35: (64,)}[qtype]:
         raw.reshape(-1, bb)[:, off + 1] &= 0x7B  # (Q8_K: the top byte of its float32 scale)
     want = oracle_c.dequant(qtype, raw)
     out = hip.alloc(4 * want.size)

@@ -1,5 +1,5 @@
 """CPU: the further ggml block formats of the reference's size table (Constants.kt:58-90) -- Q4_0, Q4_1, Q5_0, Q5_1,
-Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, F16, BF16.  The reference holds only their sizes; the packing is the published ggml definition
+Q2_K, Q3_K, Q5_K, Q8_K, IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, F16, BF16.  The reference holds only their sizes; the packing is the published ggml definition
 (parity unpinned by the reference).  Pinned here by hand-built single blocks whose answers are known in closed
 form (every field tagged so that a wrong element order, bit position or scale index shows), and by bit-for-bit
 agreement of the two independently written oracles on random bytes."""
@@ -11,9 +11,10 @@ from skainet_amd import synth
 
 Q4_0, Q4_1, Q5_0, Q5_1, Q2_K, Q5_K = 2, 3, 6, 7, 10, 13
 Q3_K, Q8_K, IQ4_NL, IQ4_XS = 11, 15, 20, 23
+TQ1_0, TQ2_0 = 34, 35
 F32, F16, BF16 = 0, 1, 30
 MORE = [(Q4_0, "q4_0"), (Q4_1, "q4_1"), (Q5_0, "q5_0"), (Q5_1, "q5_1"), (Q2_K, "q2_k"), (Q5_K, "q5_k"),
-        (Q3_K, "q3_k"), (Q8_K, "q8_k"), (IQ4_NL, "iq4_nl"), (IQ4_XS, "iq4_xs"),
+        (Q3_K, "q3_k"), (Q8_K, "q8_k"), (IQ4_NL, "iq4_nl"), (IQ4_XS, "iq4_xs"), (TQ1_0, "tq1_0"), (TQ2_0, "tq2_0"),
         (F16, "f16"), (BF16, "bf16"), (F32, "f32")]
 IQ4 = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float64)
 
@@ -43,8 +44,8 @@ def test_oracles_match_golden_blocks(golden_dir, qtype, name):
 def test_sizes_match_reference_table():
     # literal numbers of reference gguf/.../Constants.kt:60-90 and the enum ids :16-48
     want = {Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2_K: (256, 84), Q5_K: (256, 176),
-            Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136),
-            F16: (1, 2), BF16: (1, 2), F32: (1, 4)}
+            Q3_K: (256, 110), Q8_K: (256, 292), IQ4_NL: (32, 18), IQ4_XS: (256, 136), TQ1_0: (256, 54),
+            TQ2_0: (256, 66), F16: (1, 2), BF16: (1, 2), F32: (1, 4)}
     for t, sz in want.items():
         assert oracle_c.type_sizes(t) == sz
         assert oracle_np.QUANT_SIZES[t] == sz
@@ -61,7 +62,7 @@ def test_oracles_agree_bitwise_on_random_blocks(qtype, name):
     else:
         # keep the fp16 fields finite (exponent field 31 is inf / nan)
         for off in {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q2_K: (80, 82), Q5_K: (0, 2), Q3_K: (108,),
-                    Q8_K: (2,), IQ4_NL: (0,), IQ4_XS: (0,)}[qtype]:
+                    Q8_K: (2,), IQ4_NL: (0,), IQ4_XS: (0,), TQ1_0: (52,), TQ2_0: (64,)}[qtype]:
             raw.reshape(-1, bb)[:, off + 1] &= 0x7B  # (Q8_K: the top byte of its float32 scale)
     both(qtype, raw)
 
@@ -238,3 +239,44 @@ def test_matvec_reduces_to_dense(qtype, name):
     assert np.array_equal(oracle_c.matvec_q(qtype, raw, n, k, x), want) or np.allclose(
         oracle_c.matvec_q(qtype, raw, n, k, x), want, rtol=1e-6)
     assert np.allclose(oracle_np.matvec_q(qtype, raw, n, k, x), want, rtol=1e-6)
+
+
+def _trits5(v):
+    return [(v // 3 ** (4 - n)) % 3 for n in range(5)]
+
+
+def test_tq1_0_trit_packing_identity():
+    """A byte stores five trits as ceil(v * 256 / 243): every one of the 243 values must come back, most
+    significant trit first, through both oracles; the fourth-trit bytes of qh hold four trits and a zero."""
+    d = f16b(0.5)
+    for base in range(0, 243, 48):
+        vals = [(base + i) % 243 for i in range(48)]
+        qs = np.array([(v * 256 + 242) // 243 for v in vals], dtype=np.uint8)
+        qh = np.array([(3 * v4 * 256 + 242) // 243 for v4 in (base % 81, 80, 0, 41)], dtype=np.uint8)
+        y = both(TQ1_0, np.concatenate([qs, qh, d]))
+        for n in range(5):
+            want = np.array([_trits5(v)[n] - 1 for v in vals]) * 0.5
+            assert np.array_equal(y[32 * n:32 * n + 32], want[:32]), (base, n)           # bytes 0..31: 32 n + m
+            assert np.array_equal(y[160 + 16 * n:176 + 16 * n], want[32:]), (base, n)    # bytes 32..47: 160 + 16 n + m
+        for n in range(4):
+            want = np.array([_trits5(3 * v4)[n] - 1 for v4 in (base % 81, 80, 0, 41)]) * 0.5
+            assert np.array_equal(y[240 + 4 * n:244 + 4 * n], want), (base, n)           # qh: 240 + 4 n + j
+
+
+def test_tq2_0_element_order():
+    # byte 32 g + m holds elements 128 g + 32 l + m in bit pairs l = 0..3
+    qs = np.zeros(64, np.uint8)
+    want = np.zeros(256)
+    rng = np.random.default_rng(7)
+    for g in range(2):
+        for m in range(32):
+            t = rng.integers(0, 3, size=4)
+            qs[32 * g + m] = t[0] | (t[1] << 2) | (t[2] << 4) | (t[3] << 6)
+            for l in range(4):
+                want[128 * g + 32 * l + m] = (t[l] - 1) * -0.25
+    y = both(TQ2_0, np.concatenate([qs, f16b(-0.25)]))
+    assert np.array_equal(y, want.astype(np.float32))
+    # all fields 1 -> zeros carrying the sign of d; all fields 2 -> +d; all 0 -> -d
+    for fill, val in ((0x55, 0.0), (0xAA, -0.25), (0x00, 0.25)):
+        y = both(TQ2_0, np.concatenate([np.full(64, fill, np.uint8), f16b(-0.25)]))
+        assert np.all(y == val)
