@@ -400,7 +400,26 @@ __global__ __launch_bounds__(256) void matvec_blocks_kernel(const uint8_t* __res
     constexpr int QB = Fmt<T>::kElems / 4;
     const uint8_t* rowp = w + (size_t)row * (k / Fmt<T>::kElems) * Fmt<T>::kBytes;
     float acc = 0.f;
-    for (int q = lane; q < (k >> 2); q += 64) {
+    const int nq = k >> 2;
+    int q = lane;
+    // four quads per lane and turn: their loads are issued together, the row is read with four requests in flight
+    for (; q + 192 < nq; q += 256) {
+        float4 wv[4], xv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int qq = q + 64 * u;
+            wv[u] = Fmt<T>::decode4(rowp + (size_t)(qq / QB) * Fmt<T>::kBytes, qq % QB);
+            xv[u] = reinterpret_cast<const float4*>(x)[qq];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            acc = fmaf(wv[u].x, xv[u].x, acc);
+            acc = fmaf(wv[u].y, xv[u].y, acc);
+            acc = fmaf(wv[u].z, xv[u].z, acc);
+            acc = fmaf(wv[u].w, xv[u].w, acc);
+        }
+    }
+    for (; q < nq; q += 64) {
         const float4 wv = Fmt<T>::decode4(rowp + (size_t)(q / QB) * Fmt<T>::kBytes, q % QB);
         const float4 xv = reinterpret_cast<const float4*>(x)[q];
         acc = fmaf(wv.x, xv.x, acc);
@@ -436,6 +455,22 @@ __global__ __launch_bounds__(256) void matvec_dense_kernel(const uint8_t* __rest
                 acc = fmaf(lo, xs8[2 * i], acc);
                 acc = fmaf(hi, xs8[2 * i + 1], acc);
             }
+        }
+        done = k;
+    }
+    if (T == SKN_TYPE_F32 && (k & 3) == 0 && ((uintptr_t)w & 15) == 0) {
+        // four fp32 weights per 128-bit load, two loads in flight per lane and turn
+        const float4* w4 = reinterpret_cast<const float4*>(rowp);
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+        int o = lane;
+        for (; o + 64 < (k >> 2); o += 128) {
+            const float4 a0 = w4[o], a1 = w4[o + 64], b0 = x4[o], b1 = x4[o + 64];
+            acc = fmaf(a0.x, b0.x, acc), acc = fmaf(a0.y, b0.y, acc), acc = fmaf(a0.z, b0.z, acc), acc = fmaf(a0.w, b0.w, acc);
+            acc = fmaf(a1.x, b1.x, acc), acc = fmaf(a1.y, b1.y, acc), acc = fmaf(a1.z, b1.z, acc), acc = fmaf(a1.w, b1.w, acc);
+        }
+        for (; o < (k >> 2); o += 64) {
+            const float4 a0 = w4[o], b0 = x4[o];
+            acc = fmaf(a0.x, b0.x, acc), acc = fmaf(a0.y, b0.y, acc), acc = fmaf(a0.z, b0.z, acc), acc = fmaf(a0.w, b0.w, acc);
         }
         done = k;
     }
