@@ -33,22 +33,25 @@ __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t* __rest
     if (t >= n_quads) return;
     int64_t blk = t >> 6;    // 64 quads per 256-element superblock
     int e = (int)(t & 63) * 4;  // first element of this quad inside the superblock
-    const uint8_t* b = w + blk * 144;
-    const uint32_t* b32 = reinterpret_cast<const uint32_t*>(b);  // superblocks are 16-byte aligned
-    uint32_t dd = b32[0];
-    float d = h2f_bits(dd & 0xFFFF), dmin = h2f_bits(dd >> 16);
+    // superblocks are 16-byte aligned: the whole header (d, dmin, twelve scale / min bytes) is one 128-bit load
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const u32x4* b128 = reinterpret_cast<const u32x4*>(w + blk * 144);
+    const u32x4 hdr = b128[0];
+    float d = h2f_bits(hdr.x & 0xFFFF), dmin = h2f_bits(hdr.x >> 16);
     int c = e >> 6, r = e & 63;
     int j = 2 * c + (r >= 32);
-    const uint8_t* s = b + 4;
+    // bytes 0..3 of the twelve: low scales, 4..7: low mins, 8..11: low nibbles of the high ones, whose top two
+    // bits sit in bits 6..7 of the first eight bytes
+    const int sh = 8 * (j & 3);
     int sc, m;
     if (j < 4) {
-        sc = s[j] & 63;
-        m = s[j + 4] & 63;
+        sc = (hdr.y >> sh) & 63;
+        m = (hdr.z >> sh) & 63;
     } else {
-        sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4);
-        m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+        sc = ((hdr.w >> sh) & 0x0F) | (((hdr.y >> (sh + 6)) & 3) << 4);
+        m = ((hdr.w >> (sh + 4)) & 0x0F) | (((hdr.z >> (sh + 6)) & 3) << 4);
     }
-    uint32_t q = b32[4 + 8 * c + ((r & 31) >> 2)];
+    uint32_t q = reinterpret_cast<const uint32_t*>(b128)[4 + 8 * c + ((r & 31) >> 2)];
     if (r >= 32) q >>= 4;
     float d1 = __fmul_rn(d, (float)sc);
     float m1 = __fmul_rn(dmin, (float)m);
