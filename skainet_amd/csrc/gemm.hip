@@ -470,16 +470,17 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
         }
 }
 
-// the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in once
+// the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in per
+// device by skn_gemm_init
+template <int MT, int MH>
+constexpr int frag_lds_bytes() {
+    return 2 * kBN * kWPitch > MT * MH * 24576 ? 2 * kBN * kWPitch : MT * MH * 24576;
+}
+
 template <int MT, int MH>
 int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfrag, const Q4kFragSegs& segs, const float* isc,
                 int m, int k) {
-    constexpr int kLds = 2 * kBN * kWPitch > MT * MH * 24576 ? 2 * kBN * kWPitch : MT * MH * 24576;
-    static bool opted = false;
-    if (!opted) {
-        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<MT, MH>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        opted = true;
-    }
+    constexpr int kLds = frag_lds_bytes<MT, MH>();
     skn_launch(ctx, gemm_q4k_frag_kernel<MT, MH>, dim3(m_tiles * segs.n_tiles), dim3(256 * MH), kLds, afrag, sfrag, segs, isc, m, k);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
@@ -597,11 +598,6 @@ void gemm_hilo_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restr
 template <int MT, int D>
 int launch_hilo_gemm(skn_ctx* ctx, const u32x4* afrag, const u32x4* bfrag, const float* isc, float* c, int m, int n, int k) {
     constexpr int kLds = 2 * MT * 3 * 4096;
-    static bool opted = false;
-    if (!opted) {
-        SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<MT, D>, hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-        opted = true;
-    }
     const int m_tiles = (m + 32 * MT - 1) / (32 * MT), n_tiles = (n + kBN - 1) / kBN;
     const unsigned grid = (unsigned)(((n_tiles + 7) / 8) * 8 * m_tiles);
     skn_launch(ctx, gemm_hilo_frag_kernel<MT, D>, dim3(grid), dim3(256), kLds, afrag, bfrag, isc, c, m, n, k >> 4, m_tiles, n_tiles);
@@ -630,6 +626,17 @@ int gemm_workspace(skn_ctx* ctx, size_t bytes, uint8_t** out) {
 inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 }  // namespace
+
+// Dynamic LDS above 48 KiB must be allowed per kernel and device; done once per context here so that no launch
+// path has to.
+int skn_gemm_init(skn_ctx* ctx) {
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 2>()));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 1>()));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<2, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
+    return SKN_OK;
+}
 
 int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m) {
     SKN_REQUIRE(ctx, nseg >= 1 && nseg <= 3 && m > 0 && k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_ARG,
