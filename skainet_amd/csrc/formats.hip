@@ -351,21 +351,24 @@ __host__ __device__ constexpr size_t row_bytes_of(int k) {
 // dw = 4 h + t % 4 inside the 64-element chunk t / 4 -- the elements 4 dw + {0, 2}, 32 + 4 dw + {0, 2},
 // 4 dw + {1, 3}, 32 + 4 dw + {1, 3}: the order of the activation fragments.  lo is kept times 2^11 so that it is
 // a normal fp16 number wherever hi is one (the kernel keeps its products in accumulators of their own).
-// One thread per (row, chunk, dw): eight neighbouring threads read 64 consecutive elements of a row and a
-// wavefront writes whole 128-byte lines (the same piece of eight neighbouring rows).  Rows beyond n repeat row
-// n - 1 (their products are never stored).
+// One thread per (row, chunk, dw): eight neighbouring threads read 64 consecutive elements of a row.  The
+// pieces of the workgroup's 32 rows x kFragChunks chunks -- one contiguous 8 KiB run of the output per chunk -- are
+// collected in LDS and written out in order, 1 KiB per wavefront store.  Rows beyond n repeat row n - 1 (their
+// products are never stored).
 constexpr int kFragChunks = 4;  // chunks per workgroup
 template <int T>
 __global__ __launch_bounds__(256) void weights_hilo_frag_kernel(const uint8_t* __restrict__ w, half8_t* __restrict__ bfrag,
                                                                 int n, int k) {
+    __shared__ half8_t stage[kFragChunks * 512];
     const int r = threadIdx.x >> 3, dw = threadIdx.x & 7;
     const int cb = blockIdx.y, steps = k >> 4, nch = k >> 6;
     const uint8_t* row = w + (size_t)min(cb * 32 + r, n - 1) * row_bytes_of<T>(k);
     const int h = dw >> 2, s = dw & 3;
+    const int c0 = blockIdx.x * kFragChunks, chunks = min(kFragChunks, nch - c0);
 #pragma unroll
     for (int x = 0; x < kFragChunks; x++) {
-        const int c = blockIdx.x * kFragChunks + x;
-        if (c >= nch) break;
+        if (x >= chunks) break;
+        const int c = c0 + x;
         const float4 l = row_quad<T>(row, 16 * c + dw), u = row_quad<T>(row, 16 * c + dw + 8);
         const float v[8] = {l.x, l.z, u.x, u.z, l.y, l.w, u.y, u.w};
         half8_t vh, vl;
@@ -377,10 +380,13 @@ __global__ __launch_bounds__(256) void weights_hilo_frag_kernel(const uint8_t* _
             vh[i] = a;
             vl[i] = (_Float16)((f - (float)a) * 2048.0f);
         }
-        half8_t* dst = bfrag + ((size_t)cb * steps + 4 * c + s) * 128 + 32 * h + r;
+        half8_t* dst = stage + x * 512 + s * 128 + 32 * h + r;
         dst[0] = vh;
         dst[64] = vl;
     }
+    __syncthreads();
+    half8_t* out = bfrag + ((size_t)cb * steps + 4 * c0) * 128;
+    for (int i = threadIdx.x; i < chunks * 512; i += 256) out[i] = stage[i];
 }
 
 template <int T>
