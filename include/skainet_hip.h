@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define SKN_ABI_VERSION 1
+#define SKN_ABI_VERSION 2
 
 #define SKN_OK 0
 #define SKN_ERR_ARG (-1)    /* null pointer, negative size, bad handle */
@@ -101,7 +101,7 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
 /* Launch-shape tuning knobs, 0 = library default: "q4k.waves" (wavefronts per workgroup of the Q4_K matvec),
  * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention),
  * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel),
- * "llama.fused" (1 = fused per-layer kernels in the decode step when every layer matrix is Q4_K, the default). */
+ * "llama.fused" (1 = fused per-layer kernels in the decode step for the Q4_K matrices, the default). */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
 int skn_timer_start(skn_ctx* ctx);
@@ -199,7 +199,9 @@ typedef struct skn_llama_layer {
     const void* w_gate; const void* w_up;                            /* [ffn, hidden] */
     const void* w_down;                                              /* [hidden, ffn] */
     const float* attn_norm; const float* ffn_norm;                   /* [hidden] */
-    int32_t type_attn; int32_t type_ffn;                             /* ggml type ids of the matrices */
+    /* ggml type id of each matrix (files quantized with a mix give some matrices of a layer more bits) */
+    int32_t type_q; int32_t type_k; int32_t type_v; int32_t type_o;
+    int32_t type_gate; int32_t type_up; int32_t type_down;
 } skn_llama_layer;
 
 typedef struct skn_llama_weights {

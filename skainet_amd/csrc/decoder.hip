@@ -20,7 +20,6 @@ struct skn_llama {
     int32_t* tokens_out = nullptr;  // device array of produced tokens
     int tokens_cap = 0;
     int pos = 0;                    // host mirror of the position
-    bool fused = false;             // every layer matrix is Q4_K with k <= 16384: the fused decode path applies
     // prompt buffers (grown to the longest prompt seen)
     int prompt_cap = 0;
     float *px = nullptr, *pxn = nullptr, *pq = nullptr, *pk = nullptr, *pv = nullptr, *patt = nullptr, *pproj = nullptr;
@@ -293,9 +292,15 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
-        if (m->fused && ctx->opt_llama_fused) {
-            // five launches per layer: [norm + q,k,v + rope + cache store], attention, [Wo + residual],
-            // [norm + gate,up + SwiGLU], [Wdown + residual]
+        // Five launches per layer where the matrices are Q4_K: [norm + q,k,v + rope + cache store], attention,
+        // [Wo + residual], [norm + gate,up + SwiGLU], [Wdown + residual].  A group with a matrix of another
+        // type takes that type's matvec and the row-wise kernels around it.
+        const bool fuse = ctx->opt_llama_fused && H <= 16384;
+        const bool f_qkv = fuse && L.type_q == SKN_TYPE_Q4_K && L.type_k == SKN_TYPE_Q4_K && L.type_v == SKN_TYPE_Q4_K;
+        const bool f_o = fuse && L.type_o == SKN_TYPE_Q4_K;
+        const bool f_gu = fuse && L.type_gate == SKN_TYPE_Q4_K && L.type_up == SKN_TYPE_Q4_K;
+        const bool f_down = fuse && F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
+        if (f_qkv) {
             skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, H, H}};
             skn_rope_epilogue rope;
             rope.pos_dev = m->state + 1;
@@ -307,38 +312,46 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2f(c.rope_base);
             SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, 3 * H, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope));
-            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
+        } else {
+            skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
+            SKN_LAUNCH_CHECK(ctx);
+            SKN_TRY(skn_matvec_q(ctx, L.type_q, L.wq, H, H, m->xn, m->q));
+            SKN_TRY(skn_matvec_q(ctx, L.type_k, L.wk, H, H, m->xn, m->k));
+            SKN_TRY(skn_matvec_q(ctx, L.type_v, L.wv, H, H, m->xn, m->v));
+            skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
+                       kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                       kv->page_tokens, log2f(c.rope_base));
+            SKN_LAUNCH_CHECK(ctx);
+        }
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
+        if (f_o) {
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));
+        } else {
+            SKN_TRY(skn_matvec_q(ctx, L.type_o, L.wo, H, H, m->att, m->proj));
+            skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
+            SKN_LAUNCH_CHECK(ctx);
+        }
+        if (f_gu) {
             skn_q4k_segments gu = {{(const uint8_t*)L.w_gate, (const uint8_t*)L.w_up, nullptr}, {F, F, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU));
+        } else {
+            skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.ffn_norm, m->xn, H, c.rms_eps);
+            SKN_LAUNCH_CHECK(ctx);
+            SKN_TRY(skn_matvec_q(ctx, L.type_gate, L.w_gate, F, H, m->xn, m->gate));
+            SKN_TRY(skn_matvec_q(ctx, L.type_up, L.w_up, F, H, m->xn, m->up));
+            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk(F)), dim3(256), 0, (const float*)m->gate, (const float*)m->up,
+                       m->mid, (int64_t)F);
+            SKN_LAUNCH_CHECK(ctx);
+        }
+        if (f_down) {
             skn_q4k_segments wd = {{(const uint8_t*)L.w_down, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD));
-            continue;
+        } else {
+            SKN_TRY(skn_matvec_q(ctx, L.type_down, L.w_down, H, F, m->mid, m->proj));
+            skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
+            SKN_LAUNCH_CHECK(ctx);
         }
-        skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
-        SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wq, H, H, m->xn, m->q));
-        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wk, H, H, m->xn, m->k));
-        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wv, H, H, m->xn, m->v));
-        skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
-                   kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
-                   kv->page_tokens, log2f(c.rope_base));
-        SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
-        SKN_TRY(skn_matvec_q(ctx, L.type_attn, L.wo, H, H, m->att, m->proj));
-        skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
-        SKN_LAUNCH_CHECK(ctx);
-        skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.ffn_norm, m->xn, H, c.rms_eps);
-        SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_gate, F, H, m->xn, m->gate));
-        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_up, F, H, m->xn, m->up));
-        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk(F)), dim3(256), 0, (const float*)m->gate, (const float*)m->up,
-                   m->mid, (int64_t)F);
-        SKN_LAUNCH_CHECK(ctx);
-        SKN_TRY(skn_matvec_q(ctx, L.type_ffn, L.w_down, H, F, m->mid, m->proj));
-        skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
-        SKN_LAUNCH_CHECK(ctx);
     }
     skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, m->w.out_norm, m->xn, H, c.rms_eps);
     SKN_LAUNCH_CHECK(ctx);
@@ -415,8 +428,10 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
         const skn_llama_layer& L = w->layers[l];
         SKN_REQUIRE(ctx, L.wq && L.wk && L.wv && L.wo && L.w_gate && L.w_up && L.w_down && L.attn_norm && L.ffn_norm,
                     SKN_ERR_ARG, "skn_llama_create: layer %d has a null weight", l);
-        SKN_REQUIRE(ctx, skn_is_quant(L.type_attn) && skn_is_quant(L.type_ffn), SKN_ERR_TYPE,
-                    "skn_llama_create: layer %d has an unsupported weight type", l);
+        SKN_REQUIRE(ctx,
+                    skn_is_quant(L.type_q) && skn_is_quant(L.type_k) && skn_is_quant(L.type_v) && skn_is_quant(L.type_o) &&
+                        skn_is_quant(L.type_gate) && skn_is_quant(L.type_up) && skn_is_quant(L.type_down),
+                    SKN_ERR_TYPE, "skn_llama_create: layer %d has an unsupported weight type", l);
     }
     skn_llama* m = new (std::nothrow) skn_llama();
     SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_OOM, "skn_llama_create: host allocation failed");
@@ -440,9 +455,6 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
         m->k = m->q + H;
         m->v = m->q + 2 * H;
     }
-    m->fused = cfg->hidden <= 16384 && cfg->ffn <= 16384;
-    for (int l = 0; l < cfg->n_layer; l++)
-        if (m->layers[l].type_attn != SKN_TYPE_Q4_K || m->layers[l].type_ffn != SKN_TYPE_Q4_K) m->fused = false;
     A(&m->gate, F); A(&m->up, F); A(&m->mid, F); A(&m->logits, (size_t)cfg->vocab);
     A(&m->attn_partial, (size_t)cfg->n_head * max_splits * (cfg->head_dim + 2));
     A(&m->attn_counters, (size_t)cfg->n_head);
@@ -508,10 +520,12 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
         // Q4_K weights: the GEMM's preparation pass takes the fp32 rows and does the row-wise work before them
-        const bool q4k_attn = L.type_attn == SKN_TYPE_Q4_K && H <= 16384;
-        const bool q4k_ffn = L.type_ffn == SKN_TYPE_Q4_K && H <= 16384 && F <= 16384;
+        const bool q4k_qkv = H <= 16384 && L.type_q == SKN_TYPE_Q4_K && L.type_k == SKN_TYPE_Q4_K && L.type_v == SKN_TYPE_Q4_K;
+        const bool q4k_o = H <= 16384 && L.type_o == SKN_TYPE_Q4_K;
+        const bool q4k_gu = H <= 16384 && L.type_gate == SKN_TYPE_Q4_K && L.type_up == SKN_TYPE_Q4_K;
+        const bool q4k_down = F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
-        if (q4k_attn) {  // RMSNorm inside the activation pass, one launch for the three projections
+        if (q4k_qkv) {  // RMSNorm inside the activation pass, one launch for the three projections
             const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq, 0}, {L.wk, H, m->pk, 0}, {L.wv, H, m->pv, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.attn_norm, c.rms_eps};
             SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, src, T));
@@ -519,9 +533,9 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wq, H, H, m->pb16, T, m->pq));
-            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wk, H, H, m->pb16, T, m->pk));
-            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wv, H, H, m->pb16, T, m->pv));
+            SKN_TRY(skn_gemm_q(ctx, L.type_q, L.wq, H, H, m->pb16, T, m->pq));
+            SKN_TRY(skn_gemm_q(ctx, L.type_k, L.wk, H, H, m->pb16, T, m->pk));
+            SKN_TRY(skn_gemm_q(ctx, L.type_v, L.wv, H, H, m->pb16, T, m->pv));
         }
         skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
                    kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
@@ -532,40 +546,40 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             SKN_TRY(skn_attn_prefill_launch(ctx, kv, 0, m->pq, T, pos0 + 1, scale, m->patt));
         else
             SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
-        if (q4k_attn) {  // the residual is added by the GEMM's store
+        if (q4k_o) {  // the residual is added by the GEMM's store
             const skn_gemm_seg wo = {L.wo, H, m->px, 1};
             const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};
             SKN_TRY(skn_gemm_q4k_multi(ctx, &wo, 1, H, src, T));
         } else {
             SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_attn, L.wo, H, H, m->pb16, T, m->pproj));
+            SKN_TRY(skn_gemm_q(ctx, L.type_o, L.wo, H, H, m->pb16, T, m->pproj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
                        (int64_t)T * H);
             SKN_LAUNCH_CHECK(ctx);
         }
-        if (q4k_ffn) {
+        if (q4k_gu) {
             const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pgate, 0}, {L.w_up, F, m->pup, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.ffn_norm, c.rms_eps};
             SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, src, T));
-            // (SwiGLU stays a kernel of its own: inside the activation pass, which runs one wavefront per row,
-            // its exponentials cost more than the separate element-wise launch)
-            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
-                       (const float*)m->pup, m->pmid, (int64_t)T * F);
-            SKN_LAUNCH_CHECK(ctx);
-            const skn_gemm_seg down = {L.w_down, H, m->px, 1};  // residual added by the store
-            const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, mid, T));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_gate, F, H, m->pb16, T, m->pgate));
-            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_up, F, H, m->pb16, T, m->pup));
-            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
-                       (const float*)m->pup, m->pmid, (int64_t)T * F);
-            SKN_LAUNCH_CHECK(ctx);
+            SKN_TRY(skn_gemm_q(ctx, L.type_gate, L.w_gate, F, H, m->pb16, T, m->pgate));
+            SKN_TRY(skn_gemm_q(ctx, L.type_up, L.w_up, F, H, m->pb16, T, m->pup));
+        }
+        // (SwiGLU stays a kernel of its own: inside the activation pass, which runs one wavefront per row, its
+        // exponentials cost more than the separate element-wise launch)
+        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                   (const float*)m->pup, m->pmid, (int64_t)T * F);
+        SKN_LAUNCH_CHECK(ctx);
+        if (q4k_down) {
+            const skn_gemm_seg down = {L.w_down, H, m->px, 1};  // residual added by the store
+            const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
+            SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, mid, T));
+        } else {
             SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
-            SKN_TRY(skn_gemm_q(ctx, L.type_ffn, L.w_down, H, F, m->pb16, T, m->pproj));
+            SKN_TRY(skn_gemm_q(ctx, L.type_down, L.w_down, H, F, m->pb16, T, m->pproj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
                        (int64_t)T * H);
             SKN_LAUNCH_CHECK(ctx);

@@ -7,7 +7,7 @@ Module.kt:6-16, nn/topology/MLP.kt:13-19) instantiated for a Llama block stack; 
 from __future__ import annotations
 
 import ctypes as C
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import numpy as np
 
@@ -27,10 +27,17 @@ class Config:
     page_tokens: int = 256
     rope_base: float = 10000.0
     rms_eps: float = 1e-5
-    type_attn: int = Q4_K
-    type_ffn: int = Q4_K
+    type_attn: int = Q4_K   # wq, wk, wv, wo unless overridden below
+    type_ffn: int = Q4_K    # w_gate, w_up, w_down unless overridden below
     type_embd: int = Q4_K
     type_head: int = Q6_K
+    # Per-matrix overrides, the way mixed quantizations give some matrices more bits: keys are a matrix name
+    # ("wv", "w_down", ...) for every layer or "l<layer>.<name>" for one layer.
+    matrix_types: dict = field(default_factory=dict)
+
+    def matrix_type(self, layer: int, name: str) -> int:
+        default = self.type_attn if name in ("wq", "wk", "wv", "wo") else self.type_ffn
+        return self.matrix_types.get(f"l{layer}.{name}", self.matrix_types.get(name, default))
 
 
 LLAMA_7B = Config()
@@ -47,10 +54,11 @@ def random_weights(cfg: Config, seed: int):
     for l in range(cfg.n_layer):
         s = seed + 100 * (l + 1)
         for i, name in enumerate(("wq", "wk", "wv", "wo")):
-            w[f"l{l}.{name}"] = (cfg.type_attn, synth.weight(cfg.type_attn, h, h, s + i))
-        w[f"l{l}.w_gate"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, f, h, s + 10))
-        w[f"l{l}.w_up"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, f, h, s + 11))
-        w[f"l{l}.w_down"] = (cfg.type_ffn, synth.weight(cfg.type_ffn, h, f, s + 12))
+            t = cfg.matrix_type(l, name)
+            w[f"l{l}.{name}"] = (t, synth.weight(t, h, h, s + i))
+        for i, (name, rows, cols) in enumerate((("w_gate", f, h), ("w_up", f, h), ("w_down", h, f))):
+            t = cfg.matrix_type(l, name)
+            w[f"l{l}.{name}"] = (t, synth.weight(t, rows, cols, s + 10 + i))
         w[f"l{l}.attn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
         w[f"l{l}.ffn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
     return w
@@ -76,7 +84,9 @@ class LlamaModel:
             L = layers[l]
             for f in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "attn_norm", "ffn_norm"):
                 setattr(L, f, self.bufs[f"l{src}.{f}"].ptr)
-            L.type_attn, L.type_ffn = cfg.type_attn, cfg.type_ffn
+            for f, tf in (("wq", "type_q"), ("wk", "type_k"), ("wv", "type_v"), ("wo", "type_o"), ("w_gate", "type_gate"),
+                          ("w_up", "type_up"), ("w_down", "type_down")):
+                setattr(L, tf, weights[f"l{src}.{f}"][0])  # the type each matrix was built with
         self._layers = layers
         wts = LlamaWeights(self.bufs["tok_embd"].ptr, self.bufs["out_norm"].ptr, self.bufs["out_head"].ptr,
                            cfg.type_embd, cfg.type_head, layers)
@@ -123,5 +133,9 @@ class LlamaModel:
             be, bb = synth.BLOCK[t]
             return n * (k // be) * bb
 
-        per_layer = 4 * rb(c.type_attn, c.hidden, c.hidden) + 2 * rb(c.type_ffn, c.ffn, c.hidden) + rb(c.type_ffn, c.hidden, c.ffn)
-        return c.n_layer * per_layer + rb(c.type_head, c.vocab, c.hidden)
+        total = rb(c.type_head, c.vocab, c.hidden)
+        for l in range(c.n_layer):
+            total += sum(rb(c.matrix_type(l, nm), c.hidden, c.hidden) for nm in ("wq", "wk", "wv", "wo"))
+            total += sum(rb(c.matrix_type(l, nm), c.ffn, c.hidden) for nm in ("w_gate", "w_up"))
+            total += rb(c.matrix_type(l, "w_down"), c.hidden, c.ffn)
+        return total

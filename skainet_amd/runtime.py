@@ -41,7 +41,8 @@ class LlamaLayer(C.Structure):
         ("wq", C.c_void_p), ("wk", C.c_void_p), ("wv", C.c_void_p), ("wo", C.c_void_p),
         ("w_gate", C.c_void_p), ("w_up", C.c_void_p), ("w_down", C.c_void_p),
         ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p),
-        ("type_attn", C.c_int32), ("type_ffn", C.c_int32),
+        ("type_q", C.c_int32), ("type_k", C.c_int32), ("type_v", C.c_int32), ("type_o", C.c_int32),
+        ("type_gate", C.c_int32), ("type_up", C.c_int32), ("type_down", C.c_int32),
     ]
 
 

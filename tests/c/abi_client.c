@@ -18,7 +18,7 @@
 
 static int host_leg(void) {
     int elems = 0, bytes = 0;
-    CHECK(skn_abi_version() == 1);
+    CHECK(skn_abi_version() == 2);
     CHECK(skn_type_block(SKN_TYPE_Q4_K, &elems, &bytes) == SKN_OK && elems == 256 && bytes == 144);
     CHECK(skn_type_block(SKN_TYPE_Q8_0, &elems, &bytes) == SKN_OK && elems == 32 && bytes == 34);
     CHECK(skn_type_block(SKN_TYPE_Q6_K, &elems, &bytes) == SKN_OK && elems == 256 && bytes == 210);

@@ -15,6 +15,14 @@ TOL = 2e-3
 SMALL = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, head_dim=128, vocab=512, max_tokens=96, page_tokens=16)
 
 
+# A mix as files quantized with "more bits for some matrices" have it: every group of a layer (q/k/v, wo, gate/up,
+# down) appears once all-Q4_K and once with another type.  (Chosen among such mixes for its conditioning: a
+# random-weight stack amplifies the bf16 rounding of the prompt pass, for this one by about 5 as for SMALL; with
+# Q6_K value projections the oracle's own bf16 and fp32 prompt passes differ by more than 10 %.)
+MIXED = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, head_dim=128, vocab=512, max_tokens=96, page_tokens=16,
+                     matrix_types={"l0.wq": 8, "l0.w_down": 13, "l1.wo": 8, "l1.w_gate": 7})
+
+
 def _margin_ok(logits, tol_abs):
     s = np.sort(logits)
     return (s[-1] - s[-2]) > 2 * tol_abs
@@ -57,6 +65,42 @@ def test_prefill_then_decode_matches_oracle(hip):
             assert got[i] == want, i
         else:
             break
+        tok = want
+    model.free()
+
+
+def test_mixed_matrix_types_match_oracle(hip):
+    """Per-matrix weight types: the fused Q4_K kernels serve the groups that are all Q4_K, the others take their
+    type's kernels -- decode steps, then a prompt pass followed by decode steps, against the oracle."""
+    w = llama.random_weights(MIXED, seed=21)
+    assert [w[k][0] for k in ("l0.wq", "l0.wk", "l0.w_down", "l1.wo", "l1.w_gate", "l1.w_up")] == [8, 12, 13, 8, 7, 12]
+    model = llama.LlamaModel(hip, MIXED, weights=w)
+    ora = OracleLlama(MIXED, w)
+    tok = 11
+    for step in range(18):
+        got = model.decode(tok, 1)[0]
+        want = ora.step(tok)
+        err = oracle_np.rel_err(model.logits(), ora.logits)
+        assert err <= TOL, (step, err)
+        if _margin_ok(ora.logits, TOL * np.abs(ora.logits).max()):
+            assert got == want, step
+        tok = want
+    model.reset()
+    ora = OracleLlama(MIXED, w)
+    prompt = np.random.default_rng(2).integers(0, MIXED.vocab, size=41).tolist()
+    got_next = model.prefill(prompt)
+    want_next = ora.prefill(prompt, bf16_gemm=True)
+    err = oracle_np.rel_err(model.logits(), ora.logits)
+    assert err <= 5e-3, err
+    if _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+        assert got_next == want_next
+    got = model.decode(want_next, 6)
+    tok = want_next
+    for i in range(6):
+        want = ora.step(tok)
+        if not _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+            break
+        assert got[i] == want, i
         tok = want
     model.free()
 
