@@ -105,6 +105,39 @@ def test_mixed_matrix_types_match_oracle(hip):
     model.free()
 
 
+def test_full_7b_shape_matches_oracle(hip):
+    """The benchmark's model shape (32 layers, hidden 4096, FFN 11008, 32 heads x 128, vocabulary 32000, Q4_K
+    layers, Q6_K head) at full size: decode steps and a short prompt pass against the oracle.  Every layer points
+    at the same seeded weights so that the host holds one layer (the device holds 32 copies)."""
+    cfg = llama.Config(max_tokens=64, page_tokens=16)
+    one = llama.random_weights(llama.Config(**{**cfg.__dict__, "n_layer": 1}), seed=11)
+    w = dict(one)
+    for l in range(1, cfg.n_layer):
+        for nm in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down", "attn_norm", "ffn_norm"):
+            w[f"l{l}.{nm}"] = one[f"l0.{nm}"]
+    model = llama.LlamaModel(hip, cfg, weights=w)
+    ora = OracleLlama(cfg, w)
+    tok = 1234
+    for step in range(3):
+        got = model.decode(tok, 1)[0]
+        want = ora.step(tok)
+        err = oracle_np.rel_err(model.logits(), ora.logits)
+        assert err <= TOL, (step, err)
+        if _margin_ok(ora.logits, TOL * np.abs(ora.logits).max()):
+            assert got == want, step
+        tok = want
+    model.reset()
+    ora = OracleLlama(cfg, w)
+    prompt = [31999, 0, 17, 4096, 12869]
+    got_next = model.prefill(prompt)
+    want_next = ora.prefill(prompt, bf16_gemm=True)
+    err = oracle_np.rel_err(model.logits(), ora.logits)
+    assert err <= 5e-3, err
+    if _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+        assert got_next == want_next
+    model.free()
+
+
 def test_graph_replay_equals_eager(hip):
     w = llama.random_weights(SMALL, seed=9)
     model = llama.LlamaModel(hip, SMALL, weights=w)
