@@ -139,7 +139,9 @@ struct skn_gemm_seg {
     float* c;
     int accumulate;  // c += instead of c =
 };
-int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m);
+// swiglu_pair: segs[0], segs[1] are the gate and up matrices of a SwiGLU; silu(gate) * up goes to segs[0].c ([m, n])
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m,
+                       bool swiglu_pair = false);
 int skn_weights_hilo_frag(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, void* bfrag);
 
 // ---- device helpers --------------------------------------------------------------------------------

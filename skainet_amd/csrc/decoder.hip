@@ -557,22 +557,20 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
                        (int64_t)T * H);
             SKN_LAUNCH_CHECK(ctx);
         }
-        if (q4k_gu) {
-            const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pgate, 0}, {L.w_up, F, m->pup, 0}};
+        if (q4k_gu) {  // RMSNorm inside the activation pass, SwiGLU inside the store: gate and up never reach memory
+            const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pmid, 0}, {L.w_up, F, m->pmid, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.ffn_norm, c.rms_eps};
-            SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, src, T));
+            SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, src, T, true));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_gate, L.w_gate, F, H, m->pb16, T, m->pgate));
             SKN_TRY(skn_gemm_q(ctx, L.type_up, L.w_up, F, H, m->pb16, T, m->pup));
+            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                       (const float*)m->pup, m->pmid, (int64_t)T * F);
+            SKN_LAUNCH_CHECK(ctx);
         }
-        // (SwiGLU stays a kernel of its own: inside the activation pass, which runs one wavefront per row, its
-        // exponentials cost more than the separate element-wise launch)
-        skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
-                   (const float*)m->pup, m->pmid, (int64_t)T * F);
-        SKN_LAUNCH_CHECK(ctx);
         if (q4k_down) {
             const skn_gemm_seg down = {L.w_down, H, m->px, 1};  // residual added by the store
             const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};

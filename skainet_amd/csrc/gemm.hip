@@ -221,6 +221,9 @@ struct Q4kFragSegs {
     int accumulate[3];  // add to c instead of overwriting it
     int tile0[3];       // first column tile of each matrix (unused entries: n_tiles)
     int n_tiles;
+    // pair != 0: w[0], w[1] are the gate and up matrices of a SwiGLU; a tile holds the same 32 columns of both
+    // (its two 32-column halves) and stores silu(gate) * up into c[0]
+    int pair;
 };
 
 // Accumulators: acc holds the running sum of a column in units of cs = d * 2^14 of the latest superblock whose d
@@ -241,11 +244,12 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     // tile -> (row tile, weight matrix, column tile): the column tiles of up to three matrices sharing the
     // activations are laid side by side
     const int mt = blockIdx.x / segs.n_tiles, tn = blockIdx.x - mt * segs.n_tiles;
-    const int seg = tn >= segs.tile0[2] ? 2 : (tn >= segs.tile0[1] ? 1 : 0);
+    const bool pair = segs.pair != 0;
+    const int seg = pair ? 0 : (tn >= segs.tile0[2] ? 2 : (tn >= segs.tile0[1] ? 1 : 0));
     const uint8_t* __restrict__ w = segs.w[seg];
     float* __restrict__ c = segs.c[seg];
     const int n = segs.n[seg];
-    const int mb0 = (MH * mt + mh) * MT, n0 = (tn - segs.tile0[seg]) * kBN;
+    const int mb0 = (MH * mt + mh) * MT, n0 = pair ? tn * 32 : (tn - segs.tile0[seg]) * kBN;
 
     // Weight staging, global memory straight into LDS: a wavefront-wide load fills 64 sixteen-byte slots
     // i * 64 + lane; slot P holds piece P % 36 of tile row P / 36 (36 pieces = the 576 bytes of four
@@ -258,7 +262,8 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
             if (i < 36) {
                 const int p = i * 64 + lane, row = p / 36, col = p - 36 * row;
                 const int off = min(g * 576 + col * 16, nb * 144 - 16);  // (a short last group repeats the row's last piece)
-                const uint8_t* src = w + (size_t)min(n0 + row, n - 1) * nb * 144 + off;
+                const uint8_t* wsrc = pair && row >= 32 ? segs.w[1] : w;  // (pair: tile rows 32.. are the up matrix)
+                const uint8_t* src = wsrc + (size_t)min(n0 + (pair ? row & 31 : row), n - 1) * nb * 144 + off;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                                  (__attribute__((address_space(3))) void*)(lds + buf * kWBuf + i * 1024), 16, 0, 0);
             }
@@ -439,23 +444,51 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
 #pragma unroll
             for (int x = 0; x < 16; x++) acc[i][j][x] *= cs[j];
 
-    // add the four partial tiles of each half: tile t = 2 i + j belongs to wavefront kq = t % 4 of its half, the
-    // other three hand theirs over
+    // Add the four partial tiles of each half.  Tile t = 2 i + j belongs to wavefront kq = t % 4 of its half and
+    // the other three hand theirs over.  Pair: the two column halves of row block i are needed together, so
+    // wavefront i % 4 takes accumulator registers 0..7 of both and wavefront (i + 2) % 4 registers 8..15.
     float* red = reinterpret_cast<float*>(lds);
 #pragma unroll
     for (int i = 0; i < MT; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int t = 2 * i + j, owner = t & 3;
-            if (kq != owner) {
-                float* dst = red + ((mh * 2 * MT + t) * 3 + ((kq - owner + 4) & 3) - 1) * 1024 + lane;
+            const int t = 2 * i + j;
 #pragma unroll
-                for (int x = 0; x < 16; x++) dst[64 * x] = acc[i][j][x];
+            for (int xh = 0; xh < 2; xh++) {
+                const int owner = pair ? (i + 2 * xh) & 3 : t & 3;
+                if (kq != owner) {
+                    float* dst = red + ((mh * 2 * MT + t) * 3 + ((kq - owner + 4) & 3) - 1) * 1024 + lane;
+#pragma unroll
+                    for (int x = 8 * xh; x < 8 * xh + 8; x++) dst[64 * x] = acc[i][j][x];
+                }
             }
         }
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < MT; i++)
+    for (int i = 0; i < MT; i++) {
+        if (pair) {
+#pragma unroll
+            for (int xh = 0; xh < 2; xh++)
+                if (kq == ((i + 2 * xh) & 3)) {
+                    const int col = n0 + (lane & 31);
+#pragma unroll
+                    for (int x = 8 * xh; x < 8 * xh + 8; x++) {
+                        float g = acc[i][0][x], u = acc[i][1][x];
+#pragma unroll
+                        for (int o = 0; o < 3; o++) {
+                            g += red[((mh * 2 * MT + 2 * i) * 3 + o) * 1024 + 64 * x + lane];
+                            u += red[((mh * 2 * MT + 2 * i + 1) * 3 + o) * 1024 + 64 * x + lane];
+                        }
+                        // register x of lane l: row 8 (x / 4) + 4 (l / 32) + x % 4 of the 32 x 32 tile
+                        const int row = (mb0 + i) * 32 + 8 * (x >> 2) + 4 * (lane >> 5) + (x & 3);
+                        if (row < m && col < n) {
+                            const float a = g * inv_scale[row];
+                            c[(size_t)row * n + col] = a / (1.0f + expf(-a)) * (u * inv_scale[row]);  // silu(gate) * up
+                        }
+                    }
+                }
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int t = 2 * i + j;
@@ -468,6 +501,7 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 store_tile(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, inv_scale, lane, segs.accumulate[seg] != 0);
             }
         }
+    }
 }
 
 // the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in per
@@ -638,9 +672,12 @@ int skn_gemm_init(skn_ctx* ctx) {
     return SKN_OK;
 }
 
-int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m) {
+int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m,
+                       bool swiglu_pair) {
     SKN_REQUIRE(ctx, nseg >= 1 && nseg <= 3 && m > 0 && k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_ARG,
                 "Q4_K GEMM: bad segment count or shape");
+    SKN_REQUIRE(ctx, !swiglu_pair || (nseg == 2 && segs[0].n == segs[1].n && !segs[0].accumulate), SKN_ERR_ARG,
+                "Q4_K GEMM: a SwiGLU pair is two matrices of the same shape");
     Q4kFragSegs fs;
     int tiles = 0;
     for (int i = 0; i < 3; i++) {
@@ -651,7 +688,8 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
         if (i < nseg) tiles += (s.n + kBN - 1) / kBN;
     }
     for (int i = nseg; i < 3; i++) fs.tile0[i] = tiles;
-    fs.n_tiles = tiles;
+    fs.n_tiles = swiglu_pair ? (segs[0].n + 31) / 32 : tiles;
+    fs.pair = swiglu_pair ? 1 : 0;
     SKN_REQUIRE(ctx, src.a && ((uintptr_t)src.a & (src.kind == SKN_SRC_BF16 ? 7 : 15)) == 0, SKN_ERR_ARG,
                 "Q4_K GEMM: activations are null or misaligned");
     SKN_REQUIRE(ctx, src.kind == SKN_SRC_BF16 || src.kind == SKN_SRC_F32 || (src.b && ((uintptr_t)src.b & 15) == 0),
@@ -661,7 +699,7 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     // compute unit; otherwise 64 with four wavefronts, two independent workgroups per compute unit -- more weight
     // staging per product, but the two wavefronts of a SIMD no longer meet at the same barriers (measured 4-11 %
     // faster on grids of several rounds, 3 % slower on single-round grids).
-    const int n_tiles_all = [&] { int s = 0; for (int i = 0; i < nseg; i++) s += (segs[i].n + kBN - 1) / kBN; return s; }();
+    const int n_tiles_all = fs.n_tiles;
     const bool small_tiles = ctx->opt_gemm_tile == 1 ||
                              (ctx->opt_gemm_tile == 0 && (m <= 128 || ((m + 127) / 128) * n_tiles_all > ctx->compute_units));
     const int mt_rows = small_tiles ? 64 : 128;
