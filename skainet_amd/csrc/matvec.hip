@@ -597,17 +597,15 @@ struct Q4kRopeCtx {
 };
 
 __device__ __forceinline__ Q4kRopeCtx q4k_rope_prepare(const skn_q4k_segments& seg, const skn_rope_epilogue& rope,
-                                                     int unit) {
+                                                     int unit, int pos, int page) {
     Q4kRopeCtx c;
     int row = unit * 2;  // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
     c.which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
     row -= c.which == 2 ? seg.rows[0] + seg.rows[1] : c.which == 1 ? seg.rows[0] : 0;
     c.h = row / rope.head_dim;
     c.e = row % rope.head_dim;
-    const int pos = rope.pos_dev[0];
-    const int pi = pos / rope.page_tokens;
-    c.slot = pos - pi * rope.page_tokens;
-    c.page = rope.page_table[pi];
+    c.slot = pos % rope.page_tokens;
+    c.page = page;
     const float inv_freq = exp2f(-(float)c.e / (float)rope.head_dim * rope.log2_base);
     sincosf((float)pos * inv_freq, &c.sn, &c.cs);
     return c;
@@ -669,6 +667,10 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int n4 = nb * 64;
     constexpr int J = 2 * STEPS;  // 512 threads x J float4 cover k <= STEPS * 4096
 
+    // rotary epilogue: the position and, once it is known, the page id of its cache row are requested here (two
+    // dependent round trips) so that neither is waited for after the staging barrier
+    int rope_pos = 0, rope_page = 0;
+    if (EPI == SKN_EPI_ROPE) rope_pos = rope.pos_dev[0];
     Q4kStage<J> st, nw;
     q4k_stage_load<J>(x, n4, tid, 512, st);
     if (NORM) q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
@@ -715,6 +717,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         }
     };
     issue(0, 0);
+    if (EPI == SKN_EPI_ROPE) rope_page = rope.page_table[rope_pos / rope.page_tokens];
 
     // RMSNorm: y = sum_k W[., k] * (x_k * r * g_k) = r * sum_k W[., k] * (x_k * g_k): x * g is staged and the row
     // totals are multiplied by r = 1 / sqrt(mean(x^2) + eps) at the end, so the sum of squares needs no
@@ -739,7 +742,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     __syncthreads();
     // (after the staging, while the first weights are still on their way)
     Q4kRopeCtx rc;
-    if (EPI == SKN_EPI_ROPE) rc = q4k_rope_prepare(seg, rope, min(unit, (n_out + 1) / 2 - 1));
+    if (EPI == SKN_EPI_ROPE) rc = q4k_rope_prepare(seg, rope, min(unit, (n_out + 1) / 2 - 1), rope_pos, rope_page);
     float rinv = 1.0f;
     if (NORM) {
         const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
