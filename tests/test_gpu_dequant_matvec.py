@@ -101,6 +101,49 @@ def test_matvec_vs_oracle(hip, qtype, n, k):
     assert err <= TOL, f"rel err {err}"
 
 
+@pytest.mark.parametrize("nb", [16, 17, 32, 33, 48, 49, 64, 65, 144])
+def test_matvec_q4k_step_boundaries(hip, nb):
+    """Q4_K rows of exactly 1, 2, 3 and 4 sixteen-superblock steps and one superblock past each (the unrolled
+    kernels end at 64; 144 superblocks is the longest row whose staging fits the LDS), with row counts around the
+    rows a workgroup takes."""
+    k = 256 * nb
+    for n in (1, 7, 8, 9, 15, 16, 17, 31):
+        raw = synth.weight(Q4_K, n, k, seed=nb * 100 + n)
+        x = synth.activation_f32(k, seed=nb + n)
+        got = hip.matvec_q_host(Q4_K, raw, n, k, x)
+        want = oracle_c.matvec_q(Q4_K, raw, n, k, x)
+        assert oracle_np.rel_err(got, want) <= TOL, (nb, n)
+
+
+def test_matvec_extreme_activations(hip):
+    """fp32 activations towards the ends of the range: zeros, 1e-28 (the Q4_K kernel works in units of 2^-24 and
+    flushes what is smaller than about 2^-100), 1e30, one huge element among small ones."""
+    n, k = 24, 4096
+    rng = np.random.default_rng(77)
+    for qtype in (Q8_0, Q4_K, Q6_K):
+        raw = synth.weight(qtype, n, k, seed=qtype)
+        for kind in range(5):
+            x = rng.standard_normal(k).astype(np.float32)
+            if kind == 0:
+                x[:] = 0.0
+            elif kind == 1:
+                x *= 1e-28
+            elif kind == 2:
+                x *= 1e30
+            elif kind == 3:
+                x *= 1e-6
+                x[1234] = 3.0e8
+            else:
+                x[::2] = 0.0
+            got = hip.matvec_q_host(qtype, raw, n, k, x)
+            want = oracle_c.matvec_q(qtype, raw, n, k, x)
+            assert np.all(np.isfinite(got)), (qtype, kind)
+            if kind == 0:
+                assert np.all(got == 0.0)
+            else:
+                assert oracle_np.rel_err(got, want) <= TOL, (qtype, kind)
+
+
 @pytest.mark.parametrize("qtype", [Q8_0, Q4_K, Q6_K])
 def test_matvec_one_hot_and_linearity(hip, qtype):
     n, k = 64, 2048
