@@ -234,10 +234,14 @@ struct Q4kFragSegs {
 template <int MT, int MH>
 __global__ __launch_bounds__(256 * MH) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const Q4kFragSegs segs,
-                          const float* __restrict__ inv_scale, int m, int k) {
+                          const float* __restrict__ inv_scale, int m, int k, uint32_t a_bytes) {
     constexpr int kWBuf = kBN * kWPitch;
     extern __shared__ __align__(16) uint8_t lds[];  // max(2 kWBuf, MT x 48 KiB) bytes
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // (the wavefront's index as a scalar: everything derived from it -- its row blocks, its superblocks, the
+    // base addresses of its fragments -- then lives in scalar registers, and a fragment load is scalar base +
+    // lane offset instead of a 64-bit vector add per load)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kq = wave & 3, mh = wave >> 2;
     const int h = lane >> 5, r = lane & 31;
     const int nb = k >> 8, nch = k >> 6, groups = (nb + 3) >> 2;
@@ -270,15 +274,19 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
         }
     };
 
-    const u32x4* ap[MT];
+    // The activation fragments are read with buffer loads: a scalar byte offset (row block, k-step) plus the
+    // lane's sixteen bytes, no vector address arithmetic per load.
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void*)afrag, 0, (int)a_bytes, 0x00020000);
+    uint32_t abase[MT];  // byte offset of the row block's first fragment
 #pragma unroll
-    for (int i = 0; i < MT; i++) ap[i] = afrag + (size_t)(mb0 + i) * nch * 256 + lane;
+    for (int i = 0; i < MT; i++) abase[i] = (uint32_t)(mb0 + i) * (uint32_t)nch * 4096u;
     // activation fragments: a ring of eight k-steps; the slot of step t is refilled with step t + 8 as soon as
     // the matrix instructions of step t are issued
     u32x4 a[8][MT];
     auto afetch = [&](int step, int slot) __attribute__((always_inline)) {  // step: 16 per superblock, absolute
 #pragma unroll
-        for (int i = 0; i < MT; i++) a[slot][i] = ap[i][(size_t)step * 64];
+        for (int i = 0; i < MT; i++)
+            a[slot][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, lane * 16, (int)(abase[i] + (uint32_t)step * 1024u), 0));
     };
     float16_t acc[MT][2];
     float cs[2] = {1.f, 1.f};
@@ -515,7 +523,8 @@ template <int MT, int MH>
 int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfrag, const Q4kFragSegs& segs, const float* isc,
                 int m, int k) {
     constexpr int kLds = frag_lds_bytes<MT, MH>();
-    skn_launch(ctx, gemm_q4k_frag_kernel<MT, MH>, dim3(m_tiles * segs.n_tiles), dim3(256 * MH), kLds, afrag, sfrag, segs, isc, m, k);
+    const uint32_t a_bytes = (uint32_t)((size_t)m_tiles * 32 * MT * MH * k * 2);  // (checked by the caller to fit)
+    skn_launch(ctx, gemm_q4k_frag_kernel<MT, MH>, dim3(m_tiles * segs.n_tiles), dim3(256 * MH), kLds, afrag, sfrag, segs, isc, m, k, a_bytes);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
@@ -705,6 +714,8 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     const int mt_rows = small_tiles ? 64 : 128;
     const int m_tiles = (m + mt_rows - 1) / mt_rows, m_pad = m_tiles * mt_rows;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), sf_bytes = align_up((size_t)m_pad * (k / 256) * 16 * 2);
+    SKN_REQUIRE(ctx, af_bytes < ((size_t)1 << 31), SKN_ERR_SHAPE,
+                "Q4_K GEMM: %d rows of %d activations exceed the 2^30 elements one call takes", m, k);
     const size_t is_bytes = align_up((size_t)m_pad * 4);
     uint8_t* ws;
     int rc = gemm_workspace(ctx, af_bytes + sf_bytes + is_bytes, &ws);
