@@ -191,11 +191,14 @@ typedef struct skn_llama_config {
     int32_t page_tokens; /* 256 */
     float rope_base;     /* 10000 */
     float rms_eps;       /* 1e-5 */
+    int32_t n_kv_head;   /* heads of the K / V projections and of the cache: a divisor of n_head (grouped-query
+                            attention), or 0 for n_head */
 } skn_llama_config;
 
 /* Per-layer weights, all device pointers into GGUF block data ([out, in] rows) or fp32 norm vectors. */
 typedef struct skn_llama_layer {
-    const void* wq; const void* wk; const void* wv; const void* wo; /* [hidden, hidden] */
+    const void* wq; const void* wo;                                  /* [hidden, hidden] */
+    const void* wk; const void* wv;                                  /* [n_kv_head * head_dim, hidden] */
     const void* w_gate; const void* w_up;                            /* [ffn, hidden] */
     const void* w_down;                                              /* [hidden, ffn] */
     const float* attn_norm; const float* ffn_norm;                   /* [hidden] */

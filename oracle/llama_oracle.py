@@ -13,7 +13,8 @@ class OracleLlama:
     def __init__(self, cfg, weights):
         self.cfg, self.w = cfg, weights
         c = cfg
-        self.k = np.zeros((c.n_layer, c.max_tokens, c.n_head, c.head_dim), dtype=np.uint16)
+        self.kvh = getattr(c, "n_kv_head", 0) or c.n_head  # grouped-query attention: heads of k / v
+        self.k = np.zeros((c.n_layer, c.max_tokens, self.kvh, c.head_dim), dtype=np.uint16)
         self.v = np.zeros_like(self.k)
         self.pos = 0
         self.logits = None
@@ -35,13 +36,17 @@ class OracleLlama:
         for l in range(c.n_layer):
             xn = oracle_c.rmsnorm(x, self.w[f"l{l}.attn_norm"][1], c.rms_eps)
             q = self._lin(f"l{l}.wq", h, h, xn, bf16_gemm).reshape(c.n_head, c.head_dim)
-            k = self._lin(f"l{l}.wk", h, h, xn, bf16_gemm).reshape(c.n_head, c.head_dim)
-            v = self._lin(f"l{l}.wv", h, h, xn, bf16_gemm).reshape(c.n_head, c.head_dim)
+            kvd = self.kvh * c.head_dim
+            k = self._lin(f"l{l}.wk", kvd, h, xn, bf16_gemm).reshape(self.kvh, c.head_dim)
+            v = self._lin(f"l{l}.wv", kvd, h, xn, bf16_gemm).reshape(self.kvh, c.head_dim)
             q = oracle_c.rope(q, pos, c.rope_base)
             k = oracle_c.rope(k, pos, c.rope_base)
             self.k[l, pos] = oracle_c.f2h(k)
             self.v[l, pos] = oracle_c.f2h(v)
-            att = oracle_c.attn_decode(q[None], self.k[l][None, : pos + 1], self.v[l][None, : pos + 1], [pos + 1],
+            # query head i reads cached head i // (n_head / kv heads)
+            rep = c.n_head // self.kvh
+            att = oracle_c.attn_decode(q[None], np.repeat(self.k[l][None, : pos + 1], rep, axis=2),
+                                       np.repeat(self.v[l][None, : pos + 1], rep, axis=2), [pos + 1],
                                        1.0 / np.sqrt(c.head_dim))[0].reshape(h)
             x = x + self._lin(f"l{l}.wo", h, h, att, bf16_gemm)
             xn = oracle_c.rmsnorm(x, self.w[f"l{l}.ffn_norm"][1], c.rms_eps)

@@ -49,7 +49,7 @@ template <int D, bool POW2>
 __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     const uint16_t* __restrict__ k_pool, const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ table,
     const int32_t* __restrict__ nctx, const float* __restrict__ q, float* partial, int* counters, float* __restrict__ out,
-    int n_head, int page_tokens, int page_shift, int pages_per_seq, int n_splits, float scale, int seq_fixed) {
+    int n_head, int kv_heads, int page_tokens, int page_shift, int pages_per_seq, int n_splits, float scale, int seq_fixed) {
     constexpr int LPT = D / 8;                        // lanes per token
     constexpr int G = 64 / LPT;                       // token groups (streams) per wavefront
     constexpr int NS = (kAttnThreads / 64) * G;       // streams per workgroup
@@ -63,6 +63,8 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     // blockIdx.z is the query row: its own sequence by default, or one shared sequence (seq_fixed >= 0) when
     // several query rows attend to prefixes of the same cache (prompt processing)
     const int split = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
+    // grouped queries: n_head query heads share kv_heads cached heads, n_head / kv_heads consecutive ones each
+    const int kvh = kv_heads == n_head ? h : h / (n_head / kv_heads);
     const int kv_seq = seq_fixed >= 0 ? seq_fixed : s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane % LPT, g = lane / LPT;
@@ -104,7 +106,7 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const size_t off = (((size_t)page[u] * n_head + h) * page_tokens + slot[u]) * D + c * 8;
+            const size_t off = (((size_t)page[u] * kv_heads + kvh) * page_tokens + slot[u]) * D + c * 8;
             kk[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
             vv[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
         }
@@ -236,8 +238,12 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
 // n_splits * (head_dim + 2) floats and `counters` n_queries * n_head ints that are zero between launches:
 // zeroed once by their owner, left zero by every launch.
 int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
-                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev) {
+                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev,
+                       int n_q_head) {
     const int D = kv->head_dim;
+    if (n_q_head <= 0) n_q_head = kv->n_head;
+    SKN_REQUIRE(ctx, n_q_head % kv->n_head == 0, SKN_ERR_SHAPE,
+                "attention: %d query heads are not a multiple of the %d cached heads", n_q_head, kv->n_head);
     SKN_REQUIRE(ctx, D == 64 || D == 128 || D == 256, SKN_ERR_SHAPE,
                 "skn_attn_decode: head_dim %d is not supported (64, 128 or 256)", D);
     SKN_REQUIRE(ctx, n_splits <= kMaxSplits, SKN_ERR_ARG, "skn_attn_decode: %d splits (at most %d)", n_splits, kMaxSplits);
@@ -246,16 +252,16 @@ int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32
     int page_shift = -1;
     if ((kv->page_tokens & (kv->page_tokens - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < kv->page_tokens; page_shift++) {}
-    dim3 grid(n_splits, kv->n_head, n_queries), block(kAttnThreads);
+    dim3 grid(n_splits, n_q_head, n_queries), block(kAttnThreads);
 #define SKN_ATTN_LAUNCH(DD)                                                                                        \
     do {                                                                                                           \
         if (page_shift >= 0)                                                                                       \
             skn_launch(ctx, attn_decode_kernel<DD, true>, grid, block, 0, kv->k_pool, kv->v_pool,                  \
-                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, kv->n_head,                \
+                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, n_q_head, kv->n_head,      \
                        kv->page_tokens, page_shift, kv->pages_per_seq, n_splits, scale, seq_fixed);                \
         else                                                                                                       \
             skn_launch(ctx, attn_decode_kernel<DD, false>, grid, block, 0, kv->k_pool, kv->v_pool,                 \
-                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, kv->n_head,                \
+                       kv->page_table_dev, nctx_dev, q_dev, partial, counters, out_dev, n_q_head, kv->n_head,      \
                        kv->page_tokens, page_shift, kv->pages_per_seq, n_splits, scale, seq_fixed);                \
     } while (0)
     if (D == 64) SKN_ATTN_LAUNCH(64);

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void attn_frag_kernel(const uint16_t* __restri
 template <int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(const float* __restrict__ q, const u32x4* __restrict__ kfrag,
                                                           const u32x4* __restrict__ vfrag, float* __restrict__ out,
-                                                          int n_queries, int n_head, int first_ctx, int n_tiles,
+                                                          int n_queries, int n_head, int kv_group, int first_ctx, int n_tiles,
                                                           float scale_log2e) {
     constexpr int KS = D / 16, DB = D / 32;
     __shared__ float part[3][DB * 16 + 2][64];  // running maximum, sum and accumulators of wavefronts 1..3
@@ -105,8 +105,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int x = 0; x < 16; x++) o[b][x] = 0.f;
     float mrun = -INFINITY, lrun = 0.f;  // running maximum (both halves agree) and this half's share of the sum
 
-    const u32x4* kp = kfrag + (size_t)head * n_tiles * KS * 64 + lane;
-    const u32x4* vp = vfrag + (size_t)head * n_tiles * KS * 64 + lane;
+    // (grouped queries: kv_group consecutive query heads read the keys and values of one cached head)
+    const u32x4* kp = kfrag + (size_t)(head / kv_group) * n_tiles * KS * 64 + lane;
+    const u32x4* vp = vfrag + (size_t)(head / kv_group) * n_tiles * KS * 64 + lane;
     u32x4 kf[KS];
 #pragma unroll
     for (int s = 0; s < KS; s++) kf[s] = kp[((size_t)min(wave, last_tile) * KS + s) * 64];
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <int D>
 int launch_prefill(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_queries, int first_ctx, float scale,
-                   float* out_dev) {
+                   float* out_dev, int n_q_head) {
     const int n_tokens = first_ctx + n_queries - 1;  // keys the last query sees
     const int n_tiles = (n_tokens + 31) / 32;
     const size_t frag_bytes = (size_t)kv->n_head * n_tiles * 32 * D * 2;
@@ -238,8 +239,9 @@ int launch_prefill(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_
                (const uint16_t*)kv->v_pool, (const int32_t*)(kv->page_table_dev + (size_t)seq * kv->pages_per_seq), kv->n_head,
                kv->page_tokens, n_tokens, n_tiles, kfrag, vfrag);
     SKN_LAUNCH_CHECK(ctx);
-    skn_launch(ctx, attn_prefill_kernel<D>, dim3((n_queries + 31) / 32, kv->n_head), dim3(256), 0, q_dev, (const u32x4*)kfrag,
-               (const u32x4*)vfrag, out_dev, n_queries, kv->n_head, first_ctx, n_tiles, scale * 1.4426950408889634f);
+    skn_launch(ctx, attn_prefill_kernel<D>, dim3((n_queries + 31) / 32, n_q_head), dim3(256), 0, q_dev, (const u32x4*)kfrag,
+               (const u32x4*)vfrag, out_dev, n_queries, n_q_head, n_q_head / kv->n_head, first_ctx, n_tiles,
+               scale * 1.4426950408889634f);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
@@ -249,9 +251,12 @@ int launch_prefill(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_
 // Shared with the decoder.  Query row t of n_queries attends to the first first_ctx + t tokens of sequence seq
 // (first_ctx >= 1; all of them must be cached).  head_dim 64 or 128.
 int skn_attn_prefill_launch(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_queries, int first_ctx, float scale,
-                            float* out_dev) {
-    if (kv->head_dim == 64) return launch_prefill<64>(ctx, kv, seq, q_dev, n_queries, first_ctx, scale, out_dev);
-    if (kv->head_dim == 128) return launch_prefill<128>(ctx, kv, seq, q_dev, n_queries, first_ctx, scale, out_dev);
+                            float* out_dev, int n_q_head) {
+    if (n_q_head <= 0) n_q_head = kv->n_head;
+    SKN_REQUIRE(ctx, n_q_head % kv->n_head == 0, SKN_ERR_SHAPE,
+                "attention: %d query heads are not a multiple of the %d cached heads", n_q_head, kv->n_head);
+    if (kv->head_dim == 64) return launch_prefill<64>(ctx, kv, seq, q_dev, n_queries, first_ctx, scale, out_dev, n_q_head);
+    if (kv->head_dim == 128) return launch_prefill<128>(ctx, kv, seq, q_dev, n_queries, first_ctx, scale, out_dev, n_q_head);
     return skn_fail(ctx, SKN_ERR_SHAPE, "skn_attn_prefill: head_dim %d is not supported (64 or 128)", kv->head_dim);
 }
 

@@ -95,24 +95,27 @@ __global__ __launch_bounds__(1024) void embed_rows_kernel(const uint8_t* __restr
 }
 
 // Rotary embedding of q and k rows at positions pos0 + row (pos0 from device), then k and v rows go to the
-// cache as fp16 at those positions.  grid = (rows, n_head), block = head_dim / 2 threads (one pair each).
+// cache as fp16 at those positions.  grid = (rows, n_head), block = head_dim / 2 threads (one pair each); q has
+// n_head heads per row, k and v kv_heads (the first kv_heads blocks of a row handle them).
 __global__ void rope_store_kernel(float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                   uint16_t* __restrict__ k_pool, uint16_t* __restrict__ v_pool,
                                   const int32_t* __restrict__ table, const int32_t* __restrict__ pos0_dev, int n_head,
-                                  int head_dim, int page_tokens, float log2_base) {
+                                  int kv_heads, int head_dim, int page_tokens, float log2_base) {
     const int row = blockIdx.x, h = blockIdx.y, i = threadIdx.x;
     const int pos = pos0_dev[0] + row;
     const float inv_freq = exp2f(-2.0f * (float)i / (float)head_dim * log2_base);
     float sn, cs;
     sincosf((float)pos * inv_freq, &sn, &cs);
-    const size_t base = ((size_t)row * n_head + h) * head_dim + 2 * i;
-    const float qa = q[base], qb = q[base + 1];
-    q[base] = qa * cs - qb * sn;
-    q[base + 1] = qa * sn + qb * cs;
+    const size_t qbase = ((size_t)row * n_head + h) * head_dim + 2 * i;
+    const float qa = q[qbase], qb = q[qbase + 1];
+    q[qbase] = qa * cs - qb * sn;
+    q[qbase + 1] = qa * sn + qb * cs;
+    if (h >= kv_heads) return;
+    const size_t base = ((size_t)row * kv_heads + h) * head_dim + 2 * i;
     const float ka = k[base], kb = k[base + 1];
     const float k0 = ka * cs - kb * sn, k1 = ka * sn + kb * cs;
     const int page = table[pos / page_tokens];
-    const size_t dst = (((size_t)page * n_head + h) * page_tokens + (pos % page_tokens)) * head_dim + 2 * i;
+    const size_t dst = (((size_t)page * kv_heads + h) * page_tokens + (pos % page_tokens)) * head_dim + 2 * i;
     const uint32_t kk = (uint32_t)__half_as_ushort(__float2half_rn(k0)) | ((uint32_t)__half_as_ushort(__float2half_rn(k1)) << 16);
     const uint32_t vv = (uint32_t)__half_as_ushort(__float2half_rn(v[base])) |
                         ((uint32_t)__half_as_ushort(__float2half_rn(v[base + 1])) << 16);
@@ -284,7 +287,7 @@ unsigned nblk(int64_t n) { return (unsigned)((n + 255) / 256); }
 // the launches of one decode step (eagerly or under stream capture)
 int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     const skn_llama_config& c = m->cfg;
-    const int H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim;
+    const int H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim, KVH = c.n_kv_head, KVD = KVH * D;
     const float scale = 1.0f / sqrtf((float)D);
     skn_launch(ctx, embed_rows_kernel, dim3(1), dim3(1024), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
                (const int32_t*)m->state, m->x);
@@ -301,29 +304,29 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         const bool f_gu = fuse && L.type_gate == SKN_TYPE_Q4_K && L.type_up == SKN_TYPE_Q4_K;
         const bool f_down = fuse && F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
         if (f_qkv) {
-            skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, H, H}};
+            skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, KVD, KVD}};
             skn_rope_epilogue rope;
             rope.pos_dev = m->state + 1;
             rope.page_table = kv->page_table_dev;
             rope.k_pool = kv->k_pool;
             rope.v_pool = kv->v_pool;
-            rope.n_head = NH;
+            rope.n_head = KVH;  // (heads of the cache)
             rope.head_dim = D;
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2f(c.rope_base);
-            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, 3 * H, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, H + 2 * KVD, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(skn_matvec_q(ctx, L.type_q, L.wq, H, H, m->xn, m->q));
-            SKN_TRY(skn_matvec_q(ctx, L.type_k, L.wk, H, H, m->xn, m->k));
-            SKN_TRY(skn_matvec_q(ctx, L.type_v, L.wv, H, H, m->xn, m->v));
+            SKN_TRY(skn_matvec_q(ctx, L.type_k, L.wk, KVD, H, m->xn, m->k));
+            SKN_TRY(skn_matvec_q(ctx, L.type_v, L.wv, KVD, H, m->xn, m->v));
             skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
-                       kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                       kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, KVH, D,
                        kv->page_tokens, log2f(c.rope_base));
             SKN_LAUNCH_CHECK(ctx);
         }
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att));
+        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
         if (f_o) {
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));
@@ -413,6 +416,8 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
     SKN_REQUIRE(ctx, cfg->n_layer > 0 && cfg->hidden > 0 && cfg->ffn > 0 && cfg->n_head > 0 && cfg->head_dim > 0 &&
                          cfg->vocab > 0 && cfg->max_tokens > 0 && cfg->page_tokens > 0,
                 SKN_ERR_ARG, "skn_llama_create: sizes must be positive");
+    SKN_REQUIRE(ctx, cfg->n_kv_head >= 0 && (cfg->n_kv_head == 0 || cfg->n_head % cfg->n_kv_head == 0), SKN_ERR_SHAPE,
+                "skn_llama_create: n_kv_head (%d) must divide n_head (%d)", cfg->n_kv_head, cfg->n_head);
     SKN_REQUIRE(ctx, cfg->n_head * cfg->head_dim == cfg->hidden, SKN_ERR_SHAPE,
                 "skn_llama_create: n_head * head_dim (%d) must equal hidden (%d)", cfg->n_head * cfg->head_dim,
                 cfg->hidden);
@@ -436,13 +441,14 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
     skn_llama* m = new (std::nothrow) skn_llama();
     SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_OOM, "skn_llama_create: host allocation failed");
     m->cfg = *cfg;
+    if (m->cfg.n_kv_head == 0) m->cfg.n_kv_head = cfg->n_head;
     m->w = *w;
     m->layers.assign(w->layers, w->layers + cfg->n_layer);
     m->w.layers = m->layers.data();
     int rc = SKN_OK;
     for (int l = 0; l < cfg->n_layer && rc == SKN_OK; l++) {
         skn_kv* kv = nullptr;
-        rc = skn_kv_create(ctx, 1, cfg->n_head, cfg->head_dim, cfg->page_tokens, cfg->max_tokens, &kv);
+        rc = skn_kv_create(ctx, 1, m->cfg.n_kv_head, cfg->head_dim, cfg->page_tokens, cfg->max_tokens, &kv);
         if (rc == SKN_OK) m->kv.push_back(kv);
     }
     const size_t H = cfg->hidden, F = cfg->ffn;
@@ -453,7 +459,7 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
     A(&m->x, H); A(&m->xn, H); A(&m->q, 3 * H); A(&m->att, H); A(&m->proj, H);
     if (rc == SKN_OK) {  // q, k, v are one buffer so that the three projections can be one launch
         m->k = m->q + H;
-        m->v = m->q + 2 * H;
+        m->v = m->k + (size_t)m->cfg.n_kv_head * cfg->head_dim;
     }
     A(&m->gate, F); A(&m->up, F); A(&m->mid, F); A(&m->logits, (size_t)cfg->vocab);
     A(&m->attn_partial, (size_t)cfg->n_head * max_splits * (cfg->head_dim + 2));
@@ -503,6 +509,7 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         SKN_REQUIRE(ctx, tokens_host[i] >= 0 && tokens_host[i] < c.vocab, SKN_ERR_RANGE,
                     "skn_llama_prefill: token %d of a vocabulary of %d", tokens_host[i], c.vocab);
     const int T = n_tokens, H = c.hidden, F = c.ffn, NH = c.n_head, D = c.head_dim, pos0 = m->pos;
+    const int KVH = c.n_kv_head, KVD = KVH * D;
     SKN_TRY(ensure_prompt_buffers(ctx, m, T));
     SKN_HIP(ctx, hipMemcpyAsync(m->ptok, tokens_host, (size_t)T * sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
     SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -526,7 +533,7 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         const bool q4k_down = F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
         if (q4k_qkv) {  // RMSNorm inside the activation pass, one launch for the three projections
-            const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq, 0}, {L.wk, H, m->pk, 0}, {L.wv, H, m->pv, 0}};
+            const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq, 0}, {L.wk, KVD, m->pk, 0}, {L.wv, KVD, m->pv, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.attn_norm, c.rms_eps};
             SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, src, T));
         } else {
@@ -534,18 +541,18 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             SKN_LAUNCH_CHECK(ctx);
             SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_q, L.wq, H, H, m->pb16, T, m->pq));
-            SKN_TRY(skn_gemm_q(ctx, L.type_k, L.wk, H, H, m->pb16, T, m->pk));
-            SKN_TRY(skn_gemm_q(ctx, L.type_v, L.wv, H, H, m->pb16, T, m->pv));
+            SKN_TRY(skn_gemm_q(ctx, L.type_k, L.wk, KVD, H, m->pb16, T, m->pk));
+            SKN_TRY(skn_gemm_q(ctx, L.type_v, L.wv, KVD, H, m->pb16, T, m->pv));
         }
         skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
-                   kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, D,
+                   kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, KVH, D,
                    kv->page_tokens, log2f(c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
         if (D <= 128)
-            SKN_TRY(skn_attn_prefill_launch(ctx, kv, 0, m->pq, T, pos0 + 1, scale, m->patt));
+            SKN_TRY(skn_attn_prefill_launch(ctx, kv, 0, m->pq, T, pos0 + 1, scale, m->patt, NH));
         else
-            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt));
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->pq, m->pnctx, T, 0, n_splits, m->ppartial, m->pcounters, scale, m->patt, NH));
         if (q4k_o) {  // the residual is added by the GEMM's store
             const skn_gemm_seg wo = {L.wo, H, m->px, 1};
             const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};

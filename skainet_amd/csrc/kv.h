@@ -25,8 +25,9 @@ int skn_kv_reserve(skn_ctx* ctx, skn_kv* kv, int seq, int new_len);
 int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
                     float* out_dev);
 int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
-                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev);
+                       int seq_fixed, int n_splits, float* partial, int* counters, float scale, float* out_dev,
+                       int n_q_head = 0);  // query heads (a multiple of the cached heads; 0: as many)
 int skn_attn_splits(skn_ctx* ctx, int pairs, int max_ctx);
 // Causal attention of n_queries rows of one sequence: row t attends to its first first_ctx + t tokens (head_dim 64 / 128).
 int skn_attn_prefill_launch(skn_ctx* ctx, skn_kv* kv, int seq, const float* q_dev, int n_queries, int first_ctx, float scale,
-                            float* out_dev);
+                            float* out_dev, int n_q_head = 0);

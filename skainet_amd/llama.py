@@ -27,6 +27,7 @@ class Config:
     page_tokens: int = 256
     rope_base: float = 10000.0
     rms_eps: float = 1e-5
+    n_kv_head: int = 0      # heads of wk / wv and of the cache (grouped-query attention); 0 = n_head
     type_attn: int = Q4_K   # wq, wk, wv, wo unless overridden below
     type_ffn: int = Q4_K    # w_gate, w_up, w_down unless overridden below
     type_embd: int = Q4_K
@@ -34,6 +35,10 @@ class Config:
     # Per-matrix overrides, the way mixed quantizations give some matrices more bits: keys are a matrix name
     # ("wv", "w_down", ...) for every layer or "l<layer>.<name>" for one layer.
     matrix_types: dict = field(default_factory=dict)
+
+    @property
+    def kv_heads(self) -> int:
+        return self.n_kv_head or self.n_head
 
     def matrix_type(self, layer: int, name: str) -> int:
         default = self.type_attn if name in ("wq", "wk", "wv", "wo") else self.type_ffn
@@ -53,9 +58,10 @@ def random_weights(cfg: Config, seed: int):
     w["out_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
     for l in range(cfg.n_layer):
         s = seed + 100 * (l + 1)
+        kvd = cfg.kv_heads * cfg.head_dim
         for i, name in enumerate(("wq", "wk", "wv", "wo")):
             t = cfg.matrix_type(l, name)
-            w[f"l{l}.{name}"] = (t, synth.weight(t, h, h, s + i))
+            w[f"l{l}.{name}"] = (t, synth.weight(t, kvd if name in ("wk", "wv") else h, h, s + i))
         for i, (name, rows, cols) in enumerate((("w_gate", f, h), ("w_up", f, h), ("w_down", h, f))):
             t = cfg.matrix_type(l, name)
             w[f"l{l}.{name}"] = (t, synth.weight(t, rows, cols, s + 10 + i))
@@ -91,7 +97,7 @@ class LlamaModel:
         wts = LlamaWeights(self.bufs["tok_embd"].ptr, self.bufs["out_norm"].ptr, self.bufs["out_head"].ptr,
                            cfg.type_embd, cfg.type_head, layers)
         c = LlamaConfig(cfg.n_layer, cfg.hidden, cfg.ffn, cfg.n_head, cfg.head_dim, cfg.vocab, cfg.max_tokens,
-                        cfg.page_tokens, cfg.rope_base, cfg.rms_eps)
+                        cfg.page_tokens, cfg.rope_base, cfg.rms_eps, cfg.n_kv_head)
         h = C.c_void_p()
         ctx._check(ctx.lib.skn_llama_create(ctx.handle, C.byref(c), C.byref(wts), C.byref(h)))
         self.handle = h.value
@@ -135,7 +141,8 @@ class LlamaModel:
 
         total = rb(c.type_head, c.vocab, c.hidden)
         for l in range(c.n_layer):
-            total += sum(rb(c.matrix_type(l, nm), c.hidden, c.hidden) for nm in ("wq", "wk", "wv", "wo"))
+            total += sum(rb(c.matrix_type(l, nm), c.hidden, c.hidden) for nm in ("wq", "wo"))
+            total += sum(rb(c.matrix_type(l, nm), c.kv_heads * c.head_dim, c.hidden) for nm in ("wk", "wv"))
             total += sum(rb(c.matrix_type(l, nm), c.ffn, c.hidden) for nm in ("w_gate", "w_up"))
             total += rb(c.matrix_type(l, "w_down"), c.hidden, c.ffn)
         return total

@@ -32,13 +32,13 @@ class LlamaConfig(C.Structure):
     _fields_ = [
         ("n_layer", C.c_int32), ("hidden", C.c_int32), ("ffn", C.c_int32), ("n_head", C.c_int32),
         ("head_dim", C.c_int32), ("vocab", C.c_int32), ("max_tokens", C.c_int32), ("page_tokens", C.c_int32),
-        ("rope_base", C.c_float), ("rms_eps", C.c_float),
+        ("rope_base", C.c_float), ("rms_eps", C.c_float), ("n_kv_head", C.c_int32),
     ]
 
 
 class LlamaLayer(C.Structure):
     _fields_ = [
-        ("wq", C.c_void_p), ("wk", C.c_void_p), ("wv", C.c_void_p), ("wo", C.c_void_p),
+        ("wq", C.c_void_p), ("wo", C.c_void_p), ("wk", C.c_void_p), ("wv", C.c_void_p),
         ("w_gate", C.c_void_p), ("w_up", C.c_void_p), ("w_down", C.c_void_p),
         ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p),
         ("type_q", C.c_int32), ("type_k", C.c_int32), ("type_v", C.c_int32), ("type_o", C.c_int32),

@@ -105,6 +105,49 @@ def test_mixed_matrix_types_match_oracle(hip):
     model.free()
 
 
+@pytest.mark.parametrize("n_kv_head,fused", [(2, 1), (1, 1), (2, 0)])
+def test_grouped_query_attention_matches_oracle(hip, n_kv_head, fused):
+    """Fewer K / V heads than query heads (two query heads per cached head, and one cached head for all four):
+    decode steps across a page boundary, then a prompt pass and more steps, fused and unfused kernels."""
+    cfg = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=n_kv_head, head_dim=128, vocab=512,
+                       max_tokens=96, page_tokens=16)
+    w = llama.random_weights(cfg, seed=31)
+    assert w["l0.wk"][1].size == n_kv_head * 128 * (512 // 256) * 144  # [n_kv_head * head_dim, hidden] Q4_K rows
+    hip.set_option("llama.fused", fused)
+    try:
+        model = llama.LlamaModel(hip, cfg, weights=w)
+        ora = OracleLlama(cfg, w)
+        tok = 5
+        for step in range(19):
+            got = model.decode(tok, 1)[0]
+            want = ora.step(tok)
+            err = oracle_np.rel_err(model.logits(), ora.logits)
+            assert err <= TOL, (step, err)
+            if _margin_ok(ora.logits, TOL * np.abs(ora.logits).max()):
+                assert got == want, step
+            tok = want
+        model.reset()
+        ora = OracleLlama(cfg, w)
+        prompt = np.random.default_rng(3).integers(0, cfg.vocab, size=35).tolist()
+        got_next = model.prefill(prompt)
+        want_next = ora.prefill(prompt, bf16_gemm=True)
+        err = oracle_np.rel_err(model.logits(), ora.logits)
+        assert err <= 5e-3, err
+        if _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+            assert got_next == want_next
+        got = model.decode(want_next, 4)
+        tok = want_next
+        for i in range(4):
+            want = ora.step(tok)
+            if not _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+                break
+            assert got[i] == want, i
+            tok = want
+        model.free()
+    finally:
+        hip.set_option("llama.fused", 1)
+
+
 def test_full_7b_shape_matches_oracle(hip):
     """The benchmark's model shape (32 layers, hidden 4096, FFN 11008, 32 heads x 128, vocabulary 32000, Q4_K
     layers, Q6_K head) at full size: decode steps and a short prompt pass against the oracle.  Every layer points
@@ -206,3 +249,8 @@ def test_llama_argument_errors(hip):
     with pytest.raises(runtime.SknError) as e:
         llama.LlamaModel(hip, bad, weights=llama.random_weights(bad, seed=1))
     assert e.value.code == runtime.ERR_SHAPE
+    bad = llama.Config(n_layer=1, hidden=512, ffn=768, n_head=4, n_kv_head=3, head_dim=128, vocab=512, max_tokens=32,
+                       page_tokens=16)
+    with pytest.raises(runtime.SknError) as e:
+        llama.LlamaModel(hip, bad, weights=llama.random_weights(bad, seed=1))
+    assert e.value.code == runtime.ERR_SHAPE and "must divide" in e.value.message
