@@ -82,8 +82,12 @@ class LlamaModel:
             gen_cfg = cfg if not share_layers else Config(**{**cfg.__dict__, "n_layer": 1})
             weights = random_weights(gen_cfg, seed)
         self.host_weights = weights if not share_layers else None
+        self.head_type = weights["out_head"][0]
+        uploaded = {}  # an array that appears under two names (a head tied to the embedding) is uploaded once
         for name, (_, arr) in weights.items():
-            self.bufs[name] = ctx.to_device(arr)
+            if id(arr) not in uploaded:
+                uploaded[id(arr)] = ctx.to_device(arr)
+            self.bufs[name] = uploaded[id(arr)]
         layers = (LlamaLayer * cfg.n_layer)()
         for l in range(cfg.n_layer):
             src = 0 if share_layers else l
@@ -95,7 +99,7 @@ class LlamaModel:
                 setattr(L, tf, weights[f"l{src}.{f}"][0])  # the type each matrix was built with
         self._layers = layers
         wts = LlamaWeights(self.bufs["tok_embd"].ptr, self.bufs["out_norm"].ptr, self.bufs["out_head"].ptr,
-                           cfg.type_embd, cfg.type_head, layers)
+                           weights["tok_embd"][0], weights["out_head"][0], layers)
         c = LlamaConfig(cfg.n_layer, cfg.hidden, cfg.ffn, cfg.n_head, cfg.head_dim, cfg.vocab, cfg.max_tokens,
                         cfg.page_tokens, cfg.rope_base, cfg.rms_eps, cfg.n_kv_head)
         h = C.c_void_p()
@@ -127,7 +131,7 @@ class LlamaModel:
         if self.handle:
             self.ctx.lib.skn_llama_free(self.ctx.handle, self.handle)
             self.handle = None
-        for b in self.bufs.values():
+        for b in {id(b): b for b in self.bufs.values()}.values():
             b.free()
         self.bufs = {}
 
@@ -139,10 +143,119 @@ class LlamaModel:
             be, bb = synth.BLOCK[t]
             return n * (k // be) * bb
 
-        total = rb(c.type_head, c.vocab, c.hidden)
+        total = rb(self.head_type, c.vocab, c.hidden)
         for l in range(c.n_layer):
             total += sum(rb(c.matrix_type(l, nm), c.hidden, c.hidden) for nm in ("wq", "wo"))
             total += sum(rb(c.matrix_type(l, nm), c.kv_heads * c.head_dim, c.hidden) for nm in ("wk", "wv"))
             total += sum(rb(c.matrix_type(l, nm), c.ffn, c.hidden) for nm in ("w_gate", "w_up"))
             total += rb(c.matrix_type(l, "w_down"), c.hidden, c.ffn)
         return total
+
+
+# ---- a model out of a GGUF file ---------------------------------------------------------------------------------
+# Tensor and metadata names are those of llama.cpp's GGUF files for the "llama" architecture, the files the
+# reference's reader is written for (gguf/src/commonMain/kotlin/sk/ai/net/gguf/GGUFReader.kt:82-139 reads the key /
+# value fields, :332-401 the tensors).  Their q and k projections are stored for the rotary embedding of adjacent
+# pairs (2i, 2i + 1), which is the convention of this decoder.
+_GGUF_LAYER_TENSORS = {"wq": "attn_q", "wk": "attn_k", "wv": "attn_v", "wo": "attn_output", "w_gate": "ffn_gate",
+                       "w_up": "ffn_up", "w_down": "ffn_down"}
+
+
+def config_from_gguf(reader, max_tokens=None, page_tokens=256) -> Config:
+    """The decoder's shape from the metadata of an opened GGUFReader (ValueError when a field is missing or the
+    file describes something this decoder does not compute)."""
+    f = reader.fields
+    arch = f.get("general.architecture")
+    if arch != "llama":
+        raise ValueError(f"general.architecture is {arch!r}: only 'llama' files are decoded")
+
+    def need(key):
+        if f"{arch}.{key}" not in f:
+            raise ValueError(f"GGUF metadata lacks {arch}.{key}")
+        return f[f"{arch}.{key}"]
+
+    hidden, n_head = int(need("embedding_length")), int(need("attention.head_count"))
+    head_dim = int(f.get(f"{arch}.attention.key_length", hidden // n_head))
+    rope_dims = int(f.get(f"{arch}.rope.dimension_count", head_dim))
+    if rope_dims != head_dim:
+        raise ValueError(f"partial rotary embedding ({rope_dims} of {head_dim} dimensions) is not supported")
+    embd = reader.tensor("token_embd.weight")
+    n_kv = int(f.get(f"{arch}.attention.head_count_kv", n_head))
+    return Config(
+        n_layer=int(need("block_count")), hidden=hidden, ffn=int(need("feed_forward_length")), n_head=n_head,
+        head_dim=head_dim, vocab=int(embd.shape[0]),
+        max_tokens=int(max_tokens or f.get(f"{arch}.context_length", 2048)), page_tokens=page_tokens,
+        rope_base=float(f.get(f"{arch}.rope.freq_base", 10000.0)),
+        rms_eps=float(f.get(f"{arch}.attention.layer_norm_rms_epsilon", 1e-5)),
+        n_kv_head=0 if n_kv == n_head else n_kv, type_embd=embd.tensor_type)
+
+
+def weights_from_gguf(reader, cfg: Config):
+    """name -> (ggml type or None for fp32 vectors, array) in the form LlamaModel takes; the arrays are views of the
+    mapped file.  A file without output.weight shares the embedding table with the head."""
+    names = {t.name for t in reader.tensors}
+
+    def matrix(name, rows, cols):
+        t = reader.tensor(name)
+        if t.shape != (rows, cols):
+            raise ValueError(f"{name} is {t.shape}, expected {(rows, cols)}")
+        return (t.tensor_type, t.data if t.data.dtype == np.uint8 else np.ascontiguousarray(t.data).view(np.uint8).reshape(-1))
+
+    def vector(name, n):
+        t = reader.tensor(name)
+        if t.shape != (n,):
+            raise ValueError(f"{name} is {t.shape}, expected {(n,)}")
+        return (None, np.ascontiguousarray(t.data, dtype=np.float32))
+
+    h, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
+    w = {"tok_embd": matrix("token_embd.weight", cfg.vocab, h), "out_norm": vector("output_norm.weight", h)}
+    w["out_head"] = matrix("output.weight", cfg.vocab, h) if "output.weight" in names else w["tok_embd"]
+    shapes = {"wq": (h, h), "wk": (kvd, h), "wv": (kvd, h), "wo": (h, h), "w_gate": (cfg.ffn, h), "w_up": (cfg.ffn, h),
+              "w_down": (h, cfg.ffn)}
+    for l in range(cfg.n_layer):
+        for ours, theirs in _GGUF_LAYER_TENSORS.items():
+            w[f"l{l}.{ours}"] = matrix(f"blk.{l}.{theirs}.weight", *shapes[ours])
+        w[f"l{l}.attn_norm"] = vector(f"blk.{l}.attn_norm.weight", h)
+        w[f"l{l}.ffn_norm"] = vector(f"blk.{l}.ffn_norm.weight", h)
+    return w
+
+
+def model_from_gguf(ctx: runtime.Context, path: str, max_tokens=None, page_tokens=256) -> LlamaModel:
+    """Opens a llama-architecture GGUF file, uploads its tensors as they are and returns the decoder over them."""
+    from . import gguf
+
+    reader = gguf.GGUFReader(path)
+    try:
+        cfg = config_from_gguf(reader, max_tokens, page_tokens)
+        w = weights_from_gguf(reader, cfg)
+        cfg.type_head = w["out_head"][0]
+        model = LlamaModel(ctx, cfg, weights=w)
+        model.host_weights = None  # (views of the mapped file: not kept)
+        del w
+        return model
+    finally:
+        reader.close()
+
+
+def write_gguf_model(path, cfg: Config, weights):
+    """The inverse, for tests and for handing a synthetic model to other GGUF consumers."""
+    from . import gguf
+
+    fields = {"general.architecture": "llama", "llama.block_count": cfg.n_layer, "llama.embedding_length": cfg.hidden,
+              "llama.feed_forward_length": cfg.ffn, "llama.attention.head_count": cfg.n_head,
+              "llama.attention.head_count_kv": cfg.kv_heads, "llama.context_length": cfg.max_tokens,
+              "llama.rope.freq_base": float(cfg.rope_base), "llama.attention.layer_norm_rms_epsilon": float(cfg.rms_eps)}
+    h, kvd = cfg.hidden, cfg.kv_heads * cfg.head_dim
+    shapes = {"wq": (h, h), "wk": (kvd, h), "wv": (kvd, h), "wo": (h, h), "w_gate": (cfg.ffn, h), "w_up": (cfg.ffn, h),
+              "w_down": (h, cfg.ffn)}
+    tensors = [("token_embd.weight", weights["tok_embd"][0], (cfg.vocab, h), weights["tok_embd"][1]),
+               ("output_norm.weight", 0, (h,), weights["out_norm"][1]),
+               ("output.weight", weights["out_head"][0], (cfg.vocab, h), weights["out_head"][1])]
+    for l in range(cfg.n_layer):
+        for ours, theirs in _GGUF_LAYER_TENSORS.items():
+            t, arr = weights[f"l{l}.{ours}"]
+            tensors.append((f"blk.{l}.{theirs}.weight", t, shapes[ours], arr))
+        tensors.append((f"blk.{l}.attn_norm.weight", 0, (h,), weights[f"l{l}.attn_norm"][1]))
+        tensors.append((f"blk.{l}.ffn_norm.weight", 0, (h,), weights[f"l{l}.ffn_norm"][1]))
+    gguf.write_gguf(path, fields, tensors)
+

@@ -81,3 +81,37 @@ def test_bad_row_size_message(tmp_path):
         _ = t.byte_shape
     del t
     r.close()
+
+
+def test_llama_config_and_weights_from_gguf(tmp_path):
+    """A llama-architecture file written with the names and metadata keys of llama.cpp's files comes back as the
+    decoder's configuration and weight table: grouped K / V heads, per-matrix types, shapes checked."""
+    from skainet_amd import llama
+
+    cfg = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=2, head_dim=128, vocab=256, max_tokens=64,
+                       page_tokens=16, rope_base=50000.0, rms_eps=1e-6, type_embd=8,
+                       matrix_types={"wv": 14, "l1.w_down": 8})
+    w = llama.random_weights(cfg, seed=4)
+    path = str(tmp_path / "tiny-llama.gguf")
+    llama.write_gguf_model(path, cfg, w)
+    r = gguf.GGUFReader(path)
+    got = llama.config_from_gguf(r, page_tokens=16)
+    for key in ("n_layer", "hidden", "ffn", "n_head", "n_kv_head", "head_dim", "vocab", "max_tokens", "rope_base"):
+        assert getattr(got, key) == getattr(cfg, key), key
+    assert abs(got.rms_eps - 1e-6) < 1e-12 and got.type_embd == 8
+    gw = llama.weights_from_gguf(r, got)
+    assert set(gw) == set(w)
+    for name, (t, arr) in w.items():
+        assert gw[name][0] == t, name
+        assert np.array_equal(np.asarray(gw[name][1]).view(np.uint8).reshape(-1), np.asarray(arr).view(np.uint8).reshape(-1)), name
+    assert gw["l0.wv"][0] == 14 and gw["l1.w_down"][0] == 8 and gw["l0.wk"][1].size == 2 * 128 * 2 * 144
+    del gw
+    r.close()
+    # a file of another architecture, and one with a tensor of the wrong shape
+    bad = str(tmp_path / "bad.gguf")
+    gguf.write_gguf(bad, {"general.architecture": "gpt2"}, [("token_embd.weight", 0, (4, 4), np.zeros((4, 4), np.float32))])
+    r = gguf.GGUFReader(bad)
+    with pytest.raises(ValueError, match="only 'llama' files"):
+        llama.config_from_gguf(r)
+    r.close()
+

@@ -148,6 +148,32 @@ def test_grouped_query_attention_matches_oracle(hip, n_kv_head, fused):
         hip.set_option("llama.fused", 1)
 
 
+def test_model_from_gguf_file_equals_model_from_weights(hip, tmp_path):
+    """GGUF file -> device -> decoder: a file with llama.cpp's tensor names and metadata (grouped K / V heads, a
+    mix of matrix types, Q8_0 embedding) decodes bit for bit like the model built from the same weights in memory."""
+    cfg = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=2, head_dim=128, vocab=512, max_tokens=64,
+                       page_tokens=16, type_embd=8, matrix_types={"l0.wq": 8, "l0.w_down": 13, "l1.wo": 8, "l1.w_gate": 7})
+    w = llama.random_weights(cfg, seed=41)
+    path = str(tmp_path / "tiny-llama.gguf")
+    llama.write_gguf_model(path, cfg, w)
+    direct = llama.LlamaModel(hip, cfg, weights=w)
+    loaded = llama.model_from_gguf(hip, path, page_tokens=16)
+    assert loaded.cfg.n_kv_head == 2 and loaded.cfg.max_tokens == 64
+    prompt = [3, 141, 59, 26, 5, 35]
+    a, b = direct.prefill(prompt), loaded.prefill(prompt)
+    assert a == b and np.array_equal(direct.logits(), loaded.logits())
+    assert direct.decode(a, 10) == loaded.decode(b, 10)
+    assert np.array_equal(direct.logits(), loaded.logits())
+    ora = OracleLlama(cfg, w)
+    ora.prefill(prompt, bf16_gemm=True)
+    tok = a
+    for _ in range(10):
+        tok = ora.step(tok)
+    assert oracle_np.rel_err(loaded.logits(), ora.logits) <= 2e-2  # (loose: 16 tokens of a random-weight stack)
+    direct.free()
+    loaded.free()
+
+
 def test_full_7b_shape_matches_oracle(hip):
     """The benchmark's model shape (32 layers, hidden 4096, FFN 11008, 32 heads x 128, vocabulary 32000, Q4_K
     layers, Q6_K head) at full size: decode steps and a short prompt pass against the oracle.  Every layer points
