@@ -46,6 +46,20 @@ __device__ __forceinline__ void store_tile(const float16_t& acc, float* __restri
     }
 }
 
+// the same with the sixteen row scales in hand (sc[r]: the scale of the row that register r holds)
+__device__ __forceinline__ void store_tile_scaled(const float16_t& acc, float* __restrict__ c, int ldc, int row0, int col0,
+                                                  int m, int n, const float (&sc)[16], int lane, bool accumulate) {
+    const int col = col0 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = row0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < m && col < n) {
+            float* dst = c + (size_t)row * ldc + col;
+            *dst = accumulate ? *dst + acc[r] * sc[r] : acc[r] * sc[r];
+        }
+    }
+}
+
 // ---- Q4_K path: weights unpacked in the kernel, one MFMA per k-step, operands loaded by the wavefronts ------
 // Workgroup of eight wavefronts, tile (64 MT) x 64.  The tile is divided in two along m; along k it is not
 // divided spatially but by superblock: wavefront (mh, kq) computes rows [32 MT mh, 32 MT (mh + 1)) x all 64
@@ -226,6 +240,13 @@ struct Q4kFragSegs {
     int pair;
 };
 
+// the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit (the scales of the tile's rows follow it): dynamic, opted in per
+// device by skn_gemm_init
+template <int MT, int MH>
+constexpr int frag_lds_bytes() {
+    return 2 * kBN * kWPitch > MT * MH * 24576 ? 2 * kBN * kWPitch : MT * MH * 24576;
+}
+
 // Accumulators: acc holds the running sum of a column in units of cs = d * 2^14 of the latest superblock whose d
 // is not zero.  Entering a superblock it is rescaled by cs_old / cs_new (a relative error of 2^-23 per
 // superblock, against the 1e-3 asked of the op); the superblock's integer products then add to it as they come
@@ -297,13 +318,19 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
 #pragma unroll
             for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
 
+    // the scales of the tile's rows, for the store at the end
+    float* isc_lds = reinterpret_cast<float*>(lds + frag_lds_bytes<MT, MH>());
     wfetch(0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (tid < 32 * MT * MH) isc_lds[tid] = inv_scale[MH * mt * MT * 32 + tid];
     if (kq < nb) {
+        // (the first eight fragment steps are requested behind the weights and stay in flight past the barrier)
 #pragma unroll
         for (int s = 0; s < 8; s++) afetch(16 * kq + s, s);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * MT) : "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    asm volatile("s_barrier" ::: "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     for (int g = 0; g < groups; g++) {
         const int sb = 4 * g + kq;
@@ -490,8 +517,9 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                         // register x of lane l: row 8 (x / 4) + 4 (l / 32) + x % 4 of the 32 x 32 tile
                         const int row = (mb0 + i) * 32 + 8 * (x >> 2) + 4 * (lane >> 5) + (x & 3);
                         if (row < m && col < n) {
-                            const float a = g * inv_scale[row];
-                            c[(size_t)row * n + col] = a / (1.0f + expf(-a)) * (u * inv_scale[row]);  // silu(gate) * up
+                            const float sc = isc_lds[row - MH * mt * MT * 32];
+                            const float a = g * sc;
+                            c[(size_t)row * n + col] = a / (1.0f + expf(-a)) * (u * sc);  // silu(gate) * up
                         }
                     }
                 }
@@ -506,23 +534,20 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 for (int o = 0; o < 3; o++)
 #pragma unroll
                     for (int x = 0; x < 16; x++) sum[x] += red[((mh * 2 * MT + t) * 3 + o) * 1024 + 64 * x + lane];
-                store_tile(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, inv_scale, lane, segs.accumulate[seg] != 0);
+                float sc[16];
+#pragma unroll
+                for (int x = 0; x < 16; x++) sc[x] = isc_lds[(mh * MT + i) * 32 + 8 * (x >> 2) + 4 * (lane >> 5) + (x & 3)];
+                store_tile_scaled(sum, c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, sc, lane, segs.accumulate[seg] != 0);
             }
         }
     }
 }
 
-// the kernel's LDS (weight buffers, then the tile exchange) exceeds the static limit: dynamic, opted in per
-// device by skn_gemm_init
-template <int MT, int MH>
-constexpr int frag_lds_bytes() {
-    return 2 * kBN * kWPitch > MT * MH * 24576 ? 2 * kBN * kWPitch : MT * MH * 24576;
-}
 
 template <int MT, int MH>
 int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfrag, const Q4kFragSegs& segs, const float* isc,
                 int m, int k) {
-    constexpr int kLds = frag_lds_bytes<MT, MH>();
+    constexpr int kLds = frag_lds_bytes<MT, MH>() + 32 * MT * MH * 4;
     const uint32_t a_bytes = (uint32_t)((size_t)m_tiles * 32 * MT * MH * k * 2);  // (checked by the caller to fit)
     skn_launch(ctx, gemm_q4k_frag_kernel<MT, MH>, dim3(m_tiles * segs.n_tiles), dim3(256 * MH), kLds, afrag, sfrag, segs, isc, m, k, a_bytes);
     SKN_LAUNCH_CHECK(ctx);
@@ -673,8 +698,8 @@ inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 // Dynamic LDS above 48 KiB must be allowed per kernel and device; done once per context here so that no launch
 // path has to.
 int skn_gemm_init(skn_ctx* ctx) {
-    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 2>()));
-    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 1>()));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 2>() + 32 * 2 * 2 * 4));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 1>() + 32 * 2 * 1 * 4));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<2, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
