@@ -265,6 +265,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     else if (!strcmp(key, "llama.graph")) ctx->opt_llama_graph = value;
     else if (!strcmp(key, "llama.fused")) ctx->opt_llama_fused = value;
     else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
+    else if (!strcmp(key, "matvec.stage")) ctx->opt_matvec_stage = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
     return SKN_OK;
 }

@@ -60,6 +60,50 @@ def test_matvec_vs_oracle(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, want) <= TOL
 
 
+STAGED = [(3, "q4_1"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
+
+
+@pytest.mark.parametrize("qtype,name", STAGED)
+@pytest.mark.parametrize("n,k", [(7, 11008), (4, 16384), (9, 2048), (3, 256)])
+def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
+    """The formats whose rows pass through LDS: several chunks per row with a short last one (k = 11008), the
+    longest row, fewer rows than a workgroup takes -- both kernels against the oracle and against each other."""
+    raw = synth.weight(qtype, n, k, seed=3 * n + k + qtype)
+    x = synth.activation_f32(k, seed=k + 1)
+    want = oracle_c.matvec_q(qtype, raw, n, k, x)
+    got = {}
+    try:
+        for stage in (0, 1):
+            hip.set_option("matvec.stage", stage)
+            got[stage] = hip.matvec_q_host(qtype, raw, n, k, x)
+            assert oracle_np.rel_err(got[stage], want) <= TOL
+    finally:
+        hip.set_option("matvec.stage", 1)
+    assert np.abs(got[1] - got[0]).max() <= 1e-5 * np.abs(want).max()  # (fp32 sums in a different order)
+
+
+@pytest.mark.parametrize("qtype,name", [(3, "q4_1"), (10, "q2_k")])
+def test_matvec_rows_not_16_byte_aligned(hip, qtype, name):
+    """Rows whose byte length is not a multiple of 16 (three Q4_1 blocks, one Q2_K block) and a weight pointer off
+    the 16-byte grid take the kernel that reads global memory directly."""
+    be, bb = synth.BLOCK[qtype]
+    n, k = 6, 3 * be if qtype == 3 else be
+    raw = synth.weight(qtype, n, k, seed=11)
+    x = synth.activation_f32(k, seed=12)
+    want = oracle_c.matvec_q(qtype, raw, n, k, x)
+    assert oracle_np.rel_err(hip.matvec_q_host(qtype, raw, n, k, x), want) <= TOL
+    # base pointer 4 bytes into an allocation
+    n, k = 5, 16 * be
+    raw = synth.weight(qtype, n, k, seed=13)
+    x = synth.activation_f32(k, seed=14)
+    buf = hip.alloc(raw.nbytes + 16)
+    flat = np.concatenate([np.zeros(4, np.uint8), raw.reshape(-1)])
+    buf.upload(flat)
+    xd, yd = hip.to_device(x), hip.alloc(4 * n)
+    hip.matvec_q(qtype, buf.ptr + 4, n, k, xd, yd)
+    assert oracle_np.rel_err(yd.download(np.float32, n), oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
+
+
 def test_dense_matvec_odd_row_length(hip):
     for qtype in (0, 1, 30):
         n, k = 9, 333  # no block structure: any row length
