@@ -4,6 +4,7 @@
 // read once per workgroup and y written once.  One wavefront owns one output row, so the only cross-lane
 // traffic is a single DPP reduction per row and rows never need atomics.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -73,6 +74,27 @@ __device__ __forceinline__ void q4k_dot_dword(uint32_t q, const float4& xl, cons
     ahi = fmaf((float)h13.y, xh.w, ahi);
 }
 
+// Q5_K: the same dword of nibbles with the dword of qh that holds the fifth bits of its four elements, already
+// shifted so that bit 0 of each byte belongs to the low-nibble sub-block and bit 1 to the high-nibble one.  The
+// fifth bit joins its nibble before the multiply (bit 4 of the low value, bit 8 of the sixteen-fold high value),
+// so the fp16 subnormal read by v_fma_mix_f32 is the whole five-bit quant.
+__device__ __forceinline__ void q5k_dot_dword(uint32_t q, uint32_t hq, const float4& xl, const float4& xh, float& alo,
+                                              float& ahi) {
+    const uint32_t q8 = q >> 8, hq8 = hq >> 8;
+    const half2_t l02 = __builtin_bit_cast(half2_t, (q & 0x000F000Fu) | ((hq & 0x00010001u) << 4));
+    const half2_t h02 = __builtin_bit_cast(half2_t, (q & 0x00F000F0u) | ((hq & 0x00020002u) << 7));
+    const half2_t l13 = __builtin_bit_cast(half2_t, (q8 & 0x000F000Fu) | ((hq8 & 0x00010001u) << 4));
+    const half2_t h13 = __builtin_bit_cast(half2_t, (q8 & 0x00F000F0u) | ((hq8 & 0x00020002u) << 7));
+    alo = fmaf((float)l02.x, xl.x, alo);
+    ahi = fmaf((float)h02.x, xh.x, ahi);
+    alo = fmaf((float)l13.x, xl.y, alo);
+    ahi = fmaf((float)h13.x, xh.y, ahi);
+    alo = fmaf((float)l02.y, xl.z, alo);
+    ahi = fmaf((float)h02.y, xh.z, ahi);
+    alo = fmaf((float)l13.y, xl.w, alo);
+    ahi = fmaf((float)h13.y, xh.w, ahi);
+}
+
 // Staging of x, split in two so that the weight loads can be issued in between: coalesced global loads
 // (thread t takes float4 t, t + blockDim, ...: a wavefront reads 1 KiB contiguous per instruction) into
 // registers, and later the LDS stores, which do the transposition into lane order.  float4 f of x belongs to
@@ -123,10 +145,21 @@ struct Q4kLoads {
     bool ok;  // false: the slot lies past the row end / past the last row and must contribute nothing
 };
 
+// Q5_K (176 bytes: header chunk, two chunks of qh, eight of qs): the 32 bytes of fifth bits as well -- bit j of
+// qh[l] belongs to element l of sub-block j, so every lane of a superblock needs all of them
+struct Q5kLoads : Q4kLoads {
+    u32x4 ha, hb;
+};
+
+template <typename LT>
+constexpr bool kIsQ5 = false;
+template <>
+constexpr bool kIsQ5<Q5kLoads> = true;
+
 // One step for R rows: the lane's 64 activations are read from LDS in two halves of 32 (8 float4 live at a
 // time) and each half meets the matching nibble chunk of every row.
-template <int R>
-__device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+template <int R, typename LT>
+__device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
                                          int s, int lane, int pair, float (&acc)[R]) {
     float alo[R], ahi[R];
 #pragma unroll
@@ -142,10 +175,18 @@ __device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* _
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const u32x4 qq = half == 0 ? L[r].qa : L[r].qb;
-            q4k_dot_dword(qq.x, xl[0], xh[0], alo[r], ahi[r]);
-            q4k_dot_dword(qq.y, xl[1], xh[1], alo[r], ahi[r]);
-            q4k_dot_dword(qq.z, xl[2], xh[2], alo[r], ahi[r]);
-            q4k_dot_dword(qq.w, xl[3], xh[3], alo[r], ahi[r]);
+            if constexpr (kIsQ5<LT>) {
+                const u32x4 hh = (half == 0 ? L[r].ha : L[r].hb) >> (uint32_t)(2 * pair);
+                q5k_dot_dword(qq.x, hh.x, xl[0], xh[0], alo[r], ahi[r]);
+                q5k_dot_dword(qq.y, hh.y, xl[1], xh[1], alo[r], ahi[r]);
+                q5k_dot_dword(qq.z, hh.z, xl[2], xh[2], alo[r], ahi[r]);
+                q5k_dot_dword(qq.w, hh.w, xl[3], xh[3], alo[r], ahi[r]);
+            } else {
+                q4k_dot_dword(qq.x, xl[0], xh[0], alo[r], ahi[r]);
+                q4k_dot_dword(qq.y, xl[1], xh[1], alo[r], ahi[r]);
+                q4k_dot_dword(qq.z, xl[2], xh[2], alo[r], ahi[r]);
+                q4k_dot_dword(qq.w, xl[3], xh[3], alo[r], ahi[r]);
+            }
         }
     }
     const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];
@@ -170,9 +211,12 @@ __device__ __forceinline__ void q4k_step(const Q4kLoads (&L)[R], const float4* _
 // next step, consume the current one.  A compute unit's memory pipeline accepts only so many requests before
 // a wavefront stalls at issue, so the loads are kept one step ahead instead of all up front -- otherwise the
 // x stores (and with them every wavefront at the barrier) would sit behind the issue of a whole row.
-template <int STEPS, int R>
+// Q5: Q5_K blocks (eleven chunks, the quants from the fourth on) with the same lane map, staging and scales.
+template <int STEPS, int R, bool Q5 = false>
 __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                          float* __restrict__ y, int n_rows, int nb) {
+    using Loads = std::conditional_t<Q5, Q5kLoads, Q4kLoads>;
+    constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
@@ -185,7 +229,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     const int row0 = (blockIdx.x * waves + wave) * R;
     const int sub = lane >> 2;  // superblock within the step
     const int p = lane & 3;     // sub-block pair within the superblock
-    const size_t row_chunks = (size_t)nb * 9;
+    const size_t row_chunks = (size_t)nb * kChunks;
     const int n4 = nb * 64;  // float4 count of x
 
     // the first J float4 per thread go into registers now; J covers all of x in the unrolled kernels
@@ -202,23 +246,27 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         acc[r] = 0.f;
         row_ok[r] = row0 + r < n_rows;
         // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
-        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + 1 + 2 * p;
+        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + kFirst + 2 * p;
     }
-    auto issue = [&](int s, int tie, Q4kLoads (&L)[R]) __attribute__((always_inline)) {
+    auto issue = [&](int s, int tie, Loads (&L)[R]) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
-        const int off = min(blk, nb - 1) * 9 + tie;
+        const int off = min(blk, nb - 1) * kChunks + tie;
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const u32x4* bp = rp[r] + off;
             L[r].qa = bp[0];
             L[r].qb = bp[1];
-            L[r].h = bp[-1 - 2 * p];
+            L[r].h = bp[-kFirst - 2 * p];
+            if constexpr (Q5) {
+                L[r].ha = bp[1 - kFirst - 2 * p];
+                L[r].hb = bp[2 - kFirst - 2 * p];
+            }
             L[r].ok = row_ok[r] && blk < nb;
         }
     };
 
     if constexpr (STEPS > 0) {
-        Q4kLoads L[STEPS][R];
+        Loads L[STEPS][R];
         issue(0, 0, L[0]);
         q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
         __syncthreads();
@@ -235,7 +283,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
             asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
         }
     } else {
-        Q4kLoads bufa[R], bufb[R];
+        Loads bufa[R], bufb[R];
         issue(0, 0, bufa);
         q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
         for (int f = tid + J * blockDim.x; f < n4; f += blockDim.x)
@@ -811,14 +859,14 @@ hipError_t allow_big_lds_fused_all() {
     return e;
 }
 
-template <int STEPS, int R>
+template <int STEPS, int R, bool Q5 = false>
 int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
-    if (STEPS > 0 && waves != 8) return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
+    if (STEPS > 0 && waves != 8) return launch_q4k<0, R, Q5>(ctx, w, n, nb, x, y, waves);
     const int steps = (nb + 15) / 16;
     const size_t lds = (size_t)steps * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
     SKN_REQUIRE(ctx, lds <= 160 * 1024, SKN_ERR_SHAPE, "skn_matvec_q: k = %d needs %zu bytes of LDS (limit 163840)",
                 nb * 256, lds);
-    auto kern = matvec_q4k_kernel<STEPS, R>;
+    auto kern = matvec_q4k_kernel<STEPS, R, Q5>;
     const int rows_per_wg = waves * R;
     dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block((unsigned)(waves * 64));
     skn_launch(ctx, kern, grid, block, lds, w, x, y, n, nb);
@@ -826,14 +874,14 @@ int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, fl
     return SKN_OK;
 }
 
-template <int R>
+template <int R, bool Q5 = false>
 int dispatch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
     switch ((nb + 15) / 16) {
-        case 1: return launch_q4k<1, R>(ctx, w, n, nb, x, y, waves);
-        case 2: return launch_q4k<2, R>(ctx, w, n, nb, x, y, waves);
-        case 3: return launch_q4k<3, R>(ctx, w, n, nb, x, y, waves);
-        case 4: return launch_q4k<4, R>(ctx, w, n, nb, x, y, waves);
-        default: return launch_q4k<0, R>(ctx, w, n, nb, x, y, waves);
+        case 1: return launch_q4k<1, R, Q5>(ctx, w, n, nb, x, y, waves);
+        case 2: return launch_q4k<2, R, Q5>(ctx, w, n, nb, x, y, waves);
+        case 3: return launch_q4k<3, R, Q5>(ctx, w, n, nb, x, y, waves);
+        case 4: return launch_q4k<4, R, Q5>(ctx, w, n, nb, x, y, waves);
+        default: return launch_q4k<0, R, Q5>(ctx, w, n, nb, x, y, waves);
     }
 }
 
@@ -869,9 +917,9 @@ hipError_t allow_big_lds_q80() {
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
-template <int STEPS, int R>
+template <int STEPS, int R, bool Q5 = false>
 hipError_t allow_big_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R, Q5>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
@@ -883,7 +931,11 @@ int skn_matvec_init(skn_ctx* ctx) {
     hipError_t (*fns[])() = {allow_big_lds<0, 1>, allow_big_lds<1, 1>, allow_big_lds<2, 1>, allow_big_lds<3, 1>,
                              allow_big_lds<4, 1>, allow_big_lds<0, 2>, allow_big_lds<1, 2>, allow_big_lds<2, 2>,
                              allow_big_lds<3, 2>, allow_big_lds<4, 2>, allow_big_lds<0, 4>, allow_big_lds<1, 4>,
-                             allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>};
+                             allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>,
+                             allow_big_lds<0, 1, true>, allow_big_lds<1, 1, true>, allow_big_lds<2, 1, true>,
+                             allow_big_lds<3, 1, true>, allow_big_lds<4, 1, true>, allow_big_lds<0, 2, true>,
+                             allow_big_lds<1, 2, true>, allow_big_lds<2, 2, true>, allow_big_lds<3, 2, true>,
+                             allow_big_lds<4, 2, true>};
     for (auto f : fns) SKN_HIP(ctx, f());
     SKN_HIP(ctx, allow_big_lds_q6k<1>());
     SKN_HIP(ctx, allow_big_lds_q6k<2>());
@@ -940,8 +992,11 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     SKN_REQUIRE(ctx, ((uintptr_t)w_dev & (ggml_type == SKN_TYPE_Q4_K ? 15 : ggml_type == SKN_TYPE_F32 ? 3 : 1)) == 0,
                 SKN_ERR_ARG, "skn_matvec_q: weight pointer is misaligned for its block type");
     const uint8_t* w = (const uint8_t*)w_dev;
-    if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     const int nb = k / be;
+    // Q5_K on the lane map of the Q4_K kernel (16-byte aligned blocks, x within the LDS of a compute unit)
+    if (ggml_type == SKN_TYPE_Q5_K && ((uintptr_t)w_dev & 15) == 0 && nb <= 144 && ctx->opt_matvec_stage == 1)
+        return nb > 32 ? dispatch_q4k<1, true>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, true>(ctx, w, n, nb, x_dev, y_dev, 8);
+    if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;
         if (waves <= 0) waves = 8;

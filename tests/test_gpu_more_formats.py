@@ -67,19 +67,49 @@ STAGED = [(3, "q4_1"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (2
 @pytest.mark.parametrize("n,k", [(7, 11008), (4, 16384), (9, 2048), (3, 256)])
 def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
     """The formats whose rows pass through LDS: several chunks per row with a short last one (k = 11008), the
-    longest row, fewer rows than a workgroup takes -- both kernels against the oracle and against each other."""
+    longest row, fewer rows than a workgroup takes -- every kernel the option selects (0: direct reads, 2: row
+    staged in LDS, 1: the default, which for Q5_K is the kernel on the Q4_K lane map) against the oracle and
+    against each other."""
     raw = synth.weight(qtype, n, k, seed=3 * n + k + qtype)
     x = synth.activation_f32(k, seed=k + 1)
     want = oracle_c.matvec_q(qtype, raw, n, k, x)
     got = {}
     try:
-        for stage in (0, 1):
+        for stage in (0, 1, 2):
             hip.set_option("matvec.stage", stage)
             got[stage] = hip.matvec_q_host(qtype, raw, n, k, x)
             assert oracle_np.rel_err(got[stage], want) <= TOL
     finally:
         hip.set_option("matvec.stage", 1)
-    assert np.abs(got[1] - got[0]).max() <= 1e-5 * np.abs(want).max()  # (fp32 sums in a different order)
+    for stage in (1, 2):  # (fp32 sums in a different order)
+        assert np.abs(got[stage] - got[0]).max() <= 1e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
+def test_q5k_matvec_every_step_count(hip, n, k):
+    """Q5_K rows of one to four unrolled steps (16 superblocks each), a partial last step, the rolled loop beyond
+    four steps, the longest row the lane-map kernel takes (144 superblocks) and one past it (direct kernel)."""
+    raw = synth.weight(13, n, k, seed=n + k)
+    x = synth.activation_f32(k, seed=k + 3)
+    got = hip.matvec_q_host(13, raw, n, k, x)
+    assert oracle_np.rel_err(got, oracle_c.matvec_q(13, raw, n, k, x)) <= TOL
+
+
+def test_q5k_matvec_fifth_bits_alone(hip):
+    """Quants whose nibbles are all zero and whose fifth bits are random, and the reverse: each bit plane of the
+    kernel against the oracle separately (a misplaced qh bit or sub-block shift shows at full scale)."""
+    n, k = 8, 4096
+    rng = np.random.default_rng(5)
+    raw = synth.weight(13, n, k, seed=21).reshape(n, k // 256, 176).copy()
+    x = synth.activation_f32(k, seed=22)
+    only_bits = raw.copy()
+    only_bits[:, :, 48:] = 0
+    only_bits[:, :, 16:48] = rng.integers(0, 256, size=(n, k // 256, 32), dtype=np.uint8)
+    only_nibbles = raw.copy()
+    only_nibbles[:, :, 16:48] = 0
+    for blocks in (only_bits, only_nibbles):
+        got = hip.matvec_q_host(13, blocks.reshape(n, -1), n, k, x)
+        assert oracle_np.rel_err(got, oracle_c.matvec_q(13, blocks.reshape(n, -1), n, k, x)) <= TOL
 
 
 @pytest.mark.parametrize("qtype,name", [(3, "q4_1"), (10, "q2_k")])
