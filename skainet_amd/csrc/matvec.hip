@@ -115,11 +115,13 @@ __device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int 
 
 // Q4K: the scalings of the Q4_K kernel.  Otherwise (Q8_0): x is stored as is and the half-column sums are
 // multiplied by 128, the offset that turns the signed quants into unsigned bytes.
-template <bool Q4K = true>
+// HI: the bit of the float4's position among the lane's sixteen that tells a high-nibble one (8: the second 32 of
+// the 64 activations, as in Q4_K / Q5_K; 4: elements 16..31 of each block of 32, as in Q4_0 / Q4_1).
+template <bool Q4K = true, int HI = 8>
 __device__ __forceinline__ void q4k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
     const int cc = f >> 4, i16 = f & 15;
     const int step = cc >> 6, ln = cc & 63;
-    const float mul = (Q4K && (i16 & 8)) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
+    const float mul = (Q4K && (i16 & HI)) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
     xs[(step * 16 + i16) * kXPitch + ln] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
     float sum = (v.x + v.y) + (v.z + v.w);
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));   // lane ^ 1
@@ -128,7 +130,7 @@ __device__ __forceinline__ void q4k_stage_store_one(const float4& v, int f, floa
     if ((f & 7) == 0) ss[f >> 3] = sum * (Q4K ? 5.9604644775390625e-08f : 128.0f);  // 2^-24, see the scaling note above
 }
 
-template <int J, bool Q4K = true>
+template <int J, bool Q4K = true, int HI = 8>
 __device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, int tid, int nthreads, float4* xs,
                                                 float* ss) {
 #pragma unroll
@@ -136,7 +138,7 @@ __device__ __forceinline__ void q4k_stage_store(const Q4kStage<J>& st, int n4, i
         // a float4 index past the end repeats the last one: same data to the same slot (no branch; whole
         // groups of eight lanes are clamped together because n4 is a multiple of 64)
         const int f = min(tid + j * nthreads, n4 - 1);
-        q4k_stage_store_one<Q4K>(st.v[j], f, xs, ss);
+        q4k_stage_store_one<Q4K, HI>(st.v[j], f, xs, ss);
     }
 }
 
@@ -150,6 +152,70 @@ struct Q4kLoads {
 struct Q5kLoads : Q4kLoads {
     u32x4 ha, hb;
 };
+
+// Q4_0 (18 bytes: f16 d, 16 bytes of nibbles; low nibbles are elements 0..15, high nibbles 16..31; d (q - 8)) and
+// Q4_1 (20 bytes: f16 d, f16 m, nibbles; d q + m) on the same lane map: eight blocks stand where a superblock
+// stands, lane (sub, p) takes blocks 2p and 2p + 1 of its eight -- 36 or 40 contiguous bytes at 4-byte alignment,
+// nine or ten dwords.  Q4_0: dword 0 = d | q0 q1, dwords 1..3, dword 4 = q14 q15 | d', dwords 5..8 the second
+// block's nibbles; the first block's are realigned with v_alignbyte.  Q4_1: every field is an aligned dword.
+constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3;
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+struct Q4xLoads {
+    u32x4 a, b;       // dwords 0..7
+    uint32_t c0, c1;  // dwords 8, 9 (the latter Q4_1 only)
+    bool ok;
+};
+
+template <int R, int F>
+__device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, float (&acc)[R]) {
+    float sum[R][2];
+#pragma unroll
+    for (int half = 0; half < 2; half++) {  // the lane's first and second block
+        float4 xl[4], xh[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            xl[j] = xs[(s * 16 + 8 * half + j) * kXPitch + lane];
+            xh[j] = xs[(s * 16 + 8 * half + 4 + j) * kXPitch + lane];
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const u32x4 &a = L[r].a, &b = L[r].b;
+            uint32_t q[4];
+            if (F == kFmtQ40) {
+                if (half == 0) {
+                    q[0] = __builtin_amdgcn_alignbyte(a.y, a.x, 2), q[1] = __builtin_amdgcn_alignbyte(a.z, a.y, 2);
+                    q[2] = __builtin_amdgcn_alignbyte(a.w, a.z, 2), q[3] = __builtin_amdgcn_alignbyte(b.x, a.w, 2);
+                } else {
+                    q[0] = b.y, q[1] = b.z, q[2] = b.w, q[3] = L[r].c0;
+                }
+            } else {
+                if (half == 0) q[0] = a.y, q[1] = a.z, q[2] = a.w, q[3] = b.x;
+                else q[0] = b.z, q[1] = b.w, q[2] = L[r].c0, q[3] = L[r].c1;
+            }
+            float alo = 0.f, ahi = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) q4k_dot_dword(q[i], xl[i], xh[i], alo, ahi);
+            sum[r][half] = alo + ahi;
+        }
+    }
+    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // the sums of x over the two blocks (x 2^-24)
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float v;
+        if (F == kFmtQ40) {
+            const uint32_t w0 = L[r].a.x, w4 = L[r].b.x;
+            const float d0 = (float)__builtin_bit_cast(half2_t, w0).x, d1 = (float)__builtin_bit_cast(half2_t, w4).y;
+            v = fmaf(d0, fmaf(-8.0f, sx.x, sum[r][0]), d1 * fmaf(-8.0f, sx.y, sum[r][1]));
+        } else {
+            const uint32_t w0 = L[r].a.x, w5 = L[r].b.y;
+            const half2_t h0 = __builtin_bit_cast(half2_t, w0), h1 = __builtin_bit_cast(half2_t, w5);
+            v = fmaf((float)h0.x, sum[r][0], (float)h0.y * sx.x) + fmaf((float)h1.x, sum[r][1], (float)h1.y * sx.y);
+        }
+        acc[r] += L[r].ok ? v : 0.f;
+    }
+}
 
 template <typename LT>
 constexpr bool kIsQ5 = false;
@@ -211,12 +277,15 @@ __device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restr
 // next step, consume the current one.  A compute unit's memory pipeline accepts only so many requests before
 // a wavefront stalls at issue, so the loads are kept one step ahead instead of all up front -- otherwise the
 // x stores (and with them every wavefront at the barrier) would sit behind the issue of a whole row.
-// Q5: Q5_K blocks (eleven chunks, the quants from the fourth on) with the same lane map, staging and scales.
-template <int STEPS, int R, bool Q5 = false>
+// F: Q4_K; Q5_K blocks (eleven chunks, the quants from the fourth on) with the same lane map, staging and scales;
+// Q4_0 / Q4_1, eight blocks for a superblock (nb counts groups of eight).
+template <int STEPS, int R, int F = kFmtQ4K>
 __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                          float* __restrict__ y, int n_rows, int nb) {
-    using Loads = std::conditional_t<Q5, Q5kLoads, Q4kLoads>;
+    constexpr bool Q5 = F == kFmtQ5K, kSmall = F == kFmtQ40 || F == kFmtQ41;
+    using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
+    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : 20, kHi = kSmall ? 4 : 8;
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
@@ -229,7 +298,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     const int row0 = (blockIdx.x * waves + wave) * R;
     const int sub = lane >> 2;  // superblock within the step
     const int p = lane & 3;     // sub-block pair within the superblock
-    const size_t row_chunks = (size_t)nb * kChunks;
+    const size_t row_chunks = kSmall ? (size_t)nb * (kSmallBytes / 2) : (size_t)nb * kChunks;  // (eight blocks: kSmallBytes / 2 chunks)
     const int n4 = nb * 64;  // float4 count of x
 
     // the first J float4 per thread go into registers now; J covers all of x in the unrolled kernels
@@ -246,29 +315,40 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         acc[r] = 0.f;
         row_ok[r] = row0 + r < n_rows;
         // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
-        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + kFirst + 2 * p;
+        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + (kSmall ? 0 : kFirst + 2 * p);
     }
     auto issue = [&](int s, int tie, Loads (&L)[R]) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
-        const int off = min(blk, nb - 1) * kChunks + tie;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const u32x4* bp = rp[r] + off;
-            L[r].qa = bp[0];
-            L[r].qb = bp[1];
-            L[r].h = bp[-kFirst - 2 * p];
-            if constexpr (Q5) {
-                L[r].ha = bp[1 - kFirst - 2 * p];
-                L[r].hb = bp[2 - kFirst - 2 * p];
+            if constexpr (kSmall) {
+                const uint8_t* bp = reinterpret_cast<const uint8_t*>(rp[r]) + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
+                L[r].a = *reinterpret_cast<const u32x4_a4*>(bp);
+                L[r].b = *reinterpret_cast<const u32x4_a4*>(bp + 16);
+                L[r].c0 = *reinterpret_cast<const uint32_t*>(bp + 32);
+                L[r].c1 = F == kFmtQ41 ? *reinterpret_cast<const uint32_t*>(bp + 36) : 0u;
+            } else {
+                const u32x4* bp = rp[r] + min(blk, nb - 1) * kChunks + tie;
+                L[r].qa = bp[0];
+                L[r].qb = bp[1];
+                L[r].h = bp[-kFirst - 2 * p];
+                if constexpr (Q5) {
+                    L[r].ha = bp[1 - kFirst - 2 * p];
+                    L[r].hb = bp[2 - kFirst - 2 * p];
+                }
             }
             L[r].ok = row_ok[r] && blk < nb;
         }
+    };
+    auto step = [&](const Loads (&L)[R], int s, int ln) __attribute__((always_inline)) {
+        if constexpr (kSmall) q4x_step<R, F>(L, xs, ss, s, ln, acc);
+        else q4k_step<R>(L, xs, ss, s, ln, p, acc);
     };
 
     if constexpr (STEPS > 0) {
         Loads L[STEPS][R];
         issue(0, 0, L[0]);
-        q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
+        q4k_stage_store<J, true, kHi>(st, n4, tid, blockDim.x, xs, ss);
         __syncthreads();
         // `tie` is always 0; an empty asm after each step makes it look rewritten from the finished accumulator,
         // which pins the loads of step s+1 between the arithmetic of steps s-1 and s (one step of lookahead) and
@@ -279,22 +359,22 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         for (int s = 0; s < STEPS; s++) {
             if (s + 1 < STEPS) issue(s + 1, tie, L[s + 1]);
             asm volatile("" ::: "memory");  // the loads above stay above the LDS reads below
-            q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
+            step(L[s], s, lane + tie);
             asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
         }
     } else {
         Loads bufa[R], bufb[R];
         issue(0, 0, bufa);
-        q4k_stage_store<J>(st, n4, tid, blockDim.x, xs, ss);
+        q4k_stage_store<J, true, kHi>(st, n4, tid, blockDim.x, xs, ss);
         for (int f = tid + J * blockDim.x; f < n4; f += blockDim.x)
-            q4k_stage_store_one(reinterpret_cast<const float4*>(x)[f], f, xs, ss);
+            q4k_stage_store_one<true, kHi>(reinterpret_cast<const float4*>(x)[f], f, xs, ss);
         __syncthreads();
         for (int s = 0; s < steps; s += 2) {
             if (s + 1 < steps) issue(s + 1, 0, bufb);
-            q4k_step<R>(bufa, xs, ss, s, lane, p, acc);
+            step(bufa, s, lane);
             if (s + 1 < steps) {
                 if (s + 2 < steps) issue(s + 2, 0, bufa);
-                q4k_step<R>(bufb, xs, ss, s + 1, lane, p, acc);
+                step(bufb, s + 1, lane);
             }
         }
     }
@@ -316,8 +396,6 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
 // multiply-add per weight; the offset comes back out as 128 * sum(x of the block), formed once per workgroup
 // while x is staged.  Staging, lookahead and reduction are those of the Q4_K kernel (a lane's 64 activations
 // are the same 64 consecutive elements there and here).
-typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
-
 struct Q80Loads {
     u32x4 w[4];    // dwords 0..15
     uint32_t w16;  // dword 16
@@ -859,14 +937,14 @@ hipError_t allow_big_lds_fused_all() {
     return e;
 }
 
-template <int STEPS, int R, bool Q5 = false>
+template <int STEPS, int R, int F = kFmtQ4K>
 int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
-    if (STEPS > 0 && waves != 8) return launch_q4k<0, R, Q5>(ctx, w, n, nb, x, y, waves);
+    if (STEPS > 0 && waves != 8) return launch_q4k<0, R, F>(ctx, w, n, nb, x, y, waves);
     const int steps = (nb + 15) / 16;
     const size_t lds = (size_t)steps * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
     SKN_REQUIRE(ctx, lds <= 160 * 1024, SKN_ERR_SHAPE, "skn_matvec_q: k = %d needs %zu bytes of LDS (limit 163840)",
                 nb * 256, lds);
-    auto kern = matvec_q4k_kernel<STEPS, R, Q5>;
+    auto kern = matvec_q4k_kernel<STEPS, R, F>;
     const int rows_per_wg = waves * R;
     dim3 grid((unsigned)((n + rows_per_wg - 1) / rows_per_wg)), block((unsigned)(waves * 64));
     skn_launch(ctx, kern, grid, block, lds, w, x, y, n, nb);
@@ -874,14 +952,14 @@ int launch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, fl
     return SKN_OK;
 }
 
-template <int R, bool Q5 = false>
+template <int R, int F = kFmtQ4K>
 int dispatch_q4k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y, int waves) {
     switch ((nb + 15) / 16) {
-        case 1: return launch_q4k<1, R, Q5>(ctx, w, n, nb, x, y, waves);
-        case 2: return launch_q4k<2, R, Q5>(ctx, w, n, nb, x, y, waves);
-        case 3: return launch_q4k<3, R, Q5>(ctx, w, n, nb, x, y, waves);
-        case 4: return launch_q4k<4, R, Q5>(ctx, w, n, nb, x, y, waves);
-        default: return launch_q4k<0, R, Q5>(ctx, w, n, nb, x, y, waves);
+        case 1: return launch_q4k<1, R, F>(ctx, w, n, nb, x, y, waves);
+        case 2: return launch_q4k<2, R, F>(ctx, w, n, nb, x, y, waves);
+        case 3: return launch_q4k<3, R, F>(ctx, w, n, nb, x, y, waves);
+        case 4: return launch_q4k<4, R, F>(ctx, w, n, nb, x, y, waves);
+        default: return launch_q4k<0, R, F>(ctx, w, n, nb, x, y, waves);
     }
 }
 
@@ -917,9 +995,9 @@ hipError_t allow_big_lds_q80() {
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
-template <int STEPS, int R, bool Q5 = false>
+template <int STEPS, int R, int F = kFmtQ4K>
 hipError_t allow_big_lds() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R, Q5>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_kernel<STEPS, R, F>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
@@ -932,10 +1010,12 @@ int skn_matvec_init(skn_ctx* ctx) {
                              allow_big_lds<4, 1>, allow_big_lds<0, 2>, allow_big_lds<1, 2>, allow_big_lds<2, 2>,
                              allow_big_lds<3, 2>, allow_big_lds<4, 2>, allow_big_lds<0, 4>, allow_big_lds<1, 4>,
                              allow_big_lds<2, 4>, allow_big_lds<3, 4>, allow_big_lds<4, 4>,
-                             allow_big_lds<0, 1, true>, allow_big_lds<1, 1, true>, allow_big_lds<2, 1, true>,
-                             allow_big_lds<3, 1, true>, allow_big_lds<4, 1, true>, allow_big_lds<0, 2, true>,
-                             allow_big_lds<1, 2, true>, allow_big_lds<2, 2, true>, allow_big_lds<3, 2, true>,
-                             allow_big_lds<4, 2, true>};
+#define SKN_ALLOW_FMT(F)                                                                                       \
+    allow_big_lds<0, 1, F>, allow_big_lds<1, 1, F>, allow_big_lds<2, 1, F>, allow_big_lds<3, 1, F>,             \
+        allow_big_lds<4, 1, F>, allow_big_lds<0, 2, F>, allow_big_lds<1, 2, F>, allow_big_lds<2, 2, F>,         \
+        allow_big_lds<3, 2, F>, allow_big_lds<4, 2, F>
+                             SKN_ALLOW_FMT(kFmtQ5K), SKN_ALLOW_FMT(kFmtQ40), SKN_ALLOW_FMT(kFmtQ41)};
+#undef SKN_ALLOW_FMT
     for (auto f : fns) SKN_HIP(ctx, f());
     SKN_HIP(ctx, allow_big_lds_q6k<1>());
     SKN_HIP(ctx, allow_big_lds_q6k<2>());
@@ -995,7 +1075,15 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     const int nb = k / be;
     // Q5_K on the lane map of the Q4_K kernel (16-byte aligned blocks, x within the LDS of a compute unit)
     if (ggml_type == SKN_TYPE_Q5_K && ((uintptr_t)w_dev & 15) == 0 && nb <= 144 && ctx->opt_matvec_stage == 1)
-        return nb > 32 ? dispatch_q4k<1, true>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, true>(ctx, w, n, nb, x_dev, y_dev, 8);
+        return nb > 32 ? dispatch_q4k<1, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8);
+    // Q4_0 / Q4_1 likewise, eight blocks standing for a superblock (rows of whole groups of eight are 16-byte aligned)
+    if ((ggml_type == SKN_TYPE_Q4_0 || ggml_type == SKN_TYPE_Q4_1) && k % 256 == 0 && ((uintptr_t)w_dev & 15) == 0 &&
+        k <= 144 * 256 && ctx->opt_matvec_stage == 1) {
+        const int ng = k / 256;
+        if (ggml_type == SKN_TYPE_Q4_0)
+            return ng > 32 ? dispatch_q4k<1, kFmtQ40>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ40>(ctx, w, n, ng, x_dev, y_dev, 8);
+        return ng > 32 ? dispatch_q4k<1, kFmtQ41>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ41>(ctx, w, n, ng, x_dev, y_dev, 8);
+    }
     if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;
