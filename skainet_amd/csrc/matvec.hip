@@ -153,24 +153,60 @@ struct Q5kLoads : Q4kLoads {
     u32x4 ha, hb;
 };
 
-// Q4_0 (18 bytes: f16 d, 16 bytes of nibbles; low nibbles are elements 0..15, high nibbles 16..31; d (q - 8)) and
-// Q4_1 (20 bytes: f16 d, f16 m, nibbles; d q + m) on the same lane map: eight blocks stand where a superblock
-// stands, lane (sub, p) takes blocks 2p and 2p + 1 of its eight -- 36 or 40 contiguous bytes at 4-byte alignment,
-// nine or ten dwords.  Q4_0: dword 0 = d | q0 q1, dwords 1..3, dword 4 = q14 q15 | d', dwords 5..8 the second
-// block's nibbles; the first block's are realigned with v_alignbyte.  Q4_1: every field is an aligned dword.
-constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3;
+// The formats with blocks of 32 on the same lane map: eight blocks stand where a superblock stands, lane (sub, p)
+// takes blocks 2p and 2p + 1 of its eight -- 36 to 48 contiguous bytes at 4-byte alignment, nine to twelve dwords.
+//   Q4_0 (18 bytes: f16 d, 16 bytes of nibbles; low nibbles are elements 0..15, high nibbles 16..31; d (q - 8)):
+//     dword 0 = d | q0 q1, dwords 1..3, dword 4 = q14 q15 | d', dwords 5..8 the second block's nibbles; the first
+//     block's are realigned with v_alignbyte.
+//   Q4_1 (20 bytes: d, f16 m, nibbles; d q + m): every field is an aligned dword.
+//   Q5_0 (22 bytes: d, four bytes of fifth bits -- bit e of the dword belongs to element e --, nibbles; d (q - 16)):
+//     first block realigned (fifth bits and nibbles), second block aligned from dword 6.
+//   Q5_1 (24 bytes: d, m, fifth bits, nibbles; d q + m): aligned.
+// The four fifth bits that go with a dword of nibbles are spread to bit 0 of its four bytes by one multiply
+// ((bits * 0x00204081) & 0x01010101: bit k lands on 8k, no two partial products meet), those of the high nibbles
+// to bit 1, which is the form q5k_dot_dword takes.
+constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5;
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
+typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 
 struct Q4xLoads {
-    u32x4 a, b;       // dwords 0..7
-    uint32_t c0, c1;  // dwords 8, 9 (the latter Q4_1 only)
+    u32x4 a, b, c;  // dwords 0..11 (c: as many as the format has)
     bool ok;
 };
+
+// the fields of the lane's first (half 0) or second block: nibble dwords, fifth bits, scale and offset
+template <int F>
+__device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t (&q)[4], uint32_t& qh, float& d, float& m) {
+    const u32x4 &a = L.a, &b = L.b, &c = L.c;
+    auto lo16 = [](uint32_t w) { return (float)__builtin_bit_cast(half2_t, w).x; };
+    auto hi16 = [](uint32_t w) { return (float)__builtin_bit_cast(half2_t, w).y; };
+    auto al = [](uint32_t hi, uint32_t lo) { return __builtin_amdgcn_alignbyte(hi, lo, 2); };
+    qh = 0u, m = 0.f;
+    if (F == kFmtQ40) {
+        if (half == 0) q[0] = al(a.y, a.x), q[1] = al(a.z, a.y), q[2] = al(a.w, a.z), q[3] = al(b.x, a.w), d = lo16(a.x);
+        else q[0] = b.y, q[1] = b.z, q[2] = b.w, q[3] = c.x, d = hi16(b.x);
+    } else if (F == kFmtQ41) {
+        if (half == 0) q[0] = a.y, q[1] = a.z, q[2] = a.w, q[3] = b.x, d = lo16(a.x), m = hi16(a.x);
+        else q[0] = b.z, q[1] = b.w, q[2] = c.x, q[3] = c.y, d = lo16(b.y), m = hi16(b.y);
+    } else if (F == kFmtQ50) {
+        if (half == 0) qh = al(a.y, a.x), q[0] = al(a.z, a.y), q[1] = al(a.w, a.z), q[2] = al(b.x, a.w), q[3] = al(b.y, b.x), d = lo16(a.x);
+        else qh = b.z, q[0] = b.w, q[1] = c.x, q[2] = c.y, q[3] = c.z, d = hi16(b.y);
+    } else {
+        if (half == 0) qh = a.y, q[0] = a.z, q[1] = a.w, q[2] = b.x, q[3] = b.y, d = lo16(a.x), m = hi16(a.x);
+        else qh = b.w, q[0] = c.x, q[1] = c.y, q[2] = c.z, q[3] = c.w, d = lo16(b.z), m = hi16(b.z);
+    }
+}
 
 template <int R, int F>
 __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
                                          int s, int lane, float (&acc)[R]) {
-    float sum[R][2];
+    constexpr bool kFive = F == kFmtQ50 || F == kFmtQ51;
+    constexpr float kZero = F == kFmtQ40 ? -8.0f : (F == kFmtQ50 ? -16.0f : 0.0f);  // the quant that stands for zero
+    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // the sums of x over the two blocks (x 2^-24)
+    float v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) v[r] = 0.f;
 #pragma unroll
     for (int half = 0; half < 2; half++) {  // the lane's first and second block
         float4 xl[4], xh[4];
@@ -179,42 +215,28 @@ __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* _
             xl[j] = xs[(s * 16 + 8 * half + j) * kXPitch + lane];
             xh[j] = xs[(s * 16 + 8 * half + 4 + j) * kXPitch + lane];
         }
+        const float sxb = half == 0 ? sx.x : sx.y;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const u32x4 &a = L[r].a, &b = L[r].b;
-            uint32_t q[4];
-            if (F == kFmtQ40) {
-                if (half == 0) {
-                    q[0] = __builtin_amdgcn_alignbyte(a.y, a.x, 2), q[1] = __builtin_amdgcn_alignbyte(a.z, a.y, 2);
-                    q[2] = __builtin_amdgcn_alignbyte(a.w, a.z, 2), q[3] = __builtin_amdgcn_alignbyte(b.x, a.w, 2);
-                } else {
-                    q[0] = b.y, q[1] = b.z, q[2] = b.w, q[3] = L[r].c0;
-                }
-            } else {
-                if (half == 0) q[0] = a.y, q[1] = a.z, q[2] = a.w, q[3] = b.x;
-                else q[0] = b.z, q[1] = b.w, q[2] = L[r].c0, q[3] = L[r].c1;
-            }
+            uint32_t q[4], qh;
+            float d, m;
+            q4x_fields<F>(L[r], half, q, qh, d, m);
             float alo = 0.f, ahi = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) q4k_dot_dword(q[i], xl[i], xh[i], alo, ahi);
-            sum[r][half] = alo + ahi;
+            for (int i = 0; i < 4; i++) {
+                if (kFive) {
+                    const uint32_t lo = (((qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u;
+                    const uint32_t hi = (((qh >> (16 + 4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u;
+                    q5k_dot_dword(q[i], lo | (hi << 1), xl[i], xh[i], alo, ahi);
+                } else {
+                    q4k_dot_dword(q[i], xl[i], xh[i], alo, ahi);
+                }
+            }
+            v[r] = fmaf(d, fmaf(kZero, sxb, alo + ahi), fmaf(m, sxb, v[r]));
         }
     }
-    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // the sums of x over the two blocks (x 2^-24)
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        float v;
-        if (F == kFmtQ40) {
-            const uint32_t w0 = L[r].a.x, w4 = L[r].b.x;
-            const float d0 = (float)__builtin_bit_cast(half2_t, w0).x, d1 = (float)__builtin_bit_cast(half2_t, w4).y;
-            v = fmaf(d0, fmaf(-8.0f, sx.x, sum[r][0]), d1 * fmaf(-8.0f, sx.y, sum[r][1]));
-        } else {
-            const uint32_t w0 = L[r].a.x, w5 = L[r].b.y;
-            const half2_t h0 = __builtin_bit_cast(half2_t, w0), h1 = __builtin_bit_cast(half2_t, w5);
-            v = fmaf((float)h0.x, sum[r][0], (float)h0.y * sx.x) + fmaf((float)h1.x, sum[r][1], (float)h1.y * sx.y);
-        }
-        acc[r] += L[r].ok ? v : 0.f;
-    }
+    for (int r = 0; r < R; r++) acc[r] += L[r].ok ? v[r] : 0.f;
 }
 
 template <typename LT>
@@ -282,10 +304,10 @@ __device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restr
 template <int STEPS, int R, int F = kFmtQ4K>
 __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                          float* __restrict__ y, int n_rows, int nb) {
-    constexpr bool Q5 = F == kFmtQ5K, kSmall = F == kFmtQ40 || F == kFmtQ41;
+    constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40;
     using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
-    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : 20, kHi = kSmall ? 4 : 8;
+    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
@@ -325,8 +347,18 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
                 const uint8_t* bp = reinterpret_cast<const uint8_t*>(rp[r]) + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
                 L[r].a = *reinterpret_cast<const u32x4_a4*>(bp);
                 L[r].b = *reinterpret_cast<const u32x4_a4*>(bp + 16);
-                L[r].c0 = *reinterpret_cast<const uint32_t*>(bp + 32);
-                L[r].c1 = F == kFmtQ41 ? *reinterpret_cast<const uint32_t*>(bp + 36) : 0u;
+                L[r].c = u32x4{0u, 0u, 0u, 0u};
+                if (F == kFmtQ40) {
+                    L[r].c.x = *reinterpret_cast<const uint32_t*>(bp + 32);
+                } else if (F == kFmtQ41) {
+                    const u32x2_a4 t = *reinterpret_cast<const u32x2_a4*>(bp + 32);
+                    L[r].c.x = t.x, L[r].c.y = t.y;
+                } else if (F == kFmtQ50) {
+                    const u32x3_a4 t = *reinterpret_cast<const u32x3_a4*>(bp + 32);
+                    L[r].c.x = t.x, L[r].c.y = t.y, L[r].c.z = t.z;
+                } else {
+                    L[r].c = *reinterpret_cast<const u32x4_a4*>(bp + 32);
+                }
             } else {
                 const u32x4* bp = rp[r] + min(blk, nb - 1) * kChunks + tie;
                 L[r].qa = bp[0];
@@ -1014,7 +1046,8 @@ int skn_matvec_init(skn_ctx* ctx) {
     allow_big_lds<0, 1, F>, allow_big_lds<1, 1, F>, allow_big_lds<2, 1, F>, allow_big_lds<3, 1, F>,             \
         allow_big_lds<4, 1, F>, allow_big_lds<0, 2, F>, allow_big_lds<1, 2, F>, allow_big_lds<2, 2, F>,         \
         allow_big_lds<3, 2, F>, allow_big_lds<4, 2, F>
-                             SKN_ALLOW_FMT(kFmtQ5K), SKN_ALLOW_FMT(kFmtQ40), SKN_ALLOW_FMT(kFmtQ41)};
+                             SKN_ALLOW_FMT(kFmtQ5K), SKN_ALLOW_FMT(kFmtQ40), SKN_ALLOW_FMT(kFmtQ41),
+                             SKN_ALLOW_FMT(kFmtQ50), SKN_ALLOW_FMT(kFmtQ51)};
 #undef SKN_ALLOW_FMT
     for (auto f : fns) SKN_HIP(ctx, f());
     SKN_HIP(ctx, allow_big_lds_q6k<1>());
@@ -1076,13 +1109,19 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     // Q5_K on the lane map of the Q4_K kernel (16-byte aligned blocks, x within the LDS of a compute unit)
     if (ggml_type == SKN_TYPE_Q5_K && ((uintptr_t)w_dev & 15) == 0 && nb <= 144 && ctx->opt_matvec_stage == 1)
         return nb > 32 ? dispatch_q4k<1, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8);
-    // Q4_0 / Q4_1 likewise, eight blocks standing for a superblock (rows of whole groups of eight are 16-byte aligned)
-    if ((ggml_type == SKN_TYPE_Q4_0 || ggml_type == SKN_TYPE_Q4_1) && k % 256 == 0 && ((uintptr_t)w_dev & 15) == 0 &&
-        k <= 144 * 256 && ctx->opt_matvec_stage == 1) {
+    // Q4_0 / Q4_1 / Q5_0 / Q5_1 likewise, eight blocks standing for a superblock (rows of whole groups of eight are
+    // 16-byte aligned)
+    if ((ggml_type == SKN_TYPE_Q4_0 || ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1) &&
+        k % 256 == 0 && ((uintptr_t)w_dev & 15) == 0 && k <= 144 * 256 && ctx->opt_matvec_stage == 1) {
         const int ng = k / 256;
-        if (ggml_type == SKN_TYPE_Q4_0)
-            return ng > 32 ? dispatch_q4k<1, kFmtQ40>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ40>(ctx, w, n, ng, x_dev, y_dev, 8);
-        return ng > 32 ? dispatch_q4k<1, kFmtQ41>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ41>(ctx, w, n, ng, x_dev, y_dev, 8);
+#define SKN_SMALL(F) (ng > 32 ? dispatch_q4k<1, F>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, F>(ctx, w, n, ng, x_dev, y_dev, 8))
+        switch (ggml_type) {
+            case SKN_TYPE_Q4_0: return SKN_SMALL(kFmtQ40);
+            case SKN_TYPE_Q4_1: return SKN_SMALL(kFmtQ41);
+            case SKN_TYPE_Q5_0: return SKN_SMALL(kFmtQ50);
+            default: return SKN_SMALL(kFmtQ51);
+        }
+#undef SKN_SMALL
     }
     if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q4_K) {

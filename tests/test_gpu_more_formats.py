@@ -60,7 +60,7 @@ def test_matvec_vs_oracle(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, want) <= TOL
 
 
-STAGED = [(2, "q4_0"), (3, "q4_1"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
+STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
 
 
 @pytest.mark.parametrize("qtype,name", STAGED)
@@ -85,7 +85,7 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
         assert np.abs(got[stage] - got[0]).max() <= 1e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1")])
+@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
@@ -97,10 +97,11 @@ def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
 
 
-@pytest.mark.parametrize("qtype,name,bb", [(2, "q4_0", 18), (3, "q4_1", 20)])
+@pytest.mark.parametrize("qtype,name,bb", [(2, "q4_0", 18), (3, "q4_1", 20), (6, "q5_0", 22), (7, "q5_1", 24)])
 def test_small_block_matvec_field_positions(hip, qtype, name, bb):
-    """Q4_0 / Q4_1 with one block of every pair zeroed, and with only low or only high nibbles set: the realigned
-    first block, the aligned second one and the two nibble planes each against the oracle on their own."""
+    """Q4_0 / Q4_1 / Q5_0 / Q5_1 with one block of every pair zeroed, with only low or only high nibbles set and
+    (the five-bit formats) with only one half of the fifth bits set: the realigned first block, the aligned second
+    one and every bit plane against the oracle on their own."""
     n, k = 8, 2048
     raw = synth.weight(qtype, n, k, seed=31).reshape(n, k // 32, bb).copy()
     x = synth.activation_f32(k, seed=32)
@@ -113,6 +114,12 @@ def test_small_block_matvec_field_positions(hip, qtype, name, bb):
         v = raw.copy()
         v[:, :, bb - 16:] &= mask
         variants.append(v)
+    if bb >= 22:  # the four bytes before the nibbles: fifth bits of elements 0..15 (first two), 16..31 (last two)
+        for lo, hi in ((bb - 20, bb - 18), (bb - 18, bb - 16)):
+            v = raw.copy()
+            v[:, :, bb - 16:] = 0
+            v[:, :, lo:hi] = 0
+            variants.append(v)
     for v in variants:
         got = hip.matvec_q_host(qtype, v.reshape(n, -1), n, k, x)
         assert oracle_np.rel_err(got, oracle_c.matvec_q(qtype, v.reshape(n, -1), n, k, x)) <= TOL
