@@ -269,6 +269,19 @@ def cpu_baseline(qtype, n, k, budget_s=10.0):
     }
 
 
+def bench_other_formats(ctx):
+    """The further formats: matvec at 4096 x 4096 and 4096 x 11008, kernel time and GB/s of block bytes."""
+    out = {}
+    for nn, kk in ((4096, 4096), (4096, 11008)):
+        res = {}
+        for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q3_k", 11), ("q5_k", 13),
+                         ("q8_k", 15), ("iq4_nl", 20), ("iq4_xs", 23), ("f16", 1)):
+            r = bench_matvec(ctx, qt, nn, kk, 200, 20, copies=24, seed=7000 + qt)
+            res[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
+        out[f"{nn}x{kk}"] = res
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -276,7 +289,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm"], default="bench",
+    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats"], default="bench",
                     help="decode / attention / gemm: only that leg (for kernel traces).  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
     ap.add_argument("--no-graph", action="store_true",
@@ -315,6 +328,10 @@ def main():
         print(json.dumps({"mode": "attention", **bench_attention(ctx, min(args.steps, 200), 10)}))
         ctx.close()
         return
+    if args.mode == "formats":
+        print(json.dumps({"mode": "formats", **bench_other_formats(ctx)}))
+        ctx.close()
+        return
     if args.mode == "gemm":
         print(json.dumps({"mode": "gemm", **{f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
                                              for nm, qt, mm, nn, kk in gemm_shapes}}))
@@ -332,12 +349,7 @@ def main():
             extra[name] = {key: (round(r[key], 3) if isinstance(r[key], float) else r[key])
                            for key in ("kernel_us", "kernel_gbs", "hot_kernel_us", "hot_kernel_gbs", "wall_gbs")}
             extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
-        # the further formats (plain streaming kernels): 4096 x 4096 matvec, kernel GB/s
-        other = {}
-        for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q3_k", 11), ("q5_k", 13),
-                         ("q8_k", 15), ("iq4_nl", 20), ("iq4_xs", 23), ("f16", 1)):
-            r = bench_matvec(ctx, qt, 4096, 4096, 200, 20, copies=24, seed=7000 + qt)
-            other[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
+        other = bench_other_formats(ctx)["4096x4096"]
         extra["other_formats_4096x4096"] = other
         extra["dequant_4096x4096"] = {name: bench_dequant(ctx, qt, 4096, 4096)
                                       for name, qt in (("q8_0", Q8_0), ("q4_k", Q4_K), ("q6_k", Q6_K))}
