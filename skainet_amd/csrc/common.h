@@ -65,7 +65,9 @@ struct skn_rope_epilogue {
     float log2_base = 0.f;
 };
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
-                         float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr);
+                         float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr, int ggml_type = SKN_TYPE_Q4_K);
+// the formats the fused kernels take (every matrix of a launch in the same one; k a multiple of 256)
+bool skn_matvec_fusable(int ggml_type);
 
 // Records a failure on the context (or on the context-less slot) and returns `code`.
 int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);

@@ -295,14 +295,15 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
-        // Five launches per layer where the matrices are Q4_K: [norm + q,k,v + rope + cache store], attention,
-        // [Wo + residual], [norm + gate,up + SwiGLU], [Wdown + residual].  A group with a matrix of another
-        // type takes that type's matvec and the row-wise kernels around it.
-        const bool fuse = ctx->opt_llama_fused && H <= 16384;
-        const bool f_qkv = fuse && L.type_q == SKN_TYPE_Q4_K && L.type_k == SKN_TYPE_Q4_K && L.type_v == SKN_TYPE_Q4_K;
-        const bool f_o = fuse && L.type_o == SKN_TYPE_Q4_K;
-        const bool f_gu = fuse && L.type_gate == SKN_TYPE_Q4_K && L.type_up == SKN_TYPE_Q4_K;
-        const bool f_down = fuse && F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
+        // Five launches per layer where the matrices of a group share one of the formats the fused kernels take
+        // (Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1): [norm + q,k,v + rope + cache store], attention, [Wo + residual],
+        // [norm + gate,up + SwiGLU], [Wdown + residual].  A group of mixed or other types takes each type's
+        // matvec and the row-wise kernels around it.
+        const bool fuse = ctx->opt_llama_fused && H <= 16384 && H % 256 == 0;
+        const bool f_qkv = fuse && skn_matvec_fusable(L.type_q) && L.type_k == L.type_q && L.type_v == L.type_q;
+        const bool f_o = fuse && skn_matvec_fusable(L.type_o);
+        const bool f_gu = fuse && skn_matvec_fusable(L.type_gate) && L.type_up == L.type_gate;
+        const bool f_down = ctx->opt_llama_fused && F <= 16384 && F % 256 == 0 && skn_matvec_fusable(L.type_down);
         if (f_qkv) {
             skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, KVD, KVD}};
             skn_rope_epilogue rope;
@@ -314,7 +315,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.head_dim = D;
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2f(c.rope_base);
-            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, H + 2 * KVD, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, H + 2 * KVD, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope, L.type_q));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
@@ -329,7 +330,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
         if (f_o) {
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
-            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD, nullptr, L.type_o));
         } else {
             SKN_TRY(skn_matvec_q(ctx, L.type_o, L.wo, H, H, m->att, m->proj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
@@ -337,7 +338,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         }
         if (f_gu) {
             skn_q4k_segments gu = {{(const uint8_t*)L.w_gate, (const uint8_t*)L.w_up, nullptr}, {F, F, 0}};
-            SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU, nullptr, L.type_gate));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.ffn_norm, m->xn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
@@ -349,7 +350,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         }
         if (f_down) {
             skn_q4k_segments wd = {{(const uint8_t*)L.w_down, nullptr, nullptr}, {H, 0, 0}};
-            SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD, nullptr, L.type_down));
         } else {
             SKN_TRY(skn_matvec_q(ctx, L.type_down, L.w_down, H, F, m->mid, m->proj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);

@@ -175,6 +175,25 @@ struct Q4xLoads {
     bool ok;
 };
 
+// the lane's two blocks: two 16-byte vectors and the format's tail of one to four dwords
+template <int F>
+__device__ __forceinline__ void q4x_load(const uint8_t* bp, Q4xLoads& L) {
+    L.a = *reinterpret_cast<const u32x4_a4*>(bp);
+    L.b = *reinterpret_cast<const u32x4_a4*>(bp + 16);
+    L.c = u32x4{0u, 0u, 0u, 0u};
+    if (F == kFmtQ40) {
+        L.c.x = *reinterpret_cast<const uint32_t*>(bp + 32);
+    } else if (F == kFmtQ41) {
+        const u32x2_a4 t = *reinterpret_cast<const u32x2_a4*>(bp + 32);
+        L.c.x = t.x, L.c.y = t.y;
+    } else if (F == kFmtQ50) {
+        const u32x3_a4 t = *reinterpret_cast<const u32x3_a4*>(bp + 32);
+        L.c.x = t.x, L.c.y = t.y, L.c.z = t.z;
+    } else {
+        L.c = *reinterpret_cast<const u32x4_a4*>(bp + 32);
+    }
+}
+
 // the fields of the lane's first (half 0) or second block: nibble dwords, fifth bits, scale and offset
 template <int F>
 __device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t (&q)[4], uint32_t& qh, float& d, float& m) {
@@ -345,20 +364,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         for (int r = 0; r < R; r++) {
             if constexpr (kSmall) {
                 const uint8_t* bp = reinterpret_cast<const uint8_t*>(rp[r]) + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
-                L[r].a = *reinterpret_cast<const u32x4_a4*>(bp);
-                L[r].b = *reinterpret_cast<const u32x4_a4*>(bp + 16);
-                L[r].c = u32x4{0u, 0u, 0u, 0u};
-                if (F == kFmtQ40) {
-                    L[r].c.x = *reinterpret_cast<const uint32_t*>(bp + 32);
-                } else if (F == kFmtQ41) {
-                    const u32x2_a4 t = *reinterpret_cast<const u32x2_a4*>(bp + 32);
-                    L[r].c.x = t.x, L[r].c.y = t.y;
-                } else if (F == kFmtQ50) {
-                    const u32x3_a4 t = *reinterpret_cast<const u32x3_a4*>(bp + 32);
-                    L[r].c.x = t.x, L[r].c.y = t.y, L[r].c.z = t.z;
-                } else {
-                    L[r].c = *reinterpret_cast<const u32x4_a4*>(bp + 32);
-                }
+                q4x_load<F>(bp, L[r]);
             } else {
                 const u32x4* bp = rp[r] + min(blk, nb - 1) * kChunks + tie;
                 L[r].qa = bp[0];
@@ -810,12 +816,17 @@ __device__ __forceinline__ void q4k_epilogue(const skn_rope_epilogue& rope, cons
 // gate and up paired row by row), optional RMSNorm of x folded into the staging (every workgroup needs all of
 // x anyway, so it also forms sum(x^2) and stores x * r * norm_w), and an epilogue that stores, adds into the
 // residual stream, or applies SwiGLU to a (gate, up) row pair.  Two rows per wavefront.
-template <int STEPS, int EPI, bool NORM>
+// F: the format of all the matrices of the launch, as in matvec_q4k_kernel.
+template <int STEPS, int EPI, bool NORM, int F = kFmtQ4K>
 __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments seg, const float* __restrict__ x,
                                                                const float* __restrict__ norm_w, float eps,
                                                                float* __restrict__ y, int n_out, int nb,
                                                                skn_rope_epilogue rope) {
     constexpr int R = 2;
+    constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40;
+    using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
+    constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
+    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
     float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
@@ -837,7 +848,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int unit = blockIdx.x * 8 + wave;
     const uint8_t* rowp[R];
     bool row_ok[R];
-    const size_t row_bytes = (size_t)nb * 144;
+    const size_t row_bytes = (size_t)nb * (kSmall ? 8 * kSmallBytes : 16 * kChunks);
     if (EPI == SKN_EPI_SWIGLU) {
         const int i = min(unit, n_out - 1);
         row_ok[0] = row_ok[1] = unit < n_out;
@@ -861,16 +872,24 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
             rowp[r] = base + (size_t)row * row_bytes;
         }
     }
-    Q4kLoads L[STEPS][R];
+    Loads L[STEPS][R];
     auto issue = [&](int s, int tie) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
-        const int off = min(blk, nb - 1) * 9 + 1 + 2 * p + tie;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const u32x4* bp = reinterpret_cast<const u32x4*>(rowp[r]) + off;
-            L[s][r].qa = bp[0];
-            L[s][r].qb = bp[1];
-            L[s][r].h = bp[-1 - 2 * p];
+            if constexpr (kSmall) {
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
+                q4x_load<F>(bp, L[s][r]);
+            } else {
+                const u32x4* bp = reinterpret_cast<const u32x4*>(rowp[r]) + min(blk, nb - 1) * kChunks + kFirst + 2 * p + tie;
+                L[s][r].qa = bp[0];
+                L[s][r].qb = bp[1];
+                L[s][r].h = bp[-kFirst - 2 * p];
+                if constexpr (Q5) {
+                    L[s][r].ha = bp[1 - kFirst - 2 * p];
+                    L[s][r].hb = bp[2 - kFirst - 2 * p];
+                }
+            }
             L[s][r].ok = row_ok[r] && blk < nb;
         }
     };
@@ -896,7 +915,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
     }
-    q4k_stage_store<J>(st, n4, tid, 512, xs, ss);
+    q4k_stage_store<J, true, kHi>(st, n4, tid, 512, xs, ss);
     __syncthreads();
     // (after the staging, while the first weights are still on their way)
     Q4kRopeCtx rc;
@@ -914,7 +933,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     for (int s = 0; s < STEPS; s++) {
         if (s + 1 < STEPS) issue(s + 1, tie);
         asm volatile("" ::: "memory");
-        q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
+        if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
+        else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
     const float t0 = wave_sum(acc[0]) * (16777216.0f * rinv);
@@ -922,50 +942,50 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
 }
 
-template <int STEPS, int EPI, bool NORM>
+template <int STEPS, int EPI, bool NORM, int F>
 int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
                      float eps, float* y, const skn_rope_epilogue& rope) {
     const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2)) + 8 * sizeof(float);
     const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
     dim3 grid((unsigned)((units + 7) / 8)), block(512);
-    skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
+    skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM, F>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
 
-template <int STEPS>
+template <int STEPS, int F>
 int dispatch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
                        float eps, float* y, int epi, const skn_rope_epilogue& rope) {
     const bool norm = norm_w != nullptr;
     if (epi == SKN_EPI_ROPE)
-        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ROPE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
-                    : launch_q4k_fused<STEPS, SKN_EPI_ROPE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ROPE, true, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_ROPE, false, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
     if (epi == SKN_EPI_SWIGLU)
-        return norm ? launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
-                    : launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, true, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_SWIGLU, false, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
     if (epi == SKN_EPI_ADD)
-        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ADD, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
-                    : launch_q4k_fused<STEPS, SKN_EPI_ADD, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
-    return norm ? launch_q4k_fused<STEPS, SKN_EPI_STORE, true>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
-                : launch_q4k_fused<STEPS, SKN_EPI_STORE, false>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
+        return norm ? launch_q4k_fused<STEPS, SKN_EPI_ADD, true, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                    : launch_q4k_fused<STEPS, SKN_EPI_ADD, false, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
+    return norm ? launch_q4k_fused<STEPS, SKN_EPI_STORE, true, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope)
+                : launch_q4k_fused<STEPS, SKN_EPI_STORE, false, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, rope);
 }
 
-template <int STEPS, int EPI, bool NORM>
+template <int STEPS, int EPI, bool NORM, int F>
 hipError_t allow_big_lds_fused() {
-    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_fused_kernel<STEPS, EPI, NORM>),
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q4k_fused_kernel<STEPS, EPI, NORM, F>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 
-template <int STEPS>
+template <int STEPS, int F>
 hipError_t allow_big_lds_fused_all() {
-    hipError_t e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, false>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, true>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, false>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, true>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, false>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, true>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, false>();
-    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, true>();
+    hipError_t e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, false, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_STORE, true, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, false, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ADD, true, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, false, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_SWIGLU, true, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, false, F>();
+    if (e == hipSuccess) e = allow_big_lds_fused<STEPS, SKN_EPI_ROPE, true, F>();
     return e;
 }
 
@@ -1058,16 +1078,31 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_HIP(ctx, allow_big_lds_q80<2>());
     SKN_HIP(ctx, allow_big_lds_q80<3>());
     SKN_HIP(ctx, allow_big_lds_q80<4>());
-    SKN_HIP(ctx, allow_big_lds_fused_all<1>());
-    SKN_HIP(ctx, allow_big_lds_fused_all<2>());
-    SKN_HIP(ctx, allow_big_lds_fused_all<3>());
-    SKN_HIP(ctx, allow_big_lds_fused_all<4>());
+#define SKN_ALLOW_FUSED(F)                              \
+    SKN_HIP(ctx, (allow_big_lds_fused_all<1, F>()));    \
+    SKN_HIP(ctx, (allow_big_lds_fused_all<2, F>()));    \
+    SKN_HIP(ctx, (allow_big_lds_fused_all<3, F>()));    \
+    SKN_HIP(ctx, (allow_big_lds_fused_all<4, F>()))
+    SKN_ALLOW_FUSED(kFmtQ4K);
+    SKN_ALLOW_FUSED(kFmtQ5K);
+    SKN_ALLOW_FUSED(kFmtQ40);
+    SKN_ALLOW_FUSED(kFmtQ41);
+    SKN_ALLOW_FUSED(kFmtQ50);
+    SKN_ALLOW_FUSED(kFmtQ51);
+#undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
 
-// Fused Q4_K matvec for the decoder; k <= 16384 (four unrolled steps).  Returns SKN_ERR_SHAPE otherwise.
+bool skn_matvec_fusable(int ggml_type) {
+    return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
+           ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1;
+}
+
+// Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
+// Returns SKN_ERR_SHAPE otherwise.
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
-                         float eps, float* y, int epi, const skn_rope_epilogue* rope_in) {
+                         float eps, float* y, int epi, const skn_rope_epilogue* rope_in, int ggml_type) {
+    SKN_REQUIRE(ctx, skn_matvec_fusable(ggml_type), SKN_ERR_TYPE, "fused matvec: ggml type %d has no fused kernel", ggml_type);
     SKN_REQUIRE(ctx, k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_SHAPE, "fused Q4_K matvec: unsupported k %d", k);
     skn_rope_epilogue rope;
     if (epi == SKN_EPI_ROPE) {
@@ -1080,12 +1115,22 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
                     rope.head_dim);
     }
     const int nb = k / 256;
-    switch ((nb + 15) / 16) {
-        case 1: return dispatch_q4k_fused<1>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
-        case 2: return dispatch_q4k_fused<2>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
-        case 3: return dispatch_q4k_fused<3>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
-        default: return dispatch_q4k_fused<4>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);
+#define SKN_FUSED(F)                                                                                      \
+    switch ((nb + 15) / 16) {                                                                             \
+        case 1: return dispatch_q4k_fused<1, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);       \
+        case 2: return dispatch_q4k_fused<2, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);       \
+        case 3: return dispatch_q4k_fused<3, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);       \
+        default: return dispatch_q4k_fused<4, F>(ctx, seg, n_out, nb, x, norm_w, eps, y, epi, rope);      \
     }
+    switch (ggml_type) {
+        case SKN_TYPE_Q5_K: SKN_FUSED(kFmtQ5K)
+        case SKN_TYPE_Q4_0: SKN_FUSED(kFmtQ40)
+        case SKN_TYPE_Q4_1: SKN_FUSED(kFmtQ41)
+        case SKN_TYPE_Q5_0: SKN_FUSED(kFmtQ50)
+        case SKN_TYPE_Q5_1: SKN_FUSED(kFmtQ51)
+        default: SKN_FUSED(kFmtQ4K)
+    }
+#undef SKN_FUSED
 }
 
 extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev,

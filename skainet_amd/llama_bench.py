@@ -8,8 +8,10 @@ import numpy as np
 from . import llama
 
 
-def run(ctx, prompt_len=512, steps=128, seed=11, share_layers=False):
-    cfg = llama.Config(max_tokens=1024)
+def run(ctx, prompt_len=512, steps=128, seed=11, share_layers=False, matrix_type=None):
+    """matrix_type: a ggml type id for the seven matrices of every layer instead of Q4_K."""
+    types = {} if matrix_type is None else {m: matrix_type for m in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")}
+    cfg = llama.Config(max_tokens=1024, matrix_types=types)
     t0 = time.perf_counter()
     model = llama.LlamaModel(ctx, cfg, seed=seed, share_layers=share_layers)
     build_s = time.perf_counter() - t0
