@@ -300,12 +300,12 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         // [norm + gate,up + SwiGLU], [Wdown + residual].  A group of mixed or other types takes each type's
         // matvec and the row-wise kernels around it.
         const bool fuse = ctx->opt_llama_fused && H <= 16384 && H % 256 == 0;
-        const bool f_qkv = fuse && skn_matvec_fusable(L.type_q) && L.type_k == L.type_q && L.type_v == L.type_q;
+        // (q, k, v of different fusable formats: one fused launch per format, each with the rows of its matrices only)
+        const bool f_qkv = fuse && skn_matvec_fusable(L.type_q) && skn_matvec_fusable(L.type_k) && skn_matvec_fusable(L.type_v);
         const bool f_o = fuse && skn_matvec_fusable(L.type_o);
         const bool f_gu = fuse && skn_matvec_fusable(L.type_gate) && L.type_up == L.type_gate;
         const bool f_down = ctx->opt_llama_fused && F <= 16384 && F % 256 == 0 && skn_matvec_fusable(L.type_down);
         if (f_qkv) {
-            skn_q4k_segments qkv = {{(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv}, {H, KVD, KVD}};
             skn_rope_epilogue rope;
             rope.pos_dev = m->state + 1;
             rope.page_table = kv->page_table_dev;
@@ -315,7 +315,17 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.head_dim = D;
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2f(c.rope_base);
-            SKN_TRY(skn_matvec_q4k_fused(ctx, qkv, H + 2 * KVD, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope, L.type_q));
+            const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
+            const uint8_t* mats[3] = {(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv};
+            bool done[3] = {false, false, false};
+            for (int i = 0; i < 3; i++) {
+                if (done[i]) continue;
+                skn_q4k_segments part = {{nullptr, nullptr, nullptr}, {0, 0, 0}};
+                int n_out = 0;
+                for (int j = i; j < 3; j++)
+                    if (types[j] == types[i]) part.w[j] = mats[j], part.rows[j] = rows[j], n_out += rows[j], done[j] = true;
+                SKN_TRY(skn_matvec_q4k_fused(ctx, part, n_out, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope, types[i]));
+            }
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);

@@ -166,6 +166,7 @@ struct Q5kLoads : Q4kLoads {
 // ((bits * 0x00204081) & 0x01010101: bit k lands on 8k, no two partial products meet), those of the high nibbles
 // to bit 1, which is the form q5k_dot_dword takes.
 constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5;
+constexpr int kFmtQ6K = 6;  // (fused kernels only: the lane map, staging and step of matvec_q6k_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
@@ -823,14 +824,14 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                                                                float* __restrict__ y, int n_out, int nb,
                                                                skn_rope_epilogue rope) {
     constexpr int R = 2;
-    constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40;
-    using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
+    constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, kSmall = F >= kFmtQ40 && !Q6;
+    using Loads = std::conditional_t<Q6, Q6kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
     constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
     float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
-    float* red = ss + STEPS * 128;  // eight partial sums of x^2 (all LDS here is dynamic)
+    float* red = ss + STEPS * (Q6 ? 256 : 128);  // eight partial sums of x^2 (all LDS here is dynamic)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane >> 2, p = lane & 3;
     const int n4 = nb * 64;
@@ -848,7 +849,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int unit = blockIdx.x * 8 + wave;
     const uint8_t* rowp[R];
     bool row_ok[R];
-    const size_t row_bytes = (size_t)nb * (kSmall ? 8 * kSmallBytes : 16 * kChunks);
+    const size_t row_bytes = (size_t)nb * (Q6 ? 210 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
     if (EPI == SKN_EPI_SWIGLU) {
         const int i = min(unit, n_out - 1);
         row_ok[0] = row_ok[1] = unit < n_out;
@@ -877,7 +878,15 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         const int blk = s * 16 + sub;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if constexpr (kSmall) {
+            if constexpr (Q6) {
+                const int n = p >> 1, hsel = p & 1;
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 210;
+                L[s][r].la = *reinterpret_cast<const u32x4_a2*>(bp + 64 * n + 16 * hsel);
+                L[s][r].lb = *reinterpret_cast<const u32x4_a2*>(bp + 64 * n + 32 + 16 * hsel);
+                L[s][r].h = *reinterpret_cast<const u32x4_a2*>(bp + 128 + 32 * n + 16 * hsel);
+                L[s][r].sc = *reinterpret_cast<const u32x2_a2*>(bp + 192 + 8 * n);
+                L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 208);
+            } else if constexpr (kSmall) {
                 const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
                 q4x_load<F>(bp, L[s][r]);
             } else {
@@ -915,7 +924,12 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
     }
-    q4k_stage_store<J, true, kHi>(st, n4, tid, 512, xs, ss);
+    if constexpr (Q6) {
+#pragma unroll
+        for (int jj = 0; jj < J; jj++) q6k_stage_store_one(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
+    } else {
+        q4k_stage_store<J, true, kHi>(st, n4, tid, 512, xs, ss);
+    }
     __syncthreads();
     // (after the staging, while the first weights are still on their way)
     Q4kRopeCtx rc;
@@ -933,7 +947,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     for (int s = 0; s < STEPS; s++) {
         if (s + 1 < STEPS) issue(s + 1, tie);
         asm volatile("" ::: "memory");
-        if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
+        if constexpr (Q6) q6k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
+        else if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
         else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
@@ -945,7 +960,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
 template <int STEPS, int EPI, bool NORM, int F>
 int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
                      float eps, float* y, const skn_rope_epilogue& rope) {
-    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2)) + 8 * sizeof(float);
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * (F == kFmtQ6K ? sizeof(float4) : sizeof(float2))) + 8 * sizeof(float);
     const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
     dim3 grid((unsigned)((units + 7) / 8)), block(512);
     skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM, F>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
@@ -1089,13 +1104,15 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_ALLOW_FUSED(kFmtQ41);
     SKN_ALLOW_FUSED(kFmtQ50);
     SKN_ALLOW_FUSED(kFmtQ51);
+    SKN_ALLOW_FUSED(kFmtQ6K);
 #undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
 
 bool skn_matvec_fusable(int ggml_type) {
     return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
-           ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1;
+           ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
+           ggml_type == SKN_TYPE_Q6_K;
 }
 
 // Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
@@ -1109,8 +1126,10 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         SKN_REQUIRE(ctx, rope_in && rope_in->pos_dev && rope_in->page_table && rope_in->k_pool && rope_in->v_pool,
                     SKN_ERR_ARG, "fused Q4_K matvec: the rotary epilogue needs its cache arguments");
         rope = *rope_in;
+        // (a launch may carry a subset of q, k, v: an absent matrix has no rows)
         SKN_REQUIRE(ctx, rope.head_dim > 0 && rope.head_dim % 2 == 0 && seg.rows[0] % rope.head_dim == 0 &&
-                             seg.rows[1] == rope.n_head * rope.head_dim && seg.rows[2] == seg.rows[1],
+                             (seg.rows[1] == 0 || seg.rows[1] == rope.n_head * rope.head_dim) &&
+                             (seg.rows[2] == 0 || seg.rows[2] == rope.n_head * rope.head_dim),
                     SKN_ERR_SHAPE, "fused Q4_K matvec: q/k/v rows do not match %d heads of %d", rope.n_head,
                     rope.head_dim);
     }
@@ -1128,6 +1147,7 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         case SKN_TYPE_Q4_1: SKN_FUSED(kFmtQ41)
         case SKN_TYPE_Q5_0: SKN_FUSED(kFmtQ50)
         case SKN_TYPE_Q5_1: SKN_FUSED(kFmtQ51)
+        case SKN_TYPE_Q6_K: SKN_FUSED(kFmtQ6K)
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED
