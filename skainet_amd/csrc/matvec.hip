@@ -166,7 +166,7 @@ struct Q5kLoads : Q4kLoads {
 // ((bits * 0x00204081) & 0x01010101: bit k lands on 8k, no two partial products meet), those of the high nibbles
 // to bit 1, which is the form q5k_dot_dword takes.
 constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5;
-constexpr int kFmtQ6K = 6;  // (fused kernels only: the lane map, staging and step of matvec_q6k_kernel)
+constexpr int kFmtQ6K = 6, kFmtQ80 = 7;  // (fused kernels only: the lane maps, staging and steps of matvec_q6k_kernel / matvec_q80_pairs_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
@@ -824,8 +824,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                                                                float* __restrict__ y, int n_out, int nb,
                                                                skn_rope_epilogue rope) {
     constexpr int R = 2;
-    constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, kSmall = F >= kFmtQ40 && !Q6;
-    using Loads = std::conditional_t<Q6, Q6kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>;
+    constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, Q8 = F == kFmtQ80, kSmall = F >= kFmtQ40 && !Q6 && !Q8;
+    using Loads = std::conditional_t<Q8, Q80Loads, std::conditional_t<Q6, Q6kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
     constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
     extern __shared__ float4 lds4[];
@@ -849,7 +849,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int unit = blockIdx.x * 8 + wave;
     const uint8_t* rowp[R];
     bool row_ok[R];
-    const size_t row_bytes = (size_t)nb * (Q6 ? 210 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
+    const size_t row_bytes = (size_t)nb * (Q8 ? 272 : Q6 ? 210 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
     if (EPI == SKN_EPI_SWIGLU) {
         const int i = min(unit, n_out - 1);
         row_ok[0] = row_ok[1] = unit < n_out;
@@ -878,7 +878,14 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         const int blk = s * 16 + sub;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if constexpr (Q6) {
+            if constexpr (Q8) {  // lane = pair of blocks, 64 pairs per step
+                const int pr = s * 64 + lane, npairs = 4 * nb;
+                const uint8_t* bp = rowp[r] + (size_t)(min(pr, npairs - 1) + tie) * 68;
+#pragma unroll
+                for (int i = 0; i < 4; i++) L[s][r].w[i] = reinterpret_cast<const u32x4_a4*>(bp)[i];
+                L[s][r].w16 = *reinterpret_cast<const uint32_t*>(bp + 64);
+                L[s][r].ok = row_ok[r] && pr < npairs;
+            } else if constexpr (Q6) {
                 const int n = p >> 1, hsel = p & 1;
                 const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 210;
                 L[s][r].la = *reinterpret_cast<const u32x4_a2*>(bp + 64 * n + 16 * hsel);
@@ -899,7 +906,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                     L[s][r].hb = bp[2 - kFirst - 2 * p];
                 }
             }
-            L[s][r].ok = row_ok[r] && blk < nb;
+            if constexpr (!Q8) L[s][r].ok = row_ok[r] && blk < nb;
         }
     };
     issue(0, 0);
@@ -924,7 +931,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
     }
-    if constexpr (Q6) {
+    if constexpr (Q8) {
+        q4k_stage_store<J, false>(st, n4, tid, 512, xs, ss);
+    } else if constexpr (Q6) {
 #pragma unroll
         for (int jj = 0; jj < J; jj++) q6k_stage_store_one(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
     } else {
@@ -947,13 +956,15 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     for (int s = 0; s < STEPS; s++) {
         if (s + 1 < STEPS) issue(s + 1, tie);
         asm volatile("" ::: "memory");
-        if constexpr (Q6) q6k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
+        if constexpr (Q8) q80_step<R>(L[s], xs, ss, s, lane + tie, acc);
+        else if constexpr (Q6) q6k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
         else if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
         else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
-    const float t0 = wave_sum(acc[0]) * (16777216.0f * rinv);
-    const float t1 = wave_sum(acc[1]) * (16777216.0f * rinv);
+    const float back = Q8 ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
+    const float t0 = wave_sum(acc[0]) * back;
+    const float t1 = wave_sum(acc[1]) * back;
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
 }
 
@@ -1105,6 +1116,7 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_ALLOW_FUSED(kFmtQ50);
     SKN_ALLOW_FUSED(kFmtQ51);
     SKN_ALLOW_FUSED(kFmtQ6K);
+    SKN_ALLOW_FUSED(kFmtQ80);
 #undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
@@ -1112,7 +1124,7 @@ int skn_matvec_init(skn_ctx* ctx) {
 bool skn_matvec_fusable(int ggml_type) {
     return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
            ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
-           ggml_type == SKN_TYPE_Q6_K;
+           ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0;
 }
 
 // Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
@@ -1120,6 +1132,12 @@ bool skn_matvec_fusable(int ggml_type) {
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
                          float eps, float* y, int epi, const skn_rope_epilogue* rope_in, int ggml_type) {
     SKN_REQUIRE(ctx, skn_matvec_fusable(ggml_type), SKN_ERR_TYPE, "fused matvec: ggml type %d has no fused kernel", ggml_type);
+    {
+        const uintptr_t mask = ggml_type == SKN_TYPE_Q6_K ? 1 : ggml_type == SKN_TYPE_Q8_0 ? 3 : 15;
+        for (int i = 0; i < 3; i++)
+            SKN_REQUIRE(ctx, seg.rows[i] == 0 || (seg.w[i] && ((uintptr_t)seg.w[i] & mask) == 0), SKN_ERR_ARG,
+                        "fused matvec: weights of type %d must be %d-byte aligned", ggml_type, (int)mask + 1);
+    }
     SKN_REQUIRE(ctx, k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_SHAPE, "fused Q4_K matvec: unsupported k %d", k);
     skn_rope_epilogue rope;
     if (epi == SKN_EPI_ROPE) {
@@ -1148,6 +1166,7 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         case SKN_TYPE_Q5_0: SKN_FUSED(kFmtQ50)
         case SKN_TYPE_Q5_1: SKN_FUSED(kFmtQ51)
         case SKN_TYPE_Q6_K: SKN_FUSED(kFmtQ6K)
+        case SKN_TYPE_Q8_0: SKN_FUSED(kFmtQ80)
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED
