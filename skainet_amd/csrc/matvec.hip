@@ -1,8 +1,10 @@
-// Batch-1 quantized matvec  y[n] = sum_k deq(W)[n,k] * x[k]  for GGUF Q4_K, Q8_0 and Q6_K weights.
+// Batch-1 quantized matvec  y[n] = sum_k deq(W)[n,k] * x[k]  for GGUF Q4_K, Q8_0 and Q6_K weights, and -- on the
+// Q4_K kernel's lane map -- Q5_K, Q4_0, Q4_1, Q5_0 and Q5_1; the fused forms the decoder uses (norm folded into the
+// staging of x, several matrices per launch, residual / SwiGLU / rotary + cache-store epilogues) for all of these.
 //
-// The op is bound by the HBM read of the weight blocks (0.5625 / 1.0625 / 0.8203 bytes per weight); x is
-// read once per workgroup and y written once.  One wavefront owns one output row, so the only cross-lane
-// traffic is a single DPP reduction per row and rows never need atomics.
+// The op is bound by the HBM read of the weight blocks (0.5625 / 1.0625 / 0.8203 bytes per weight for the first
+// three); x is read once per workgroup and y written once.  One wavefront owns one output row, so the only
+// cross-lane traffic is a single DPP reduction per row and rows never need atomics.
 #include "common.h"
 #include <type_traits>
 
