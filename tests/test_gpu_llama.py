@@ -292,6 +292,29 @@ def test_fused_groups_of_further_formats(hip, qtype, name, group):
     _decode_against_oracle(hip, cfg, w, 5)
 
 
+@pytest.mark.parametrize("qtype,name", [(12, "q4_k"), (13, "q5_k"), (2, "q4_0"), (6, "q5_0"), (14, "q6_k"), (8, "q8_0")])
+@pytest.mark.parametrize("ffn", [8192, 11008, 14336])
+def test_fused_down_projection_of_two_to_four_steps(hip, qtype, name, ffn):
+    """Rows of 8192, 11008 and 14336 weights take two, three and four unrolled steps of the fused kernel (4096
+    weights per step): the down projection of a one-layer model in every format that has a fused kernel."""
+    cfg = llama.Config(n_layer=1, hidden=512, ffn=ffn, n_head=4, n_kv_head=2, head_dim=128, vocab=512, max_tokens=32,
+                       page_tokens=16, matrix_types={"w_down": qtype})
+    w = llama.random_weights(cfg, seed=ffn + qtype)
+    assert w["l0.w_down"][0] == qtype
+    _decode_against_oracle(hip, cfg, w, 3)
+
+
+@pytest.mark.parametrize("group,qtype", [("qkv", 12), ("qkv", 13), ("gu", 2), ("gu", 14), ("o", 6), ("o", 8)])
+def test_fused_groups_of_two_steps(hip, group, qtype):
+    """hidden = 8192: every group reads rows of two steps -- the rotary, SwiGLU and residual epilogues and the
+    norm folded into a two-step staging, one group at a time in another format."""
+    mats = {"qkv": ("wq", "wk", "wv"), "o": ("wo",), "gu": ("w_gate", "w_up"), "down": ("w_down",)}[group]
+    cfg = llama.Config(n_layer=1, hidden=8192, ffn=512, n_head=64, n_kv_head=4, head_dim=128, vocab=256, max_tokens=32,
+                       page_tokens=16, matrix_types={m: qtype for m in mats})
+    w = llama.random_weights(cfg, seed=3 + qtype)
+    _decode_against_oracle(hip, cfg, w, 3)
+
+
 @pytest.mark.parametrize("tq,tk,tv", [(12, 12, 14), (13, 2, 14), (14, 12, 12), (12, 8, 14), (12, 10, 12)])
 def test_qkv_of_mixed_formats(hip, tq, tk, tv):
     """q, k and v of different formats (value projections with more bits, as mixed quantizations have them): one
