@@ -362,6 +362,10 @@ def main():
         try:
             from skainet_amd import llama_bench
             extra["decode_7b_q4_k"] = llama_bench.run(ctx)
+            # the same shape as mixed quantizations have it: Q6_K value and down projections in every second layer
+            mix = {f"l{i}.{m}": Q6_K for i in range(0, 32, 2) for m in ("wv", "w_down")}
+            r = llama_bench.run(ctx, steps=64, matrix_types=mix)
+            extra["decode_7b_q4_k_q6_k_mix"] = {key: r[key] for key in ("decode_tok_s", "ms_per_token", "prefill_ms", "weight_bytes_per_token")}
         except Exception as e:  # the decoder leg reports its own absence instead of failing the headline
             extra["decode_7b_q4_k"] = {"error": f"{type(e).__name__}: {e}"}
 

@@ -8,9 +8,11 @@ import numpy as np
 from . import llama
 
 
-def run(ctx, prompt_len=512, steps=128, seed=11, share_layers=False, matrix_type=None):
-    """matrix_type: a ggml type id for the seven matrices of every layer instead of Q4_K."""
+def run(ctx, prompt_len=512, steps=128, seed=11, share_layers=False, matrix_type=None, matrix_types=None):
+    """matrix_type: a ggml type id for the seven matrices of every layer instead of Q4_K; matrix_types: per-matrix
+    types as llama.Config takes them (e.g. {"l0.wv": 14})."""
     types = {} if matrix_type is None else {m: matrix_type for m in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")}
+    types.update(matrix_types or {})
     cfg = llama.Config(max_tokens=1024, matrix_types=types)
     t0 = time.perf_counter()
     model = llama.LlamaModel(ctx, cfg, seed=seed, share_layers=share_layers)
