@@ -102,9 +102,9 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention),
  * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel),
  * "llama.fused" (1 = fused per-layer kernels in the decode step, the default: for every group of matrices whose
- * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, Q6_K, Q8_0), "gemm.tile" (0 = choose, 1 = 64-row tiles,
+ * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
- * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1, rows staged through LDS for the other
+ * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL, rows staged through LDS for the other
  * formats with 4-byte-multiple blocks; 2 = staged rows for all of those; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);

@@ -296,7 +296,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
         // Five launches per layer where the matrices of a group share one of the formats the fused kernels take
-        // (Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, Q6_K, Q8_0): [norm + q,k,v + rope + cache store], attention, [Wo + residual],
+        // (Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0): [norm + q,k,v + rope + cache store], attention, [Wo + residual],
         // [norm + gate,up + SwiGLU], [Wdown + residual].  A group of mixed or other types takes each type's
         // matvec and the row-wise kernels around it.
         const bool fuse = ctx->opt_llama_fused && H <= 16384 && H % 256 == 0;

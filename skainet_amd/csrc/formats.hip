@@ -5,7 +5,7 @@
 // once (explicitly rounded intrinsics, so no contraction can change a bit) -- serves a dequantization kernel
 // (one thread per four outputs, 16-byte stores) and a batch-1 matvec (one wavefront per row, the lane's four
 // weights against one aligned float4 of x, DPP reduction; for blocks of a multiple of four bytes the row passes
-// through LDS first).  These are plain streaming kernels: Q5_K, Q4_0, Q4_1, Q5_0 and Q5_1 reach them only when a
+// through LDS first).  These are plain streaming kernels: Q5_K, Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL reach them only when a
 // row or pointer is off the 16-byte grid -- otherwise their matvec runs on the lane map of the Q4_K kernel
 // (matvec.hip), like the hand-tuned Q4_K, Q8_0 and Q6_K.
 #include "common.h"

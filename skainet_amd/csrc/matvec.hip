@@ -1,5 +1,5 @@
 // Batch-1 quantized matvec  y[n] = sum_k deq(W)[n,k] * x[k]  for GGUF Q4_K, Q8_0 and Q6_K weights, and -- on the
-// Q4_K kernel's lane map -- Q5_K, Q4_0, Q4_1, Q5_0 and Q5_1; the fused forms the decoder uses (norm folded into the
+// Q4_K kernel's lane map -- Q5_K, Q4_0, Q4_1, Q5_0, Q5_1 and IQ4_NL; the fused forms the decoder uses (norm folded into the
 // staging of x, several matrices per launch, residual / SwiGLU / rotary + cache-store epilogues) for all of these.
 //
 // The op is bound by the HBM read of the weight blocks (0.5625 / 1.0625 / 0.8203 bytes per weight for the first
@@ -167,7 +167,7 @@ struct Q5kLoads : Q4kLoads {
 // The four fifth bits that go with a dword of nibbles are spread to bit 0 of its four bytes by one multiply
 // ((bits * 0x00204081) & 0x01010101: bit k lands on 8k, no two partial products meet), those of the high nibbles
 // to bit 1, which is the form q5k_dot_dword takes.
-constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5;
+constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5, kFmtIQ4NL = 8;
 constexpr int kFmtQ6K = 6, kFmtQ80 = 7;  // (fused kernels only: the lane maps, staging and steps of matvec_q6k_kernel / matvec_q80_pairs_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
@@ -178,13 +178,34 @@ struct Q4xLoads {
     bool ok;
 };
 
+//   IQ4_NL (18 bytes, the layout of Q4_0; d table[q] with sixteen signed values): four nibbles at a time are looked
+//     up with two v_perm_b32 (entries 0..7 and 8..15) and a bit select on bit 3; the table holds value + 128, so
+//     the bytes are unsigned for v_cvt_f32_ubyteN and the 128 comes back out as 128 sum(x of the block), which the
+//     staging forms (x itself is staged unscaled for this format).
+__device__ __forceinline__ uint32_t iq4nl_lookup4(uint32_t idx) {  // idx: four table indices, one per byte
+    // -127 -104 -83 -65 | -49 -35 -22 -10 | 1 13 25 38 | 53 69 89 113, each plus 128
+    constexpr uint32_t T0 = 0x3F2D1801u, T1 = 0x766A5D4Fu, T2 = 0xA6998D81u, T3 = 0xF1D9C5B5u;
+    const uint32_t sel = idx & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel), hi = __builtin_amdgcn_perm(T3, T2, sel);
+    const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
+    return (hi & m) | (lo & ~m);
+}
+
+__device__ __forceinline__ float iq4nl_dot4(uint32_t t, const float4& x, float s) {
+    s = fmaf((float)(t & 0xFFu), x.x, s);
+    s = fmaf((float)((t >> 8) & 0xFFu), x.y, s);
+    s = fmaf((float)((t >> 16) & 0xFFu), x.z, s);
+    s = fmaf((float)(t >> 24), x.w, s);
+    return s;
+}
+
 // the lane's two blocks: two 16-byte vectors and the format's tail of one to four dwords
 template <int F>
 __device__ __forceinline__ void q4x_load(const uint8_t* bp, Q4xLoads& L) {
     L.a = *reinterpret_cast<const u32x4_a4*>(bp);
     L.b = *reinterpret_cast<const u32x4_a4*>(bp + 16);
     L.c = u32x4{0u, 0u, 0u, 0u};
-    if (F == kFmtQ40) {
+    if (F == kFmtQ40 || F == kFmtIQ4NL) {
         L.c.x = *reinterpret_cast<const uint32_t*>(bp + 32);
     } else if (F == kFmtQ41) {
         const u32x2_a4 t = *reinterpret_cast<const u32x2_a4*>(bp + 32);
@@ -205,7 +226,7 @@ __device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t
     auto hi16 = [](uint32_t w) { return (float)__builtin_bit_cast(half2_t, w).y; };
     auto al = [](uint32_t hi, uint32_t lo) { return __builtin_amdgcn_alignbyte(hi, lo, 2); };
     qh = 0u, m = 0.f;
-    if (F == kFmtQ40) {
+    if (F == kFmtQ40 || F == kFmtIQ4NL) {
         if (half == 0) q[0] = al(a.y, a.x), q[1] = al(a.z, a.y), q[2] = al(a.w, a.z), q[3] = al(b.x, a.w), d = lo16(a.x);
         else q[0] = b.y, q[1] = b.z, q[2] = b.w, q[3] = c.x, d = hi16(b.x);
     } else if (F == kFmtQ41) {
@@ -223,8 +244,9 @@ __device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t
 template <int R, int F>
 __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
                                          int s, int lane, float (&acc)[R]) {
-    constexpr bool kFive = F == kFmtQ50 || F == kFmtQ51;
-    constexpr float kZero = F == kFmtQ40 ? -8.0f : (F == kFmtQ50 ? -16.0f : 0.0f);  // the quant that stands for zero
+    constexpr bool kFive = F == kFmtQ50 || F == kFmtQ51, kTable = F == kFmtIQ4NL;
+    // the quant that stands for zero (IQ4_NL: the staged sums already carry the 128 of the table)
+    constexpr float kZero = F == kFmtQ40 ? -8.0f : (F == kFmtQ50 ? -16.0f : (kTable ? -1.0f : 0.0f));
     const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // the sums of x over the two blocks (x 2^-24)
     float v[R];
 #pragma unroll
@@ -246,7 +268,10 @@ __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* _
             float alo = 0.f, ahi = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                if (kFive) {
+                if (kTable) {
+                    alo = iq4nl_dot4(iq4nl_lookup4(q[i] & 0x0F0F0F0Fu), xl[i], alo);
+                    ahi = iq4nl_dot4(iq4nl_lookup4((q[i] >> 4) & 0x0F0F0F0Fu), xh[i], ahi);
+                } else if (kFive) {
                     const uint32_t lo = (((qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u;
                     const uint32_t hi = (((qh >> (16 + 4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u;
                     q5k_dot_dword(q[i], lo | (hi << 1), xl[i], xh[i], alo, ahi);
@@ -329,7 +354,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40;
     using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
-    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
+    constexpr int kSmallBytes = (F == kFmtQ40 || F == kFmtIQ4NL) ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
+    constexpr bool kPlainX = F == kFmtIQ4NL;  // x staged unscaled, block sums times 128, results in true units
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
@@ -389,7 +415,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     if constexpr (STEPS > 0) {
         Loads L[STEPS][R];
         issue(0, 0, L[0]);
-        q4k_stage_store<J, true, kHi>(st, n4, tid, blockDim.x, xs, ss);
+        q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, blockDim.x, xs, ss);
         __syncthreads();
         // `tie` is always 0; an empty asm after each step makes it look rewritten from the finished accumulator,
         // which pins the loads of step s+1 between the arithmetic of steps s-1 and s (one step of lookahead) and
@@ -406,9 +432,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     } else {
         Loads bufa[R], bufb[R];
         issue(0, 0, bufa);
-        q4k_stage_store<J, true, kHi>(st, n4, tid, blockDim.x, xs, ss);
+        q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, blockDim.x, xs, ss);
         for (int f = tid + J * blockDim.x; f < n4; f += blockDim.x)
-            q4k_stage_store_one<true, kHi>(reinterpret_cast<const float4*>(x)[f], f, xs, ss);
+            q4k_stage_store_one<!kPlainX, kHi>(reinterpret_cast<const float4*>(x)[f], f, xs, ss);
         __syncthreads();
         for (int s = 0; s < steps; s += 2) {
             if (s + 1 < steps) issue(s + 1, 0, bufb);
@@ -421,7 +447,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     }
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const float total = wave_sum(acc[r]) * 16777216.0f;
+        const float total = wave_sum(acc[r]) * (kPlainX ? 1.0f : 16777216.0f);
         if (lane == 0 && row_ok[r]) y[row0 + r] = total;
     }
 }
@@ -829,7 +855,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, Q8 = F == kFmtQ80, kSmall = F >= kFmtQ40 && !Q6 && !Q8;
     using Loads = std::conditional_t<Q8, Q80Loads, std::conditional_t<Q6, Q6kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
-    constexpr int kSmallBytes = F == kFmtQ40 ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
+    constexpr int kSmallBytes = (F == kFmtQ40 || F == kFmtIQ4NL) ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
+    constexpr bool kPlainX = F == kFmtIQ4NL;  // x staged unscaled, block sums times 128, results in true units
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
     float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
@@ -939,7 +966,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
 #pragma unroll
         for (int jj = 0; jj < J; jj++) q6k_stage_store_one(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
     } else {
-        q4k_stage_store<J, true, kHi>(st, n4, tid, 512, xs, ss);
+        q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, 512, xs, ss);
     }
     __syncthreads();
     // (after the staging, while the first weights are still on their way)
@@ -964,7 +991,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
-    const float back = Q8 ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
+    const float back = (Q8 || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
     const float t0 = wave_sum(acc[0]) * back;
     const float t1 = wave_sum(acc[1]) * back;
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
@@ -1095,7 +1122,7 @@ int skn_matvec_init(skn_ctx* ctx) {
         allow_big_lds<4, 1, F>, allow_big_lds<0, 2, F>, allow_big_lds<1, 2, F>, allow_big_lds<2, 2, F>,         \
         allow_big_lds<3, 2, F>, allow_big_lds<4, 2, F>
                              SKN_ALLOW_FMT(kFmtQ5K), SKN_ALLOW_FMT(kFmtQ40), SKN_ALLOW_FMT(kFmtQ41),
-                             SKN_ALLOW_FMT(kFmtQ50), SKN_ALLOW_FMT(kFmtQ51)};
+                             SKN_ALLOW_FMT(kFmtQ50), SKN_ALLOW_FMT(kFmtQ51), SKN_ALLOW_FMT(kFmtIQ4NL)};
 #undef SKN_ALLOW_FMT
     for (auto f : fns) SKN_HIP(ctx, f());
     SKN_HIP(ctx, allow_big_lds_q6k<1>());
@@ -1119,6 +1146,7 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_ALLOW_FUSED(kFmtQ51);
     SKN_ALLOW_FUSED(kFmtQ6K);
     SKN_ALLOW_FUSED(kFmtQ80);
+    SKN_ALLOW_FUSED(kFmtIQ4NL);
 #undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
@@ -1126,7 +1154,7 @@ int skn_matvec_init(skn_ctx* ctx) {
 bool skn_matvec_fusable(int ggml_type) {
     return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
            ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
-           ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0;
+           ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_IQ4_NL;
 }
 
 // Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
@@ -1169,6 +1197,7 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         case SKN_TYPE_Q5_1: SKN_FUSED(kFmtQ51)
         case SKN_TYPE_Q6_K: SKN_FUSED(kFmtQ6K)
         case SKN_TYPE_Q8_0: SKN_FUSED(kFmtQ80)
+        case SKN_TYPE_IQ4_NL: SKN_FUSED(kFmtIQ4NL)
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED
@@ -1195,9 +1224,10 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
     // Q5_K on the lane map of the Q4_K kernel (16-byte aligned blocks, x within the LDS of a compute unit)
     if (ggml_type == SKN_TYPE_Q5_K && ((uintptr_t)w_dev & 15) == 0 && nb <= 144 && ctx->opt_matvec_stage == 1)
         return nb > 32 ? dispatch_q4k<1, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtQ5K>(ctx, w, n, nb, x_dev, y_dev, 8);
-    // Q4_0 / Q4_1 / Q5_0 / Q5_1 likewise, eight blocks standing for a superblock (rows of whole groups of eight are
+    // Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL likewise, eight blocks standing for a superblock (rows of whole groups of eight are
     // 16-byte aligned)
-    if ((ggml_type == SKN_TYPE_Q4_0 || ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1) &&
+    if ((ggml_type == SKN_TYPE_Q4_0 || ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
+         ggml_type == SKN_TYPE_IQ4_NL) &&
         k % 256 == 0 && ((uintptr_t)w_dev & 15) == 0 && k <= 144 * 256 && ctx->opt_matvec_stage == 1) {
         const int ng = k / 256;
 #define SKN_SMALL(F) (ng > 32 ? dispatch_q4k<1, F>(ctx, w, n, ng, x_dev, y_dev, 8) : dispatch_q4k<2, F>(ctx, w, n, ng, x_dev, y_dev, 8))
@@ -1205,6 +1235,7 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
             case SKN_TYPE_Q4_0: return SKN_SMALL(kFmtQ40);
             case SKN_TYPE_Q4_1: return SKN_SMALL(kFmtQ41);
             case SKN_TYPE_Q5_0: return SKN_SMALL(kFmtQ50);
+            case SKN_TYPE_IQ4_NL: return SKN_SMALL(kFmtIQ4NL);
             default: return SKN_SMALL(kFmtQ51);
         }
 #undef SKN_SMALL

@@ -261,7 +261,7 @@ def _decode_against_oracle(hip, cfg, w, n_steps, modes=(1, 0), tol=TOL):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (14, "q6_k"),
-                                        (8, "q8_0")])
+                                        (8, "q8_0"), (20, "iq4_nl")])
 @pytest.mark.parametrize("group", ["qkv", "o", "gu", "down"])
 def test_fused_groups_of_further_formats(hip, qtype, name, group):
     """The fused decode kernels take Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, Q6_K and Q8_0 as well: one group of matrices at a time in
@@ -292,7 +292,8 @@ def test_fused_groups_of_further_formats(hip, qtype, name, group):
     _decode_against_oracle(hip, cfg, w, 5)
 
 
-@pytest.mark.parametrize("qtype,name", [(12, "q4_k"), (13, "q5_k"), (2, "q4_0"), (6, "q5_0"), (14, "q6_k"), (8, "q8_0")])
+@pytest.mark.parametrize("qtype,name", [(12, "q4_k"), (13, "q5_k"), (2, "q4_0"), (6, "q5_0"), (14, "q6_k"), (8, "q8_0"),
+                                        (20, "iq4_nl")])
 @pytest.mark.parametrize("ffn", [8192, 11008, 14336])
 def test_fused_down_projection_of_two_to_four_steps(hip, qtype, name, ffn):
     """Rows of 8192, 11008 and 14336 weights take two, three and four unrolled steps of the fused kernel (4096

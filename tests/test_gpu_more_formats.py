@@ -60,7 +60,7 @@ def test_matvec_vs_oracle(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, want) <= TOL
 
 
-STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
+STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
 
 
 @pytest.mark.parametrize("qtype,name", STAGED)
@@ -85,7 +85,7 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
         assert np.abs(got[stage] - got[0]).max() <= 1e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1")])
+@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
@@ -97,9 +97,9 @@ def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
 
 
-@pytest.mark.parametrize("qtype,name,bb", [(2, "q4_0", 18), (3, "q4_1", 20), (6, "q5_0", 22), (7, "q5_1", 24)])
+@pytest.mark.parametrize("qtype,name,bb", [(2, "q4_0", 18), (3, "q4_1", 20), (6, "q5_0", 22), (7, "q5_1", 24), (20, "iq4_nl", 18)])
 def test_small_block_matvec_field_positions(hip, qtype, name, bb):
-    """Q4_0 / Q4_1 / Q5_0 / Q5_1 with one block of every pair zeroed, with only low or only high nibbles set and
+    """Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL with one block of every pair zeroed, with only low or only high nibbles set and
     (the five-bit formats) with only one half of the fifth bits set: the realigned first block, the aligned second
     one and every bit plane against the oracle on their own."""
     n, k = 8, 2048
@@ -162,6 +162,22 @@ def test_matvec_rows_not_16_byte_aligned(hip, qtype, name):
     xd, yd = hip.to_device(x), hip.alloc(4 * n)
     hip.matvec_q(qtype, buf.ptr + 4, n, k, xd, yd)
     assert oracle_np.rel_err(yd.download(np.float32, n), oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
+
+
+def test_iq4_nl_matvec_every_table_entry(hip):
+    """IQ4_NL blocks whose nibbles are all one index, for each of the sixteen: the lookup of the lane-map kernel
+    entry by entry (y = d * table[i] * sum(x))."""
+    n, k = 16, 1024
+    x = synth.activation_f32(k, seed=77)
+    raw = np.zeros((n, k // 32, 18), np.uint8)
+    raw[:, :, :2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    for i in range(16):
+        raw[i, :, 2:] = i | (i << 4)
+    got = hip.matvec_q_host(20, raw.reshape(n, -1), n, k, x)
+    want = oracle_c.matvec_q(20, raw.reshape(n, -1), n, k, x)
+    table = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
+    assert np.allclose(want, 0.5 * table * x.astype(np.float64).sum(), rtol=1e-5, atol=1e-4)
+    assert oracle_np.rel_err(got, want) <= TOL
 
 
 def test_dense_matvec_odd_row_length(hip):
