@@ -174,6 +174,10 @@ int skn_rmsnorm(skn_ctx* ctx, const float* x_dev, const float* w_dev, int rows, 
 int skn_rope(skn_ctx* ctx, float* x_dev, int rows, int n_head, int head_dim, int pos0, float base);
 /* out = silu(gate) * up elementwise. */
 int skn_swiglu(skn_ctx* ctx, const float* gate_dev, const float* up_dev, int64_t n, float* out_dev);
+/* out = max(x, 0) elementwise, the reference's Tensor.relu (core/.../impl/DoublesTensor.kt:389-390: `if (elem > 0)
+ * elem else 0.0`, so a NaN gives 0), which its ReLU module applies between Linear layers
+ * (core/.../nn/activations/relu.kt:7-12).  out may be x. */
+int skn_relu(skn_ctx* ctx, const float* x_dev, int64_t n, float* out_dev);
 /* y += x elementwise. */
 int skn_add_inplace(skn_ctx* ctx, float* y_dev, const float* x_dev, int64_t n);
 /* Index of the first maximum of x[0:n] -> *index_dev (int32 on the device); the reference's inline scan

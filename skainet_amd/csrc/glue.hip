@@ -47,6 +47,14 @@ __global__ void swiglu_kernel(const float* __restrict__ g, const float* __restri
     }
 }
 
+__global__ void relu_kernel(const float* __restrict__ x, float* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float v = x[i];
+        out[i] = v > 0.f ? v : 0.f;  // (a NaN becomes 0, as `if (elem > 0) elem else 0.0` makes it)
+    }
+}
+
 __global__ void add_kernel(float* __restrict__ y, const float* __restrict__ x, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] += x[i];
@@ -141,6 +149,16 @@ int skn_swiglu(skn_ctx* ctx, const float* gate_dev, const float* up_dev, int64_t
     if (n == 0) return SKN_OK;
     SKN_REQUIRE(ctx, gate_dev && up_dev && out_dev, SKN_ERR_ARG, "skn_swiglu: null pointer");
     skn_launch(ctx, swiglu_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, gate_dev, up_dev, out_dev, n);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+int skn_relu(skn_ctx* ctx, const float* x_dev, int64_t n, float* out_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_relu: ctx is null");
+    SKN_REQUIRE(ctx, n >= 0, SKN_ERR_ARG, "skn_relu: negative size");
+    if (n == 0) return SKN_OK;
+    SKN_REQUIRE(ctx, x_dev && out_dev, SKN_ERR_ARG, "skn_relu: null pointer");
+    skn_launch(ctx, relu_kernel, dim3(blocks_for(n, 256)), dim3(256), 0, x_dev, out_dev, n);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }

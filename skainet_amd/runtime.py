@@ -92,6 +92,7 @@ _SIGNATURES = {
     "skn_rmsnorm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p]),
     "skn_rope": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
     "skn_swiglu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
+    "skn_relu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
     "skn_add_inplace": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]),
     "skn_argmax": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]),
     "skn_f32_to_f16": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]),
@@ -283,6 +284,9 @@ class Context:
     def sync(self):
         self._check(self.lib.skn_sync(self.handle))
 
+    def memset(self, dev, byte_value, nbytes):
+        self._check(self.lib.skn_memset(self.handle, _ptr(dev), int(byte_value), nbytes))
+
     def copy(self, dst_dev, src_dev, nbytes):
         self._check(self.lib.skn_copy(self.handle, _ptr(dst_dev), _ptr(src_dev), nbytes))
 
@@ -333,6 +337,9 @@ class Context:
 
     def swiglu(self, gate_dev, up_dev, n, out_dev):
         self._check(self.lib.skn_swiglu(self.handle, _ptr(gate_dev), _ptr(up_dev), n, _ptr(out_dev)))
+
+    def relu(self, x_dev, n, out_dev):
+        self._check(self.lib.skn_relu(self.handle, _ptr(x_dev), n, _ptr(out_dev)))
 
     def add_inplace(self, y_dev, x_dev, n):
         self._check(self.lib.skn_add_inplace(self.handle, _ptr(y_dev), _ptr(x_dev), n))

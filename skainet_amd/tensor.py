@@ -7,6 +7,8 @@
                    (core/.../nn/Linear.kt:26-28); t() is a view flag, never a copy (the reference's t()
                    materialises a transpose on every forward, core/.../impl/DoublesTensor.kt:362-387)
   QuantizedLinear  Module.forward for y = x . W^T (+ bias)   (core/.../nn/Module.kt:12, nn/Linear.kt:43-49)
+  ReLU, MLP        the activation module (core/.../nn/activations/relu.kt:7-12) and the sequential container
+                   (core/.../nn/topology/MLP.kt:8-19: forward feeds each module's output to the next)
 
 Error behaviour follows the reference: misaligned inner dimensions raise ValueError("Shapes do not align.")
 (core/.../impl/DoublesTensor.kt:256,268); operand ranks the reference's matmul does not know raise
@@ -129,6 +131,12 @@ class DeviceTensor:
         self.ctx.gemm_q(other.ggml_type, other.buf, n_out, n_in, a16, m, c.buf)
         return c
 
+    def relu(self):
+        """max(x, 0) elementwise (core/.../impl/DoublesTensor.kt:389-390)."""
+        out = DeviceTensor.empty(self.ctx, self.shape)
+        self.ctx.relu(self.buf, self.shape.volume, out.buf)
+        return out
+
     def __add__(self, other):
         if not isinstance(other, DeviceTensor):
             raise TypeError("device tensors add device tensors")
@@ -151,5 +159,29 @@ class QuantizedLinear:
     def forward(self, x: DeviceTensor) -> DeviceTensor:
         y = x.matmul(self.weight.t())
         return y + self.bias if self.bias is not None else y
+
+    __call__ = forward
+
+
+class ReLU:
+    def __init__(self, name="ReLU"):
+        self.name = name
+
+    def forward(self, x: DeviceTensor) -> DeviceTensor:
+        return x.relu()
+
+    __call__ = forward
+
+
+class MLP:
+    """Sequential composition: forward(x) = m_n(... m_2(m_1(x)))."""
+
+    def __init__(self, *modules, name="FeedForwardNetwork"):
+        self.name, self.modules = name, list(modules)
+
+    def forward(self, x: DeviceTensor) -> DeviceTensor:
+        for m in self.modules:
+            x = m.forward(x)
+        return x
 
     __call__ = forward

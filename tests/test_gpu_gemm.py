@@ -186,6 +186,20 @@ def test_gemm_benchmark_shapes_q6k(hip, n):
     assert err <= TOL, err
 
 
+def test_gemm_benchmark_shape_q4k_n14336(hip):
+    """M=512, K=4096, N=14336 with Q4_K weights: the wide cell of the mixed Q4_K/Q6_K prefill case, sampled columns."""
+    m, n, k = 512, 14336, 4096
+    raw = synth.weight(Q4_K, n, k, seed=13)
+    a = synth.activation_bf16((m, k), seed=14)
+    got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    rows = np.arange(0, n, 127)
+    rb = raw.reshape(n, -1)[rows].reshape(-1)
+    want = oracle_c.gemm_q(Q4_K, rb, len(rows), k, a, m)
+    floor = 1e-3 * np.abs(got).max()
+    err = np.max(np.abs(got[:, rows] - want) / np.maximum(np.abs(want), floor))
+    assert err <= TOL, err
+
+
 def test_gemm_full_width_slice(hip):
     """The benchmark shape M=512, K=4096 at N=4096: checked on a strided sample of the oracle's columns."""
     m, n, k = 512, 4096, 4096

@@ -2,6 +2,7 @@
 loaded to the device end to end.  The known answers are the reference's own TensorTest matmul cases, carried
 through Q8_0 weights that represent them exactly."""
 import json
+import math
 import os
 
 import numpy as np
@@ -9,7 +10,7 @@ import pytest
 
 from oracle import oracle_c, oracle_np
 from skainet_amd import gguf, synth
-from skainet_amd.tensor import DeviceTensor, QuantizedLinear, QuantizedTensor, Shape
+from skainet_amd.tensor import MLP, DeviceTensor, QuantizedLinear, QuantizedTensor, ReLU, Shape
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +52,55 @@ def test_reference_matmul_known_answers_through_quantized_weights(hip, golden_di
     ap[:, :3] = a
     got = DeviceTensor.from_numpy(hip, ap).matmul(w.t())
     assert got.shape == Shape(2, 2) and got.numpy().reshape(-1).tolist() == c["expected"]
+
+
+def test_reference_1x16_times_16x16_through_the_matvec(hip, golden_dir):
+    """TensorTest.kt:72-391: the 1x16 row times the 16x16 matrix, expected row within 1e-4 -- as Linear computes it,
+    x.matmul(W.t()) with W = B^T held as dense F32 rows on the device."""
+    c = json.load(open(os.path.join(golden_dir, "tensor_test_vectors.json")))["cases"]["matmul 1x16  16x16"]
+    a, b, want = (np.array(t["values"], dtype=np.float64).reshape(t["shape"]) for t in c["tensors"])
+    assert a.shape == (1, 16) and b.shape == (16, 16) and want.shape == (1, 16)
+    wt = np.ascontiguousarray(b.T, dtype=np.float32)  # [out, in]
+    w = QuantizedTensor.from_bytes(hip, synth.F32, 16, 16, wt.view(np.uint8))
+    y = DeviceTensor.from_numpy(hip, a[0]).matmul(w.t())
+    assert y.shape == Shape(16)
+    assert np.max(np.abs(y.numpy().astype(np.float64) - want[0])) < 1e-4
+
+
+def test_sine_mlp_end_to_end_on_the_device(hip, golden_dir):
+    """CsvParametersLoaderTest.kt:33-72: the 1-16-16-1 sine approximator (three Linear layers with bias, ReLU after
+    the first two) loaded from the reference's own parameter file, |mlp(pi/2) - sin(pi/2)| < 0.01 -- every layer a
+    QuantizedLinear over dense F32 rows on the device, the ReLUs device kernels, composed by the MLP container."""
+    with open(os.path.join(golden_dir, "sinus-approximator.json")) as f:
+        params = {e["unique_parameter_name"]: np.array(e["tensor"]["values"], dtype=np.float32).reshape(e["tensor"]["shape"])
+                  for e in json.load(f)}
+    assert len(params) == 6
+    mods = []
+    for i, last in ((1, False), (3, False), (5, True)):
+        w, b = params[f"linear-{i}.weight"], params[f"linear-{i}.bias"]
+        n_out, n_in = w.shape
+        qt = QuantizedTensor.from_bytes(hip, synth.F32, n_out, n_in, np.ascontiguousarray(w).view(np.uint8))
+        mods.append(QuantizedLinear(qt, DeviceTensor.from_numpy(hip, b), name=f"linear-{i}"))
+        if not last:
+            mods.append(ReLU())
+    net = MLP(*mods)
+    for angle in (math.pi / 2.0, 0.3, 1.0):
+        x = DeviceTensor.from_numpy(hip, np.array([angle]))
+        y = net(x).numpy()
+        # the same stack on the oracle (fp64): the device result follows it to fp32 rounding
+        r = np.array([angle])
+        for i, last in ((1, False), (3, False), (5, True)):
+            r = oracle_np.linear(r, params[f"linear-{i}.weight"].astype(np.float64), params[f"linear-{i}.bias"].astype(np.float64))
+            if not last:
+                r = np.maximum(r, 0.0)
+        assert y.shape == (1,) and abs(float(y[0]) - float(r[0])) < 1e-5
+    assert abs(float(net(DeviceTensor.from_numpy(hip, np.array([math.pi / 2.0]))).numpy()[0]) - 1.0) < 0.01
+
+
+def test_relu_follows_the_reference(hip):
+    x = np.array([-1.5, 0.0, -0.0, 2.25, np.nan, np.inf, -np.inf, 1e-38], dtype=np.float32)
+    got = DeviceTensor.from_numpy(hip, x).relu().numpy()
+    assert got.tolist() == [0.0, 0.0, 0.0, 2.25, 0.0, np.inf, 0.0, float(np.float32(1e-38))]
 
 
 def test_shape_errors_follow_the_reference(hip):
