@@ -159,6 +159,14 @@ int skn_kv_gather(skn_ctx* ctx, skn_kv* kv, int seq, int t0, int t1, uint16_t* k
  * q/out fp32 [n_seq][n_head][head_dim] on the device; n_ctx_host[s] = tokens to attend (NULL = all cached). */
 int skn_attn_decode(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* n_ctx_host, float scale,
                     float* out_dev);
+/* skn_attn_decode over all cached tokens of every sequence, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The split partials and split counters live in a fixed array inside the library's device image (4 MiB + 16 KiB per
+ * GPU, held until the process ends) instead of hipMalloc'd scratch; the call allocates and frees nothing.
+ * Limits: n_seq * n_head <= 4096, and n_seq * n_head * splits * (head_dim + 2) * 4 bytes <= 4 MiB -- SKN_ERR_SHAPE
+ * beyond them.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two contexts, two
+ * streams) race; serialise them. */
+int skn_attn_decode_static(skn_ctx* ctx, skn_kv* kv, const float* q_dev, float scale, float* out_dev);
 /* The same attention for the last n_queries tokens of one sequence at once (prompt processing), causal:
  * out[t,h,:] = softmax(q[t,h,:] . K[0:m_t,h,:]^T * scale) . V[0:m_t,h,:] with m_t = len - n_queries + t + 1.
  * q/out fp32 [n_queries][n_head][head_dim] on the device, 16-byte aligned; head_dim 64 or 128.  No reference

@@ -64,6 +64,7 @@ int skn_init(int device, skn_ctx** out) {
     ctx->stream = ctx->own_stream;
     int rc = skn_matvec_init(ctx);
     if (rc == SKN_OK) rc = skn_gemm_init(ctx);
+    if (rc == SKN_OK) rc = skn_attn_init(ctx);
     if (rc != SKN_OK) {
         g_ctxless_error = ctx->err;
         skn_shutdown(ctx);

@@ -292,6 +292,63 @@ int skn_attn_alloc_counters(skn_ctx* ctx, int n_pairs, int** out) {
     return SKN_OK;
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------------------
+// Split partials and split counters of skn_attn_decode_static live in one file-scope device array instead of
+// memory from hipMalloc.  `attn_static_scratch` below is the host-side stand-in of that array: only the address
+// hipGetSymbolAddress returns for it (kept per device in g_static_scratch) is ever handed to a kernel.
+namespace {
+constexpr int kStaticPairs = 4096;                                   // (sequence, head) pairs: one counter each
+constexpr size_t kStaticPartialBytes = (size_t)4 << 20;              // partials: pairs * splits * (head_dim + 2) floats
+constexpr size_t kStaticCounterBytes = (size_t)kStaticPairs * sizeof(int);
+constexpr int kMaxDevices = 64;
+__device__ __align__(256) unsigned char attn_static_scratch[kStaticPartialBytes + kStaticCounterBytes];
+unsigned char* g_static_scratch[kMaxDevices] = {};  // device address of the array, per device
+
+__global__ void attn_clear_counters_kernel(int* counters, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counters[i] = 0;
+}
+}  // namespace
+
+// Called by skn_init with the context's device current.
+int skn_attn_init(skn_ctx* ctx) {
+    SKN_REQUIRE(ctx, ctx->device >= 0 && ctx->device < kMaxDevices, SKN_ERR_ARG, "device index %d is beyond %d", ctx->device,
+                kMaxDevices);
+    if (!g_static_scratch[ctx->device]) {
+        void* p = nullptr;
+        SKN_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(attn_static_scratch)));
+        SKN_REQUIRE(ctx, p != nullptr, SKN_ERR_HIP, "hipGetSymbolAddress returned no address for the attention scratch");
+        g_static_scratch[ctx->device] = static_cast<unsigned char*>(p);
+    }
+    return SKN_OK;
+}
+
+extern "C" int skn_attn_decode_static(skn_ctx* ctx, skn_kv* kv, const float* q_dev, float scale, float* out_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_attn_decode_static: ctx is null");
+    SKN_REQUIRE(ctx, kv != nullptr, SKN_ERR_ARG, "skn_attn_decode_static: kv is null");
+    SKN_REQUIRE(ctx, q_dev && out_dev, SKN_ERR_ARG, "skn_attn_decode_static: null pointer");
+    unsigned char* base = g_static_scratch[ctx->device];
+    SKN_REQUIRE(ctx, base != nullptr, SKN_ERR_STATE, "skn_attn_decode_static: the scratch array has no address on device %d",
+                ctx->device);
+    const int pairs = kv->n_seq * kv->n_head;
+    SKN_REQUIRE(ctx, pairs <= kStaticPairs, SKN_ERR_SHAPE,
+                "skn_attn_decode_static: %d (sequence, head) pairs exceed the static scratch (at most %d)", pairs, kStaticPairs);
+    int max_ctx = 0;
+    for (int s = 0; s < kv->n_seq; s++)
+        if (kv->len[s] > max_ctx) max_ctx = kv->len[s];
+    const int n_splits = skn_attn_splits(ctx, pairs, max_ctx);
+    const size_t need = (size_t)pairs * n_splits * (kv->head_dim + 2) * sizeof(float);
+    SKN_REQUIRE(ctx, n_splits == 1 || need <= kStaticPartialBytes, SKN_ERR_SHAPE,
+                "skn_attn_decode_static: %d pairs x %d splits x head_dim %d need %zu bytes of partials (at most %zu)", pairs,
+                n_splits, kv->head_dim, need, kStaticPartialBytes);
+    float* partial = reinterpret_cast<float*>(base);
+    int* counters = reinterpret_cast<int*>(base + kStaticPartialBytes);
+    // the array keeps what the last call left (a call that was cut short may have left counts): start from zero
+    skn_launch(ctx, attn_clear_counters_kernel, dim3((pairs + 255) / 256), dim3(256), 0, counters, pairs);
+    SKN_LAUNCH_CHECK(ctx);
+    return skn_attn_launch_ex(ctx, kv, q_dev, kv->len_dev, kv->n_seq, -1, n_splits, partial, counters, scale, out_dev);
+}
+
 int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
                     float* out_dev) {
     const int D = kv->head_dim;

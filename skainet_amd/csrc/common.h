@@ -45,6 +45,7 @@ struct skn_ctx {
 // One-time kernel attribute setup (large dynamic LDS), called by skn_init.
 int skn_matvec_init(skn_ctx* ctx);
 int skn_gemm_init(skn_ctx* ctx);
+int skn_attn_init(skn_ctx* ctx);
 
 // Fused Q4_K matvec used by the decoder: up to three [rows_i, k] matrices stacked along the output axis,
 // optional RMSNorm of x (norm_w != nullptr) and a store / add-into / SwiGLU epilogue.

@@ -88,6 +88,7 @@ _SIGNATURES = {
     "skn_kv_append_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]),
     "skn_kv_gather": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "skn_attn_decode": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_float, C.c_void_p]),
+    "skn_attn_decode_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p]),
     "skn_attn_prefill": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_float, C.c_void_p]),
     "skn_rmsnorm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_void_p]),
     "skn_rope": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]),
@@ -220,6 +221,10 @@ class KVCache:
         if n_ctx is not None and len(n_ctx) != self.n_seq:
             raise ValueError("n_ctx needs one entry per sequence")
         self.ctx._check(self.ctx.lib.skn_attn_decode(self.ctx.handle, self.handle, _ptr(q_dev), arr, scale, _ptr(out_dev)))
+
+    def attn_decode_static(self, q_dev, out_dev, scale):
+        """skn_attn_decode over all cached tokens with the library's static scratch (allocates nothing)."""
+        self.ctx._check(self.ctx.lib.skn_attn_decode_static(self.ctx.handle, self.handle, _ptr(q_dev), scale, _ptr(out_dev)))
 
     def attn_prefill(self, seq, q_dev, n_queries, out_dev, scale):
         """Causal attention of the last n_queries tokens of sequence seq (q/out fp32 [n_queries][n_head][head_dim])."""
