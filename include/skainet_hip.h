@@ -100,7 +100,8 @@ int skn_sync(skn_ctx* ctx);
 int skn_set_stream(skn_ctx* ctx, void* hip_stream);
 /* Launch-shape tuning knobs, 0 = library default: "q4k.waves" (wavefronts per workgroup of the Q4_K matvec),
  * "q4k.rows" (rows per wavefront: 1, 2 or 4), "attn.splits" (context splits of decode attention),
- * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel),
+ * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel; a captured
+ * step is dropped and captured again after any change of an option or of the stream),
  * "llama.fused" (1 = fused per-layer kernels in the decode step, the default: for every group of matrices whose
  * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
@@ -108,6 +109,10 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * formats with 4-byte-multiple blocks; 2 = staged rows for all of those; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
+/* Counters of a context, for tests and reports: "launches" (kernel launches issued or recorded into a graph so far),
+ * "graph.captures" (decode-step graphs captured so far), "profiler.attached" (1 when a rocprofiler tool library is
+ * loaded into the process: "llama.graph" is then 0 and cannot be set, every decode step is launched kernel by kernel). */
+int skn_get_stat(skn_ctx* ctx, const char* key, int64_t* value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
 int skn_timer_start(skn_ctx* ctx);
 int skn_timer_stop(skn_ctx* ctx, float* elapsed_ms);
@@ -245,6 +250,18 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
 int skn_llama_decode(skn_ctx* ctx, skn_llama* m, int32_t first_token, int n_steps, int32_t* tokens_out_host);
 /* Device pointer to the fp32 [vocab] logits of the last processed token. */
 int skn_llama_logits(skn_ctx* ctx, skn_llama* m, const float** logits_dev);
+
+/* ---- test hook (not part of the surface a binding needs) ------------------------------------------------ */
+
+/* One launch of the fused matvec the decoder uses, so that tests can hold each fused form against the CPU oracle as an
+ * operation of its own: up to three [rows_i, k] matrices of one type stacked along the output, optional RMSNorm of x
+ * (norm_w_dev, eps), and an epilogue: 0 store y, 1 y +=, 2 y[i] = silu(w0 row i . x) * (w1 row i . x), 3 rotary
+ * embedding of q (rows0, to y as fp32) and k (rows1) with k and v (rows2) stored as fp16 at the end of sequence 0 of the
+ * one-sequence cache `kv` (its position is written to *pos_dev, a device int the caller provides).  No reference
+ * counterpart.  Types: Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0; k a multiple of 256, at most 16384. */
+int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const void* w0, int rows0, const void* w1, int rows1,
+                          const void* w2, int rows2, int k, const float* x_dev, const float* norm_w_dev, float eps,
+                          float* y_dev, skn_kv* kv, int32_t* pos_dev, float rope_base);
 
 #ifdef __cplusplus
 }

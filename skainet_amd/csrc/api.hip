@@ -62,6 +62,15 @@ int skn_init(int device, skn_ctx** out) {
         return rc;
     }
     ctx->stream = ctx->own_stream;
+    {
+        // rocprofv3 announces its tool library in ROCP_TOOL_LIBRARIES and preloads librocprofiler-sdk-tool; replaying a
+        // captured graph under its kernel trace has ended in a fault, so with a profiler attached every decode step
+        // is launched kernel by kernel
+        const char* tool = getenv("ROCP_TOOL_LIBRARIES");
+        const char* pre = getenv("LD_PRELOAD");
+        ctx->profiler_attached = (tool && *tool) || (pre && strstr(pre, "rocprofiler"));
+        if (ctx->profiler_attached) ctx->opt_llama_graph = 0;
+    }
     int rc = skn_matvec_init(ctx);
     if (rc == SKN_OK) rc = skn_gemm_init(ctx);
     if (rc == SKN_OK) rc = skn_attn_init(ctx);
@@ -254,6 +263,7 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream) {
     SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_set_stream: ctx is null");
     SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
     ctx->stream = hip_stream ? (hipStream_t)hip_stream : ctx->own_stream;
+    ctx->opt_generation++;  // graphs captured on the other stream are not replayed on this one
     return SKN_OK;
 }
 
@@ -263,11 +273,26 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     if (!strcmp(key, "q4k.waves")) ctx->opt_q4k_waves = value;
     else if (!strcmp(key, "q4k.rows")) ctx->opt_q4k_rows = value;
     else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
-    else if (!strcmp(key, "llama.graph")) ctx->opt_llama_graph = value;
+    else if (!strcmp(key, "llama.graph")) {
+        SKN_REQUIRE(ctx, !(value && ctx->profiler_attached), SKN_ERR_STATE,
+                    "skn_set_option: llama.graph stays 0 while a rocprofiler tool library is attached to the process");
+        ctx->opt_llama_graph = value;
+    }
     else if (!strcmp(key, "llama.fused")) ctx->opt_llama_fused = value;
     else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
     else if (!strcmp(key, "matvec.stage")) ctx->opt_matvec_stage = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
+    ctx->opt_generation++;  // whatever was captured with the old settings is stale
+    return SKN_OK;
+}
+
+int skn_get_stat(skn_ctx* ctx, const char* key, int64_t* value) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_get_stat: ctx is null");
+    SKN_REQUIRE(ctx, key && value, SKN_ERR_ARG, "skn_get_stat: null pointer");
+    if (!strcmp(key, "launches")) *value = ctx->stat_launches;
+    else if (!strcmp(key, "graph.captures")) *value = ctx->stat_captures;
+    else if (!strcmp(key, "profiler.attached")) *value = ctx->profiler_attached ? 1 : 0;
+    else return skn_fail(ctx, SKN_ERR_ARG, "skn_get_stat: unknown counter '%s'", key);
     return SKN_OK;
 }
 

@@ -29,6 +29,9 @@ struct skn_ctx {
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
     int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1;
+    int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
+    bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
+    long long stat_launches = 0, stat_captures = 0;  // kernel launches issued (or recorded) / decode-step graphs captured
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
@@ -63,7 +66,7 @@ struct skn_rope_epilogue {
     uint16_t* k_pool = nullptr;
     uint16_t* v_pool = nullptr;
     int n_head = 0, head_dim = 0, page_tokens = 0;
-    float log2_base = 0.f;
+    double log2_base = 0.0;  // log2 of the rotary base, in double: the angle pos * base^(-2i/d) is formed in double
 };
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
                          float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr, int ggml_type = SKN_TYPE_Q4_K);
@@ -94,6 +97,7 @@ int skn_fail(skn_ctx* ctx, int code, const char* fmt, ...);
 // profiler reports it, without launch gaps).
 template <typename F, typename... Args>
 inline void skn_launch(skn_ctx* ctx, F kernel, dim3 grid, dim3 block, size_t lds, Args... args) {
+    ctx->stat_launches++;
     if (ctx->prof_on && 2 * ctx->prof_used + 1 < ctx->prof_events.size()) {
         hipEvent_t e0 = ctx->prof_events[2 * ctx->prof_used], e1 = ctx->prof_events[2 * ctx->prof_used + 1];
         ctx->prof_used++;
@@ -153,6 +157,16 @@ constexpr int kWave = 64;
 
 __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
     return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+// sin and cos of the rotary angle pos * base^(-e / head_dim) for the element pair (e, e + 1).  The angle is formed and
+// reduced modulo 2 pi in double: in fp32 its rounding alone is pos * 2^-24 radians, which at a few hundred positions
+// already shows in the small outputs of a rotated pair.
+__device__ __forceinline__ void skn_rope_sincos(int pos, int e, int head_dim, double log2_base, float* sn, float* cs) {
+    const double theta = (double)pos * exp2(-(double)e / (double)head_dim * log2_base);
+    const double turns = rint(theta * 0.15915494309189535);  // 1 / (2 pi)
+    const float r = (float)fma(-turns, 6.283185307179586, theta);
+    sincosf(r, sn, cs);
 }
 
 // Sum over the 64 lanes of a wavefront; every lane returns the total.

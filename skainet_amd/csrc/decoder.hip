@@ -30,6 +30,7 @@ struct skn_llama {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     int graph_splits = 0;
+    int graph_generation = -1;  // ctx->opt_generation at capture: every option decode_step reads, and the stream
     std::vector<void*> owned;
 };
 
@@ -100,12 +101,11 @@ __global__ __launch_bounds__(1024) void embed_rows_kernel(const uint8_t* __restr
 __global__ void rope_store_kernel(float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                   uint16_t* __restrict__ k_pool, uint16_t* __restrict__ v_pool,
                                   const int32_t* __restrict__ table, const int32_t* __restrict__ pos0_dev, int n_head,
-                                  int kv_heads, int head_dim, int page_tokens, float log2_base) {
+                                  int kv_heads, int head_dim, int page_tokens, double log2_base) {
     const int row = blockIdx.x, h = blockIdx.y, i = threadIdx.x;
     const int pos = pos0_dev[0] + row;
-    const float inv_freq = exp2f(-2.0f * (float)i / (float)head_dim * log2_base);
     float sn, cs;
-    sincosf((float)pos * inv_freq, &sn, &cs);
+    skn_rope_sincos(pos, 2 * i, head_dim, log2_base, &sn, &cs);
     const size_t qbase = ((size_t)row * n_head + h) * head_dim + 2 * i;
     const float qa = q[qbase], qb = q[qbase + 1];
     q[qbase] = qa * cs - qb * sn;
@@ -182,8 +182,12 @@ __global__ void f32_to_bf16_rows_kernel(const float* __restrict__ x, uint16_t* _
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         uint32_t u = __float_as_uint(x[i]);
-        u += 0x7FFFu + ((u >> 16) & 1u);
-        out[i] = (uint16_t)(u >> 16);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) {  // NaN stays NaN (quiet), whatever its payload
+            out[i] = (uint16_t)((u >> 16) | 0x40u);
+        } else {
+            u += 0x7FFFu + ((u >> 16) & 1u);
+            out[i] = (uint16_t)(u >> 16);
+        }
     }
 }
 
@@ -314,7 +318,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.n_head = KVH;  // (heads of the cache)
             rope.head_dim = D;
             rope.page_tokens = kv->page_tokens;
-            rope.log2_base = log2f(c.rope_base);
+            rope.log2_base = log2((double)c.rope_base);
             const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
             const uint8_t* mats[3] = {(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv};
             bool done[3] = {false, false, false};
@@ -334,7 +338,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             SKN_TRY(skn_matvec_q(ctx, L.type_v, L.wv, KVD, H, m->xn, m->v));
             skn_launch(ctx, rope_store_kernel, dim3(1, NH), dim3(D / 2), 0, m->q, (const float*)m->k, (const float*)m->v,
                        kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, KVH, D,
-                       kv->page_tokens, log2f(c.rope_base));
+                       kv->page_tokens, log2((double)c.rope_base));
             SKN_LAUNCH_CHECK(ctx);
         }
         SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
@@ -382,13 +386,35 @@ void drop_graph(skn_llama* m) {
     m->graph_exec = nullptr;
     m->graph = nullptr;
     m->graph_splits = 0;
+    m->graph_generation = -1;
+}
+
+// frees a buffer of the model now (the stream must be idle) and forgets it
+template <typename T>
+void dev_release(skn_llama* m, T** p) {
+    if (!*p) return;
+    for (size_t i = 0; i < m->owned.size(); i++)
+        if (m->owned[i] == (void*)*p) {
+            m->owned.erase(m->owned.begin() + i);
+            break;
+        }
+    (void)hipFree((void*)*p);
+    *p = nullptr;
 }
 
 int ensure_prompt_buffers(skn_ctx* ctx, skn_llama* m, int T) {
     if (T <= m->prompt_cap) return SKN_OK;
     const skn_llama_config& c = m->cfg;
     const size_t H = c.hidden, F = c.ffn;
-    // earlier, smaller prompt buffers stay owned by the model until it is freed
+    // the buffers of a shorter prompt are released first (nothing on the stream may still read them)
+    if (m->prompt_cap > 0) {
+        SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        dev_release(m, &m->px); dev_release(m, &m->pxn); dev_release(m, &m->pq); dev_release(m, &m->pk);
+        dev_release(m, &m->pv); dev_release(m, &m->patt); dev_release(m, &m->pproj); dev_release(m, &m->pgate);
+        dev_release(m, &m->pup); dev_release(m, &m->pmid); dev_release(m, &m->pb16); dev_release(m, &m->ptok);
+        dev_release(m, &m->pnctx); dev_release(m, &m->ppartial); dev_release(m, &m->pcounters);
+        m->prompt_cap = 0;
+    }
     SKN_TRY(dev_alloc(ctx, m, &m->px, T * H));
     SKN_TRY(dev_alloc(ctx, m, &m->pxn, T * H));
     SKN_TRY(dev_alloc(ctx, m, &m->pq, T * H));
@@ -557,7 +583,7 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         }
         skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
                    kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, KVH, D,
-                   kv->page_tokens, log2f(c.rope_base));
+                   kv->page_tokens, log2((double)c.rope_base));
         SKN_LAUNCH_CHECK(ctx);
         // query row t attends to the first pos0 + t + 1 tokens of the (single) sequence
         if (D <= 128)
@@ -635,13 +661,14 @@ int skn_llama_decode(skn_ctx* ctx, skn_llama* m, int32_t first_token, int n_step
     for (skn_kv* kv : m->kv) SKN_TRY(skn_kv_reserve(ctx, kv, 0, m->pos + n_steps));
     skn_launch(ctx, set_state_kernel, dim3(1), dim3(64), 0, m->state, (int)first_token, m->pos);
     SKN_LAUNCH_CHECK(ctx);
-    // a fixed split count that suits the longest context of this run (the kernel derives its ranges from the
-    // actual length, so one captured step serves every position)
-    const int n_splits = skn_attn_splits(ctx, c.n_head, m->pos + n_steps);
+    // a fixed split count that suits the longest context the cache can hold (the kernel derives its ranges from the
+    // actual length, so one captured step serves every position of every run)
+    const int n_splits = skn_attn_splits(ctx, c.n_head, c.max_tokens);
     if (ctx->opt_llama_graph == 0) {
         for (int i = 0; i < n_steps; i++) SKN_TRY(decode_step(ctx, m, n_splits));
     } else {
-        if (m->graph_exec && m->graph_splits != n_splits) drop_graph(m);
+        // a captured step has the kernel set of the options (and the stream) it was captured with baked in
+        if (m->graph_exec && (m->graph_splits != n_splits || m->graph_generation != ctx->opt_generation)) drop_graph(m);
         if (!m->graph_exec) {
             SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
             SKN_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
@@ -656,6 +683,8 @@ int skn_llama_decode(skn_ctx* ctx, skn_llama* m, int32_t first_token, int n_step
             m->graph = g;
             SKN_HIP(ctx, hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
             m->graph_splits = n_splits;
+            m->graph_generation = ctx->opt_generation;
+            ctx->stat_captures++;
         }
         for (int i = 0; i < n_steps; i++) SKN_HIP(ctx, hipGraphLaunch(m->graph_exec, ctx->stream));
     }

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 }
 
 // one thread per (row, head, pair)
-__global__ void rope_kernel(float* __restrict__ x, int rows, int n_head, int head_dim, int pos0, float log2_base) {
+__global__ void rope_kernel(float* __restrict__ x, int rows, int n_head, int head_dim, int pos0, double log2_base) {
     const int half = head_dim >> 1;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t total = (int64_t)rows * n_head * half;
@@ -28,10 +28,8 @@ __global__ void rope_kernel(float* __restrict__ x, int rows, int n_head, int hea
     const int i = (int)(idx % half);
     const int64_t rh = idx / half;
     const int row = (int)(rh / n_head);
-    const float inv_freq = exp2f(-2.0f * (float)i / (float)head_dim * log2_base);
-    const float theta = (float)(pos0 + row) * inv_freq;
     float sn, cs;
-    sincosf(theta, &sn, &cs);
+    skn_rope_sincos(pos0 + row, 2 * i, head_dim, log2_base, &sn, &cs);
     float* p = x + rh * head_dim + 2 * i;
     const float a = p[0], b = p[1];
     p[0] = a * cs - b * sn;
@@ -138,7 +136,7 @@ int skn_rope(skn_ctx* ctx, float* x_dev, int rows, int n_head, int head_dim, int
     SKN_REQUIRE(ctx, x_dev != nullptr, SKN_ERR_ARG, "skn_rope: null pointer");
     const int64_t total = (int64_t)rows * n_head * (head_dim / 2);
     skn_launch(ctx, rope_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, x_dev, rows, n_head,
-                       head_dim, pos0, log2f(base));
+                       head_dim, pos0, log2((double)base));
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }

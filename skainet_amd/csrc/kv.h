@@ -21,6 +21,10 @@ struct skn_kv {
 // Maps pages so that sequence `seq` can hold `new_len` tokens; uploads new table entries on the stream.
 int skn_kv_reserve(skn_ctx* ctx, skn_kv* kv, int seq, int new_len);
 
+// Counts n more tokens into a sequence whose rows were written by a kernel outside the cache code (pages reserved
+// by the caller): host mirror and device length.
+int skn_kv_advance_len(skn_ctx* ctx, skn_kv* kv, int seq, int n);
+
 // Attention over `kv` with per-sequence lengths taken from a device array; max_ctx bounds them (host knowledge).
 int skn_attn_launch(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int max_ctx, float scale,
                     float* out_dev);

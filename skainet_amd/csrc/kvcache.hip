@@ -106,6 +106,13 @@ int skn_kv_reserve(skn_ctx* ctx, skn_kv* kv, int seq, int new_len) {
     return SKN_OK;
 }
 
+int skn_kv_advance_len(skn_ctx* ctx, skn_kv* kv, int seq, int n) {
+    skn_launch(ctx, kv_set_len_kernel, dim3((kv->n_seq + 63) / 64), dim3(64), 0, kv->len_dev, seq, kv->n_seq, n, 1);
+    SKN_LAUNCH_CHECK(ctx);
+    kv->len[seq] += n;
+    return SKN_OK;
+}
+
 extern "C" {
 
 int skn_kv_create(skn_ctx* ctx, int n_seq, int n_head, int head_dim, int page_tokens, int max_tokens, skn_kv** out) {

@@ -5,7 +5,7 @@
 // The op is bound by the HBM read of the weight blocks (0.5625 / 1.0625 / 0.8203 bytes per weight for the first
 // three); x is read once per workgroup and y written once.  One wavefront owns one output row, so the only
 // cross-lane traffic is a single DPP reduction per row and rows never need atomics.
-#include "common.h"
+#include "kv.h"
 #include <type_traits>
 
 namespace {
@@ -799,8 +799,7 @@ __device__ __forceinline__ Q4kRopeCtx q4k_rope_prepare(const skn_q4k_segments& s
     c.e = row % rope.head_dim;
     c.slot = pos % rope.page_tokens;
     c.page = page;
-    const float inv_freq = exp2f(-(float)c.e / (float)rope.head_dim * rope.log2_base);
-    sincosf((float)pos * inv_freq, &c.sn, &c.cs);
+    skn_rope_sincos(pos, c.e, rope.head_dim, rope.log2_base, &c.sn, &c.cs);
     return c;
 }
 
@@ -1201,6 +1200,41 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED
+}
+
+// Test hook: one launch of the decoder's fused matvec, so that each fused form can be held against the oracle as an
+// operation of its own.  epi 3 (rotary + cache store) appends the token at the end of sequence 0 of a one-sequence
+// cache: q goes to y (fp32, rotated), k (rotated) and v into the cache as fp16.
+extern "C" int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const void* w0, int rows0, const void* w1, int rows1,
+                                     const void* w2, int rows2, int k, const float* x_dev, const float* norm_w_dev, float eps,
+                                     float* y_dev, skn_kv* kv, int32_t* pos_dev, float rope_base) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_test_fused_matvec: ctx is null");
+    SKN_REQUIRE(ctx, epi >= SKN_EPI_STORE && epi <= SKN_EPI_ROPE && x_dev && y_dev && w0, SKN_ERR_ARG,
+                "skn_test_fused_matvec: bad arguments");
+    SKN_REQUIRE(ctx, ((uintptr_t)x_dev & 15) == 0 && (!norm_w_dev || ((uintptr_t)norm_w_dev & 15) == 0), SKN_ERR_ARG,
+                "skn_test_fused_matvec: x and the norm weights must be 16-byte aligned");
+    skn_q4k_segments seg = {{(const uint8_t*)w0, (const uint8_t*)w1, (const uint8_t*)w2}, {rows0, rows1, rows2}};
+    const int n_out = epi == SKN_EPI_SWIGLU ? rows0 : rows0 + rows1 + rows2;
+    if (epi == SKN_EPI_SWIGLU) SKN_REQUIRE(ctx, w1 && rows1 == rows0 && rows2 == 0, SKN_ERR_SHAPE, "skn_test_fused_matvec: gate and up must pair up");
+    if (epi != SKN_EPI_ROPE) return skn_matvec_q4k_fused(ctx, seg, n_out, k, x_dev, norm_w_dev, eps, y_dev, epi, nullptr, ggml_type);
+    SKN_REQUIRE(ctx, kv && pos_dev && kv->n_seq == 1, SKN_ERR_ARG, "skn_test_fused_matvec: the rotary form needs a one-sequence cache");
+    const int pos = kv->len[0];
+    int rc = skn_kv_reserve(ctx, kv, 0, pos + 1);
+    if (rc != SKN_OK) return rc;
+    SKN_HIP(ctx, hipMemcpyAsync(pos_dev, &kv->len[0], sizeof(int32_t), hipMemcpyHostToDevice, ctx->stream));
+    SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));  // (the host mirror changes below)
+    skn_rope_epilogue rope;
+    rope.pos_dev = pos_dev;
+    rope.page_table = kv->page_table_dev;
+    rope.k_pool = kv->k_pool;
+    rope.v_pool = kv->v_pool;
+    rope.n_head = kv->n_head;
+    rope.head_dim = kv->head_dim;
+    rope.page_tokens = kv->page_tokens;
+    rope.log2_base = log2((double)rope_base);
+    rc = skn_matvec_q4k_fused(ctx, seg, n_out, k, x_dev, norm_w_dev, eps, y_dev, SKN_EPI_ROPE, &rope, ggml_type);
+    if (rc != SKN_OK) return rc;
+    return skn_kv_advance_len(ctx, kv, 0, 1);
 }
 
 extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev,

@@ -73,6 +73,9 @@ _SIGNATURES = {
     "skn_sync": (C.c_int, [C.c_void_p]),
     "skn_set_stream": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
+    "skn_test_fused_matvec": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                                        C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_float]),
+    "skn_get_stat": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64)]),
     "skn_timer_start": (C.c_int, [C.c_void_p]),
     "skn_timer_stop": (C.c_int, [C.c_void_p, C.POINTER(C.c_float)]),
     "skn_prof_start": (C.c_int, [C.c_void_p, C.c_int]),
@@ -314,6 +317,20 @@ class Context:
 
     def set_option(self, key, value):
         self._check(self.lib.skn_set_option(self.handle, key.encode(), int(value)))
+
+    def test_fused_matvec(self, ggml_type, epi, mats, k, x_dev, norm_w_dev, eps, y_dev, kv=None, pos_dev=None, rope_base=10000.0):
+        """mats: up to three (device buffer, rows) pairs."""
+        mats = list(mats) + [(None, 0)] * (3 - len(mats))
+        args = []
+        for buf, rows in mats:
+            args += [_ptr(buf), int(rows)]
+        self._check(self.lib.skn_test_fused_matvec(self.handle, ggml_type, epi, *args, k, _ptr(x_dev), _ptr(norm_w_dev), eps,
+                                                   _ptr(y_dev), kv.handle if kv is not None else None, _ptr(pos_dev), rope_base))
+
+    def stat(self, key):
+        v = C.c_int64()
+        self._check(self.lib.skn_get_stat(self.handle, key.encode(), C.byref(v)))
+        return v.value
 
     def prof_start(self, max_launches):
         self._check(self.lib.skn_prof_start(self.handle, max_launches))

@@ -230,6 +230,59 @@ def test_graph_replay_equals_eager(hip):
     model.free()
 
 
+def test_option_change_recaptures_the_step(hip):
+    """A captured decode step has its kernel set baked in: changing an option on a live model drops the graph, the
+    next step is captured with the new kernels (seen in the number of launches recorded) and computes the same."""
+    w = llama.random_weights(SMALL, seed=13)
+    model = llama.LlamaModel(hip, SMALL, weights=w)
+    first = model.prefill([3, 1, 4, 1, 5])
+    hip.set_option("llama.graph", 1)
+    hip.set_option("llama.fused", 1)
+    c0, l0 = hip.stat("graph.captures"), hip.stat("launches")
+    a = model.decode(first, 3)
+    c1, l1 = hip.stat("graph.captures"), hip.stat("launches")
+    assert c1 == c0 + 1
+    fused_nodes = l1 - l0 - 1  # (one launch sets the step's state, the rest were recorded into the graph)
+    b = model.decode(a[-1], 3)  # same options, other run length and position: the graph is replayed, nothing recorded
+    assert hip.stat("graph.captures") == c1 and hip.stat("launches") == l1 + 1
+    hip.set_option("llama.fused", 0)
+    c = model.decode(b[-1], 3)
+    c2, l2 = hip.stat("graph.captures"), hip.stat("launches")
+    assert c2 == c1 + 1
+    unfused_nodes = l2 - (l1 + 1) - 1
+    assert unfused_nodes > fused_nodes, (fused_nodes, unfused_nodes)
+    hip.set_option("llama.fused", 1)
+    # the same nine steps without graphs and fused: identical tokens wherever both paths are exact enough, so compare
+    # against the oracle instead of bit for bit
+    ora = OracleLlama(SMALL, w)
+    ora.prefill([3, 1, 4, 1, 5], bf16_gemm=True)
+    tok = first
+    for got in a + b + c:
+        want = ora.step(tok)
+        if _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
+            assert got == want
+        else:
+            break
+        tok = want
+    model.free()
+
+
+def test_longer_prompt_releases_the_shorter_prompt_buffers(hip):
+    """Prompt buffers grow with the longest prompt seen; the superseded ones are freed, not kept until the model is."""
+    w = llama.random_weights(SMALL, seed=15)
+    model = llama.LlamaModel(hip, SMALL, weights=w)
+    ora = OracleLlama(SMALL, w)
+    rng = np.random.default_rng(4)
+    for n in (3, 9, 40, 17):
+        prompt = rng.integers(0, SMALL.vocab, size=n).tolist()
+        model.reset()
+        ora = OracleLlama(SMALL, w)
+        model.prefill(prompt)
+        ora.prefill(prompt, bf16_gemm=True)
+        assert oracle_np.rel_err(model.logits(), ora.logits) <= 5e-3, n
+    model.free()
+
+
 def _scale_q6k(raw, factor):
     """Q6_K block bytes with every d (fp16 at byte 208 of the 210) multiplied by a power of two."""
     blocks = raw.reshape(-1, 210).copy()
