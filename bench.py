@@ -27,7 +27,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-from skainet_amd import runtime, synth  # noqa: E402
+from skainet_amd import runtime, synth, traffic  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -369,6 +369,7 @@ def main():
         except Exception as e:  # the decoder leg reports its own absence instead of failing the headline
             extra["decode_7b_q4_k"] = {"error": f"{type(e).__name__}: {e}"}
 
+    traffic_rec = traffic.load_current(os.path.join(ROOT, "profiles", "matvec_q4k_4096x11008_traffic.json"))
     out = {
         "metric": "Q4_K matvec effective HBM GB/s (% peak); decode tok/s, 7B-shape Q4_K",
         "value": round(head["wall_gbs"], 2),
@@ -396,8 +397,10 @@ def main():
             "unit": "GB/s",
             "frac": round(head["kernel_gbs"] / HBM_PEAK_GBS, 4),
             # HBM bytes of one launch from hardware counters (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, one run
-            # each, scaled by what the same counters read for a copy kernel of this size): 1.015 x algorithmic
-            "traffic": 25813511,
+            # each, scaled by what the same counters read for a copy kernel of this size), as recorded in
+            # profiles/ by skainet_amd/traffic.py -- null when that record was taken on other kernel sources
+            "traffic": traffic_rec["traffic_bytes"] if traffic_rec else None,
+            "traffic_record": "profiles/matvec_q4k_4096x11008_traffic.json" if traffic_rec else "none for these kernel sources",
             "kernel": "matvec_q4k_kernel",
             "kernel_us": round(head["kernel_us"], 3),
             "cache_hot_gbs": round(head["hot_kernel_gbs"], 2),

@@ -33,6 +33,23 @@ def test_binding_covers_the_header():
     runtime.load_library()  # resolves every bound symbol
 
 
+def test_kotlin_ffm_binding_names_every_entry_point():
+    """bindings/kotlin/jvm/SknLib.kt (source only: no JVM here) holds one downcall handle per declared function."""
+    src = open(os.path.join(ROOT, "bindings", "kotlin", "jvm", "SknLib.kt")).read()
+    assert sorted(re.findall(r'h\("(skn_[a-z0-9_]+)"', src)) == declared_symbols()
+    for kt in ("jvm/QuantizedTensor.kt", "jvm/DeviceTensor.kt"):
+        body = open(os.path.join(ROOT, "bindings", "kotlin", kt)).read()
+        assert "TODO(" not in body
+        # every member of the reference's Tensor interface (core/src/commonMain/kotlin/sk/ai/net/Tensor.kt:6-92)
+        for member in ("plus(other: Tensor)", "plus(other: Double)", "plus(other: Int)", "minus(other: Double)",
+                       "minus(other: Int)", "minus(other: Tensor)", "matmul(other: Tensor)", "fun t()", "fun relu()",
+                       "softmax(dim: Int)", "fun softmax()", "pow(tensor: Tensor)", "pow(scalar: Double)", "fun sin()",
+                       "fun cos()", "fun tan()", "fun asin()", "fun acos()", "fun atan()", "fun sinh()", "fun cosh()",
+                       "fun tanh()", "fun exp()", "fun log()", "fun sqrt()", "fun cbrt()", "fun sigmoid()", "fun ln()",
+                       "flatten(startDim: Int, endDim: Int)", "val shape", "val dataDescriptor"):
+            assert member in body, (kt, member)
+
+
 def test_format_table_matches_reference_constants():
     # reference gguf/src/commonMain/kotlin/sk/ai/net/gguf/Constants.kt:58-90 and Quants.kt:10-20
     assert runtime.type_block(runtime.Q8_0) == (32, 34)

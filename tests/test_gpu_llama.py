@@ -2,6 +2,8 @@
 
 Tolerance: logits within 2e-3 of max(|logit|, 1e-3 * max|logit|) -- the per-op bound (1e-3) compounds over the
 layers of the stack -- and identical greedy tokens wherever the oracle's top-2 logit margin exceeds that error."""
+import os
+
 import numpy as np
 import pytest
 
@@ -177,7 +179,8 @@ def test_model_from_gguf_file_equals_model_from_weights(hip, tmp_path):
 def test_full_7b_shape_matches_oracle(hip):
     """The benchmark's model shape (32 layers, hidden 4096, FFN 11008, 32 heads x 128, vocabulary 32000, Q4_K
     layers, Q6_K head) at full size: decode steps and a short prompt pass against the oracle.  Every layer points
-    at the same seeded weights so that the host holds one layer (the device holds 32 copies)."""
+    at the same seeded weights: host and device hold one layer, which all 32 layers read (the model with 32 distinct
+    layers is the golden test below)."""
     cfg = llama.Config(max_tokens=64, page_tokens=16)
     one = llama.random_weights(llama.Config(**{**cfg.__dict__, "n_layer": 1}), seed=11)
     w = dict(one)
@@ -204,6 +207,43 @@ def test_full_7b_shape_matches_oracle(hip):
     assert err <= 5e-3, err
     if _margin_ok(ora.logits, 5e-3 * np.abs(ora.logits).max()):
         assert got_next == want_next
+    model.free()
+
+
+def test_7b_shape_at_the_benchmark_length_matches_the_oracle_golden(hip, golden_dir):
+    """The decoder benchmark itself -- 32 distinct seeded layers, 512-token prompt, 128 decode steps -- against the
+    oracle's answer kept in tests/golden/cfg5_llama7b_512_128.npz (tests/golden/make_cfg5_golden.py wrote it: 40 minutes
+    of CPU).  The decode steps are teacher-forced with the oracle's tokens so that every step sees the oracle's context.
+
+    Tolerance, fixed before the first comparison: an operation is held to 1e-3; a layer writes the residual stream
+    twice, and errors of independent operations add in quadrature, so the logits of an n-layer stack are held to
+    1e-3 * sqrt(2 n) = 8e-3 for n = 32, in the usual metric |a - r| / max(|r|, 1e-3 max|r|)."""
+    path = os.path.join(golden_dir, "cfg5_llama7b_512_128.npz")
+    if not os.path.exists(path):
+        pytest.fail("tests/golden/cfg5_llama7b_512_128.npz is missing (python tests/golden/make_cfg5_golden.py)")
+    gold = np.load(path)
+    stride = int(gold["stride"])
+    cfg = llama.Config(max_tokens=1024)
+    tol = 1e-3 * np.sqrt(2 * cfg.n_layer)
+    model = llama.LlamaModel(hip, cfg, seed=int(gold["seed"]))  # 32 distinct layers: 3.75 GB of blocks on the device
+    assert len({model.bufs[f"l{l}.wq"].ptr for l in range(cfg.n_layer)}) == cfg.n_layer
+
+    def check(tag, got_token):
+        want, absmax = gold[f"{tag}_sample"].astype(np.float64), float(gold[f"{tag}_absmax"])
+        got = model.logits()[::stride].astype(np.float64)
+        err = float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1e-3 * absmax)))
+        assert err <= tol, (tag, err)
+        if float(gold[f"{tag}_margin"]) > 2 * tol * absmax:
+            assert got_token == int(gold[f"{tag}_argmax"]), tag
+        return err
+
+    errs = {"prefill": check("prefill", model.prefill(gold["prompt"].tolist()))}
+    fed = [int(gold["first"])] + gold["tokens"].tolist()  # fed[i] goes into decode step i, fed[i + 1] is its greedy token
+    for i in range(128):
+        tok = model.decode(fed[i], 1)[0]
+        if f"step{i}_sample" in gold.files:
+            errs[f"step{i}"] = check(f"step{i}", tok)
+    print("logit errors:", {k: f"{v:.2e}" for k, v in errs.items()})
     model.free()
 
 
