@@ -74,7 +74,11 @@ __device__ __forceinline__ void store_tile_scaled(const float16_t& acc, float* _
 // nibble masked in place is the fp16 subnormal q * 2^-24 (or 16 q * 2^-24 for a high nibble) and one packed
 // fp16 multiply by sc_j * 2^10 (or sc_j * 2^6) gives sc_j * q * 2^-14 exactly -- an fp16 operand the matrix
 // core takes as is.  One set of accumulators: see the kernel.
-constexpr int kWPitch = 576;  // LDS pitch of a weight row: the 144 bytes of four superblocks
+// LDS pitch of a weight row: the 576 bytes of four superblocks plus one sixteen-byte pad piece.  With 576 (144 dwords,
+// 16 mod 64) rows r, r + 4, r + 8, ... start in the same bank and the 128-bit reads of a wavefront's 32 rows were
+// eight-fold bank conflicts; with 592 (148 dwords, 20 mod 64) sixteen consecutive rows tile all 64 banks.
+constexpr int kWPieces = 37;
+constexpr int kWPitch = kWPieces * 16;
 
 // Activations bf16 [m, k] -> fragment order.  One workgroup per R rows of the padded row count (rows >= m are
 // zero), one wavefront per row: the row's largest magnitude fixes its power-of-two scale, then the row is
@@ -227,6 +231,137 @@ __global__ __launch_bounds__(64 * R) void prep_a_frag_kernel(const skn_gemm_src 
     }
 }
 
+// The same preparation with a row spread over two wavefronts (k <= 16384): every element is read from memory once and
+// stays in registers through the three steps that the one-wavefront-per-row kernel above makes three passes for (sum of
+// squares, largest magnitude, conversion), two rows per workgroup, twice as many workgroups.  Thread t of a row takes
+// tasks t, t + 128, ... (task = chunk c, nibble dword dw: four elements at 64 c + 4 dw and four at 64 c + 32 + 4 dw);
+// its sixteen-byte pieces go straight to their place in the fragment order.  Consecutive row pairs go to workgroups of
+// one XCD (blockIdx % 8), so that the 128-byte lines they share are completed in one L2.
+template <int NT, int SRC, bool SUMS>
+__global__ __launch_bounds__(256) void prep_a_rows_kernel(const skn_gemm_src src, _Float16* __restrict__ afrag,
+                                                         float* __restrict__ inv_scale, _Float16* __restrict__ sfrag,
+                                                         int m, int k) {
+    __shared__ float red_ss[2][2], red_mx[2][2];
+    const int tid = threadIdx.x, t = tid & 127, rw = tid >> 7, wv = (tid >> 6) & 1;
+    const int n_pairs = gridDim.x, per_xcd = n_pairs >> 3;
+    const int pair = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    const int row = 2 * pair + rw;
+    const bool real = row < m;
+    const size_t row_off = (size_t)(real ? row : 0) * k;
+    const int tasks = k >> 3, nch = k >> 6, nb = k >> 8;
+    const float* xf = (const float*)src.a + row_off;
+    const uint16_t* xb = (const uint16_t*)src.a + row_off;
+    float v[NT][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const int task = min(t + 128 * j, tasks - 1), c = task >> 3, dw = task & 7;
+        const int e0 = 64 * c + 4 * dw;
+        if (SRC == SKN_SRC_BF16) {
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(xb + e0), hi = *reinterpret_cast<const u32x2*>(xb + e0 + 32);
+            v[j][0] = __uint_as_float(lo.x << 16), v[j][1] = __uint_as_float(lo.x & 0xFFFF0000u);
+            v[j][2] = __uint_as_float(lo.y << 16), v[j][3] = __uint_as_float(lo.y & 0xFFFF0000u);
+            v[j][4] = __uint_as_float(hi.x << 16), v[j][5] = __uint_as_float(hi.x & 0xFFFF0000u);
+            v[j][6] = __uint_as_float(hi.y << 16), v[j][7] = __uint_as_float(hi.y & 0xFFFF0000u);
+        } else {
+            const float4 lo = *reinterpret_cast<const float4*>(xf + e0), hi = *reinterpret_cast<const float4*>(xf + e0 + 32);
+            v[j][0] = lo.x, v[j][1] = lo.y, v[j][2] = lo.z, v[j][3] = lo.w;
+            v[j][4] = hi.x, v[j][5] = hi.y, v[j][6] = hi.z, v[j][7] = hi.w;
+            if (SRC == SKN_SRC_RMSNORM && t + 128 * j < tasks)
+                ss += ((lo.x * lo.x + lo.y * lo.y) + (lo.z * lo.z + lo.w * lo.w)) + ((hi.x * hi.x + hi.y * hi.y) + (hi.z * hi.z + hi.w * hi.w));
+        }
+    }
+    float r = 1.f;
+    if (SRC == SKN_SRC_RMSNORM) {
+        ss = wave_sum(ss);
+        if ((tid & 63) == 0) red_ss[rw][wv] = ss;
+        __syncthreads();
+        r = 1.0f / sqrtf((red_ss[rw][0] + red_ss[rw][1]) / (float)k + src.eps);
+    }
+    // the bf16 values the GEMM is defined on (fp32 sources: rounded to nearest even here), and their largest magnitude
+    float mx = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        if (SRC != SKN_SRC_BF16) {
+            const int task = min(t + 128 * j, tasks - 1), c = task >> 3, dw = task & 7;
+            float4 glo = make_float4(1.f, 1.f, 1.f, 1.f), ghi = glo;
+            if (SRC == SKN_SRC_RMSNORM) {
+                glo = *reinterpret_cast<const float4*>((const float*)src.b + 64 * c + 4 * dw);
+                ghi = *reinterpret_cast<const float4*>((const float*)src.b + 64 * c + 32 + 4 * dw);
+            }
+            const float g[8] = {glo.x, glo.y, glo.z, glo.w, ghi.x, ghi.y, ghi.z, ghi.w};
+#pragma unroll
+            for (int x = 0; x < 8; x++) {
+                const float y = SRC == SKN_SRC_RMSNORM ? v[j][x] * r * g[x] : v[j][x];
+                v[j][x] = __uint_as_float(bf16_rne(y) << 16);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+            const float f = fabsf(v[j][x]);
+            if (f == f && f < INFINITY) mx = fmaxf(mx, f);
+        }
+    }
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) red_mx[rw][wv] = mx;
+    __syncthreads();
+    mx = real ? fmaxf(red_mx[rw][0], red_mx[rw][1]) : 0.f;
+    int e = 9;  // a zero row keeps scale 1
+    if (mx > 0.f) e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+    e = max(e, -100);
+    const float scale = real ? __uint_as_float((uint32_t)(127 + 9 - e) << 23) : 0.f;
+    if (t == 0 && real) inv_scale[row] = __uint_as_float((uint32_t)(127 - 9 + e) << 23);
+    const int mb = row >> 5, rr = row & 31;
+    u32x4* out = reinterpret_cast<u32x4*>(afrag) + (size_t)mb * nch * 256 + rr;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const int task = t + 128 * j, c = task >> 3, dw = task & 7;
+        _Float16 l[4], u[4];
+#pragma unroll
+        for (int x = 0; x < 4; x++) l[x] = (_Float16)(v[j][x] * scale), u[x] = (_Float16)(v[j][4 + x] * scale);
+        float sl = ((float)l[0] + (float)l[1]) + ((float)l[2] + (float)l[3]);
+        float su = ((float)u[0] + (float)u[1]) + ((float)u[2] + (float)u[3]);
+        if (SUMS) {  // totals over the eight lanes of the chunk
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0xB1, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0xB1, 0xF, 0xF, true));
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x4E, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x4E, 0xF, 0xF, true));
+            sl += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sl), 0x141, 0xF, 0xF, true));
+            su += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(su), 0x141, 0xF, 0xF, true));
+        }
+        if (task < tasks) {
+            half8_t o;
+            o[0] = l[0], o[1] = l[2], o[2] = u[0], o[3] = u[2], o[4] = l[1], o[5] = l[3], o[6] = u[1], o[7] = u[3];
+            const int h = dw >> 2, sq = dw & 3;
+            out[((size_t)c * 4 + sq) * 64 + h * 32] = __builtin_bit_cast(u32x4, o);
+            if (SUMS && dw == 0) {
+                _Float16 h0, h1, l0, l1;
+                skn_split_hilo(sl * 0x1p-12f, h0, l0);
+                skn_split_hilo(su * 0x1p-12f, h1, l1);
+                _Float16* sf = sfrag + ((size_t)mb * nb + (c >> 2)) * 512 + 2 * (c & 3);
+                half2_t vh = {h0, h1}, vl = {l0, l1};
+                *reinterpret_cast<half2_t*>(sf + rr * 8) = vh;
+                *reinterpret_cast<half2_t*>(sf + (32 + rr) * 8) = vl;
+            }
+        }
+    }
+}
+
+template <int SRC, bool SUMS>
+void launch_prep(skn_ctx* ctx, const skn_gemm_src& src, _Float16* afrag, float* isc, _Float16* sfrag, int m, int m_pad, int k) {
+    // (m_pad is a multiple of 32: the pair count divides by the eight XCDs its workgroups are dealt to)
+    if (k <= 16384 && m_pad % 16 == 0) {
+        const dim3 grid(m_pad / 2), block(256);
+        const int nt = (k / 8 + 127) / 128;
+        if (nt <= 4) skn_launch(ctx, prep_a_rows_kernel<4, SRC, SUMS>, grid, block, 0, src, afrag, isc, sfrag, m, k);
+        else if (nt <= 8) skn_launch(ctx, prep_a_rows_kernel<8, SRC, SUMS>, grid, block, 0, src, afrag, isc, sfrag, m, k);
+        else if (nt <= 12) skn_launch(ctx, prep_a_rows_kernel<12, SRC, SUMS>, grid, block, 0, src, afrag, isc, sfrag, m, k);
+        else skn_launch(ctx, prep_a_rows_kernel<16, SRC, SUMS>, grid, block, 0, src, afrag, isc, sfrag, m, k);
+    } else {
+        skn_launch(ctx, prep_a_frag_kernel<4, SRC, SUMS>, dim3(m_pad / 4), dim3(256), 0, src, afrag, isc, sfrag, m, k);
+    }
+}
+
 // up to three weight matrices [n_i, k] multiplied by the same activations in one launch
 struct Q4kFragSegs {
     const uint8_t* w[3];
@@ -277,15 +412,15 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     const int mb0 = (MH * mt + mh) * MT, n0 = pair ? tn * 32 : (tn - segs.tile0[seg]) * kBN;
 
     // Weight staging, global memory straight into LDS: a wavefront-wide load fills 64 sixteen-byte slots
-    // i * 64 + lane; slot P holds piece P % 36 of tile row P / 36 (36 pieces = the 576 bytes of four
-    // superblocks).  The 36 loads of a group are dealt round the eight wavefronts.  Completion is waited for
+    // i * 64 + lane; slot P holds piece P % 37 of tile row P / 37 (36 pieces = the 576 bytes of four
+    // superblocks, the 37th a pad that repeats the last).  The 37 loads of a group are dealt round the wavefronts.  Completion is waited for
     // with the vector-memory counter before the barrier that publishes the buffer.
     auto wfetch = [&](int g, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int x = 0; x < (36 + 4 * MH - 1) / (4 * MH); x++) {
+        for (int x = 0; x < (kWPieces + 4 * MH - 1) / (4 * MH); x++) {
             const int i = wave + 4 * MH * x;
-            if (i < 36) {
-                const int p = i * 64 + lane, row = p / 36, col = p - 36 * row;
+            if (i < kWPieces) {
+                const int p = i * 64 + lane, row = p / kWPieces, col = min(p - kWPieces * row, 35);
                 const int off = min(g * 576 + col * 16, nb * 144 - 16);  // (a short last group repeats the row's last piece)
                 const uint8_t* wsrc = pair && row >= 32 ? segs.w[1] : w;  // (pair: tile rows 32.. are the up matrix)
                 const uint8_t* src = wsrc + (size_t)min(n0 + (pair ? row & 31 : row), n - 1) * nb * 144 + off;
@@ -439,7 +574,10 @@ void gemm_q4k_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                     }
                     // refill the slot: eight steps ahead in this superblock, or the first half of superblock sb + 4
                     // (past the end: a repeat of the last superblock, unused)
+                    // (the refill stays here: moved further down by the scheduler, the ring would be shallower than it looks)
+                    __builtin_amdgcn_sched_barrier(0);
                     afetch(step < 8 ? 16 * sb + step + 8 : 16 * min(sb + 4, nb - 1) + step - 8, slot);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             };
             chunk(std::integral_constant<int, 0>{});
@@ -748,11 +886,10 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     _Float16* afrag = (_Float16*)ws;
     _Float16* sfrag = (_Float16*)(ws + af_bytes);
     float* isc = (float*)(ws + af_bytes + sf_bytes);
-    const dim3 pgrid(m_pad / 4), pblock(256);
     switch (src.kind) {
-        case SKN_SRC_BF16: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
-        case SKN_SRC_F32: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_F32, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
-        case SKN_SRC_RMSNORM: skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_RMSNORM, true>, pgrid, pblock, 0, src, afrag, isc, sfrag, m, k); break;
+        case SKN_SRC_BF16: launch_prep<SKN_SRC_BF16, true>(ctx, src, afrag, isc, sfrag, m, m_pad, k); break;
+        case SKN_SRC_F32: launch_prep<SKN_SRC_F32, true>(ctx, src, afrag, isc, sfrag, m, m_pad, k); break;
+        case SKN_SRC_RMSNORM: launch_prep<SKN_SRC_RMSNORM, true>(ctx, src, afrag, isc, sfrag, m, m_pad, k); break;
         default: return skn_fail(ctx, SKN_ERR_ARG, "Q4_K GEMM: unknown activation source %d", src.kind);
     }
     SKN_LAUNCH_CHECK(ctx);
@@ -797,7 +934,7 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     uint8_t* bfrag = ws + af_bytes + is_bytes;
     const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
     _Float16* no_sums = nullptr;
-    skn_launch(ctx, prep_a_frag_kernel<4, SKN_SRC_BF16, false>, dim3(m_pad / 4), dim3(256), 0, src, afrag, isc, no_sums, m, k);
+    launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k);
     SKN_LAUNCH_CHECK(ctx);
     rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;

@@ -12,6 +12,7 @@ struct skn_kv {
     int32_t* page_table_dev = nullptr;  // [n_seq][pages_per_seq], -1 = not mapped
     int32_t* len_dev = nullptr;         // [n_seq] tokens held, the kernels' source of append positions
     int32_t* nctx_dev = nullptr;        // [n_seq] staging for explicit attention lengths
+    int* ticket_dev = nullptr;          // workgroups of an append launch count themselves in (zero between launches)
     std::vector<int32_t> page_table;    // host mirror
     std::vector<int32_t> len;           // host mirror
     std::vector<int32_t> free_pages;    // stack of unmapped page ids

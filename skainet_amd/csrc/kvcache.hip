@@ -18,7 +18,7 @@ struct AppendArgs {
 
 // grid (n_entries, n_head); one 16-byte chunk per thread, head_dim / 8 chunks per row.
 __global__ void kv_append_kernel(uint16_t* __restrict__ k_pool, uint16_t* __restrict__ v_pool,
-                                 const int32_t* __restrict__ table, const int32_t* __restrict__ len,
+                                 const int32_t* __restrict__ table, int32_t* len, int* ticket,
                                  const uint16_t* __restrict__ k_in, const uint16_t* __restrict__ v_in, AppendArgs a,
                                  int n_head, int head_dim, int page_tokens, int pages_per_seq) {
     const int i = blockIdx.x, h = blockIdx.y;
@@ -33,11 +33,15 @@ __global__ void kv_append_kernel(uint16_t* __restrict__ k_pool, uint16_t* __rest
         reinterpret_cast<uint4*>(k_pool + dst)[c] = reinterpret_cast<const uint4*>(k_in + src)[c];
         reinterpret_cast<uint4*>(v_pool + dst)[c] = reinterpret_cast<const uint4*>(v_in + src)[c];
     }
-}
-
-__global__ void kv_advance_kernel(int32_t* len, AppendArgs a, int n) {
-    if (threadIdx.x == 0 && blockIdx.x == 0) {
-        for (int i = 0; i < n; i++) len[a.seq[i]] += 1;
+    // The lengths advance once every workgroup of the launch has read them: each takes a ticket after its read (the
+    // read's value has been used above, so it has completed), and the holder of the last ticket counts the new tokens
+    // in and returns the ticket counter to zero for the next launch.
+    if (threadIdx.x == 0) {
+        const int total = gridDim.x * gridDim.y;
+        if (__hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total - 1) {
+            for (int e = 0; e < (int)gridDim.x; e++) len[a.seq[e]] += 1;
+            __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -139,6 +143,7 @@ int skn_kv_create(skn_ctx* ctx, int n_seq, int n_head, int head_dim, int page_to
     if (e == hipSuccess) e = hipMalloc((void**)&kv->page_table_dev, table_bytes);
     if (e == hipSuccess) e = hipMalloc((void**)&kv->len_dev, (size_t)n_seq * sizeof(int32_t));
     if (e == hipSuccess) e = hipMalloc((void**)&kv->nctx_dev, (size_t)n_seq * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&kv->ticket_dev, 16);
     if (e != hipSuccess) {
         (void)hipGetLastError();
         int rc = skn_fail(ctx, SKN_ERR_OOM, "skn_kv_create: %zu-byte pools: %s", pool_bytes, hipGetErrorString(e));
@@ -152,6 +157,7 @@ int skn_kv_create(skn_ctx* ctx, int n_seq, int n_head, int head_dim, int page_to
     int rc = skn_memset(ctx, kv->page_table_dev, 0xFF, table_bytes);
     if (rc == SKN_OK) rc = skn_memset(ctx, kv->len_dev, 0, (size_t)n_seq * sizeof(int32_t));
     if (rc == SKN_OK) rc = skn_memset(ctx, kv->nctx_dev, 0, (size_t)n_seq * sizeof(int32_t));
+    if (rc == SKN_OK) rc = skn_memset(ctx, kv->ticket_dev, 0, 16);
     if (rc != SKN_OK) {
         skn_kv_free(ctx, kv);
         return rc;
@@ -169,6 +175,7 @@ int skn_kv_free(skn_ctx* ctx, skn_kv* kv) {
     if (kv->page_table_dev) (void)hipFree(kv->page_table_dev);
     if (kv->len_dev) (void)hipFree(kv->len_dev);
     if (kv->nctx_dev) (void)hipFree(kv->nctx_dev);
+    if (kv->ticket_dev) (void)hipFree(kv->ticket_dev);
     delete kv;
     return SKN_OK;
 }
@@ -227,10 +234,8 @@ int skn_kv_append(skn_ctx* ctx, skn_kv* kv, const uint16_t* k_dev, const uint16_
             a.seq[i] = seq_ids_host[base + i];
             a.rank[i] = seen[a.seq[i]]++;
         }
-        skn_launch(ctx, kv_append_kernel, dim3(cnt, kv->n_head), dim3(64), 0, kv->k_pool, kv->v_pool, kv->page_table_dev, kv->len_dev, k_dev + base * row,
-                           v_dev + base * row, a, kv->n_head, kv->head_dim, kv->page_tokens, kv->pages_per_seq);
-        SKN_LAUNCH_CHECK(ctx);
-        skn_launch(ctx, kv_advance_kernel, dim3(1), dim3(64), 0, kv->len_dev, a, cnt);
+        skn_launch(ctx, kv_append_kernel, dim3(cnt, kv->n_head), dim3(64), 0, kv->k_pool, kv->v_pool, kv->page_table_dev, kv->len_dev, kv->ticket_dev,
+                           k_dev + base * row, v_dev + base * row, a, kv->n_head, kv->head_dim, kv->page_tokens, kv->pages_per_seq);
         SKN_LAUNCH_CHECK(ctx);
         for (int i = 0; i < cnt; i++) kv->len[a.seq[i]]++;
     }
