@@ -67,6 +67,7 @@ struct skn_rope_epilogue {
     uint16_t* v_pool = nullptr;
     int n_head = 0, head_dim = 0, page_tokens = 0;
     double log2_base = 0.0;  // log2 of the rotary base, in double: the angle pos * base^(-2i/d) is formed in double
+    const double* inv_freq = nullptr;  // optional device table base^(-2i/d), i < head_dim / 2 (saves the exp2 per wavefront)
 };
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
                          float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr, int ggml_type = SKN_TYPE_Q4_K);
@@ -162,6 +163,13 @@ __device__ __forceinline__ float h2f_bits(uint32_t bits16) {
 // sin and cos of the rotary angle pos * base^(-e / head_dim) for the element pair (e, e + 1).  The angle is formed and
 // reduced modulo 2 pi in double: in fp32 its rounding alone is pos * 2^-24 radians, which at a few hundred positions
 // already shows in the small outputs of a rotated pair.
+__device__ __forceinline__ void skn_rope_sincos_freq(int pos, double inv_freq, float* sn, float* cs) {
+    const double theta = (double)pos * inv_freq;
+    const double turns = rint(theta * 0.15915494309189535);  // 1 / (2 pi)
+    const float r = (float)fma(-turns, 6.283185307179586, theta);
+    sincosf(r, sn, cs);
+}
+
 __device__ __forceinline__ void skn_rope_sincos(int pos, int e, int head_dim, double log2_base, float* sn, float* cs) {
     const double theta = (double)pos * exp2(-(double)e / (double)head_dim * log2_base);
     const double turns = rint(theta * 0.15915494309189535);  // 1 / (2 pi)

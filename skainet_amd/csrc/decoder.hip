@@ -8,6 +8,7 @@
 #include "kv.h"
 
 #include <algorithm>
+#include <cmath>
 
 struct skn_llama {
     skn_llama_config cfg;
@@ -20,6 +21,7 @@ struct skn_llama {
     int *attn_counters = nullptr, *pcounters = nullptr;  // split counters of the attention launches (zero between launches)
     int32_t* state = nullptr;       // [0] token, [1] position, [2] context length, [3] step index
     int32_t* tokens_out = nullptr;  // device array of produced tokens
+    double* inv_freq = nullptr;     // rope_base^(-2i / head_dim), i < head_dim / 2, formed in double on the host
     int tokens_cap = 0;
     int pos = 0;                    // host mirror of the position
     // prompt buffers (grown to the longest prompt seen)
@@ -321,6 +323,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.head_dim = D;
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2((double)c.rope_base);
+            rope.inv_freq = m->inv_freq;
             const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
             const uint8_t* mats[3] = {(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv};
             bool done[3] = {false, false, false};
@@ -508,6 +511,15 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
         rc = skn_fail(ctx, SKN_ERR_HIP, "skn_llama_create: clearing the attention counters failed");
     }
     A(&m->state, (size_t)4);
+    A(&m->inv_freq, (size_t)cfg->head_dim / 2);
+    if (rc == SKN_OK) {
+        std::vector<double> f(cfg->head_dim / 2);
+        for (int i = 0; i < cfg->head_dim / 2; i++) f[i] = pow((double)cfg->rope_base, -2.0 * i / cfg->head_dim);
+        if (hipMemcpy(m->inv_freq, f.data(), f.size() * sizeof(double), hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            rc = skn_fail(ctx, SKN_ERR_HIP, "skn_llama_create: uploading the rotary frequencies failed");
+        }
+    }
     m->tokens_cap = cfg->max_tokens;
     A(&m->tokens_out, (size_t)m->tokens_cap);
     if (rc != SKN_OK) {

@@ -789,8 +789,15 @@ struct Q4kRopeCtx {
     float sn = 0.f, cs = 1.f;
 };
 
+// element index (even) inside its head of the rotary pair that output unit `unit` holds
+__device__ __forceinline__ int q4k_rope_elem(const skn_q4k_segments& seg, const skn_rope_epilogue& rope, int unit) {
+    int row = unit * 2;
+    row -= row >= seg.rows[0] + seg.rows[1] ? seg.rows[0] + seg.rows[1] : row >= seg.rows[0] ? seg.rows[0] : 0;
+    return row % rope.head_dim;
+}
+
 __device__ __forceinline__ Q4kRopeCtx q4k_rope_prepare(const skn_q4k_segments& seg, const skn_rope_epilogue& rope,
-                                                     int unit, int pos, int page) {
+                                                     int unit, int pos, int page, double freq) {
     Q4kRopeCtx c;
     int row = unit * 2;  // rows 2u, 2u+1 of the stacked q | k | v output: one rotary pair (segment sizes are even)
     c.which = row >= seg.rows[0] + seg.rows[1] ? 2 : row >= seg.rows[0] ? 1 : 0;
@@ -799,7 +806,8 @@ __device__ __forceinline__ Q4kRopeCtx q4k_rope_prepare(const skn_q4k_segments& s
     c.e = row % rope.head_dim;
     c.slot = pos % rope.page_tokens;
     c.page = page;
-    skn_rope_sincos(pos, c.e, rope.head_dim, rope.log2_base, &c.sn, &c.cs);
+    if (rope.inv_freq) skn_rope_sincos_freq(pos, freq, &c.sn, &c.cs);
+    else skn_rope_sincos(pos, c.e, rope.head_dim, rope.log2_base, &c.sn, &c.cs);
     return c;
 }
 
@@ -868,7 +876,12 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     // rotary epilogue: the position and, once it is known, the page id of its cache row are requested here (two
     // dependent round trips) so that neither is waited for after the staging barrier
     int rope_pos = 0, rope_page = 0;
-    if (EPI == SKN_EPI_ROPE) rope_pos = rope.pos_dev[0];
+    double rope_freq = 0.0;  // (the pair's frequency out of the model's table, requested with the position)
+    if (EPI == SKN_EPI_ROPE) {
+        rope_pos = rope.pos_dev[0];
+        if (rope.inv_freq)
+            rope_freq = rope.inv_freq[q4k_rope_elem(seg, rope, min((int)(blockIdx.x * 8 + (threadIdx.x >> 6)), (n_out + 1) / 2 - 1)) >> 1];
+    }
     Q4kStage<J> st, nw;
     q4k_stage_load<J>(x, n4, tid, 512, st);
     if (NORM) q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
@@ -970,7 +983,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     __syncthreads();
     // (after the staging, while the first weights are still on their way)
     Q4kRopeCtx rc;
-    if (EPI == SKN_EPI_ROPE) rc = q4k_rope_prepare(seg, rope, min(unit, (n_out + 1) / 2 - 1), rope_pos, rope_page);
+    if (EPI == SKN_EPI_ROPE) rc = q4k_rope_prepare(seg, rope, min(unit, (n_out + 1) / 2 - 1), rope_pos, rope_page, rope_freq);
     float rinv = 1.0f;
     if (NORM) {
         const float total = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
