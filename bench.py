@@ -165,25 +165,40 @@ def bench_attention_prefill(ctx, reps=20):
             "frac_mfma_f16_peak": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
-def bench_gemm(ctx, qtype, m, n, k, reps=20):
+def bench_gemm(ctx, qtype, m, n, k, reps=20, expanded=False):
     """Prefill GEMM C[m,n] = A[m,k] . deq(W)[n,k]^T (A bf16): summed kernel time of one call (activation
-    preparation included), 2mnk flops against the dense fp16 matrix-core peak."""
+    preparation included), 2mnk flops against the dense fp16 matrix-core peak.  expanded: the weight pass of the
+    formats other than Q4_K done once beforehand (skn_gemm_expand, 4 bytes per weight kept on the device)."""
     w = ctx.to_device(synth.weight(qtype, n, k, seed=3))
     a = ctx.to_device(synth.activation_bf16((m, k), seed=4))
     c = ctx.alloc(4 * m * n)
+    kept = ctx.gemm_expand(qtype, w, n, k) if expanded else None
+
+    def call():
+        if expanded:
+            ctx.gemm_expanded(kept, n, k, a, m, c)
+        else:
+            ctx.gemm_q(qtype, w, n, k, a, m, c)
+
     for _ in range(3):
-        ctx.gemm_q(qtype, w, n, k, a, m, c)
+        call()
     ctx.sync()
     ctx.prof_start(8 * reps)
     for _ in range(reps):
-        ctx.gemm_q(qtype, w, n, k, a, m, c)
+        call()
     ms, launches = ctx.prof_stop()
-    for buf in (w, a, c):
+    for buf in (w, a, c) + ((kept,) if expanded else ()):
         buf.free()
     us = ms / reps * 1e3
     tflops = 2.0 * m * n * k / us / 1e6
     return {"us_per_gemm": round(us, 1), "launches_per_gemm": launches // reps, "tflops": round(tflops, 1),
             "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
+
+
+def gemm_expanded_rows(ctx):
+    """The Q6_K shapes of the GEMM leg with their expanded weights kept between calls."""
+    return {f"q6_k_expanded_{mm}x{nn}x{kk}": bench_gemm(ctx, Q6_K, mm, nn, kk, expanded=True)
+            for mm, nn, kk in ((512, 4096, 4096), (512, 14336, 4096))}
 
 
 def bench_dequant(ctx, qtype, n, k, reps=20):
@@ -333,7 +348,7 @@ def main():
         ctx.close()
         return
     if args.mode == "gemm":
-        print(json.dumps({"mode": "gemm", **{f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
+        print(json.dumps({"mode": "gemm", **gemm_expanded_rows(ctx), **{f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
                                              for nm, qt, mm, nn, kk in gemm_shapes}}))
         ctx.close()
         return
@@ -359,6 +374,7 @@ def main():
         extra["prompt_attention_512x32x128"] = bench_attention_prefill(ctx)
         extra["prefill_gemm"] = {f"{nm}_{mm}x{nn}x{kk}": bench_gemm(ctx, qt, mm, nn, kk)
                                  for nm, qt, mm, nn, kk in gemm_shapes}
+        extra["prefill_gemm"].update(gemm_expanded_rows(ctx))
         try:
             from skainet_amd import llama_bench
             extra["decode_7b_q4_k"] = llama_bench.run(ctx)
@@ -366,6 +382,12 @@ def main():
             mix = {f"l{i}.{m}": Q6_K for i in range(0, 32, 2) for m in ("wv", "w_down")}
             r = llama_bench.run(ctx, steps=64, matrix_types=mix)
             extra["decode_7b_q4_k_q6_k_mix"] = {key: r[key] for key in ("decode_tok_s", "ms_per_token", "prefill_ms", "weight_bytes_per_token")}
+            ctx.set_option("llama.expand_weights", 1)  # the Q6_K matrices keep their expanded copies: 4 GB more
+            try:
+                r = llama_bench.run(ctx, steps=8, matrix_types=mix)
+                extra["decode_7b_q4_k_q6_k_mix"]["prefill_ms_expanded_weights"] = r["prefill_ms"]
+            finally:
+                ctx.set_option("llama.expand_weights", 0)
         except Exception as e:  # the decoder leg reports its own absence instead of failing the headline
             extra["decode_7b_q4_k"] = {"error": f"{type(e).__name__}: {e}"}
 

@@ -57,6 +57,9 @@ object SknLib {
     val dequant: MethodHandle = h("skn_dequant", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_LONG, ADDRESS))
     val matvecQ: MethodHandle = h("skn_matvec_q", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS))
     val gemmQ: MethodHandle = h("skn_gemm_q", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS))
+    val gemmExpandedBytes: MethodHandle = h("skn_gemm_expanded_bytes", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, JAVA_INT, ADDRESS))
+    val gemmExpand: MethodHandle = h("skn_gemm_expand", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS))
+    val gemmExpanded: MethodHandle = h("skn_gemm_expanded", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS))
     val kvCreate: MethodHandle = h("skn_kv_create", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, JAVA_INT, JAVA_INT, JAVA_INT, ADDRESS))
     val kvFree: MethodHandle = h("skn_kv_free", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS))
     val kvReset: MethodHandle = h("skn_kv_reset", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT))

@@ -103,14 +103,17 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel; a captured
  * step is dropped and captured again after any change of an option or of the stream),
  * "llama.fused" (1 = fused per-layer kernels in the decode step, the default: for every group of matrices whose
- * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0), "gemm.tile" (0 = choose, 1 = 64-row tiles,
+ * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0), "llama.expand_weights" (1 = the prompt pass of a decoder keeps an expanded
+ * copy, see skn_gemm_expand, of every layer matrix that is not Q4_K, made at the first prompt: 4 bytes per weight of
+ * device memory on top of the blocks; 0 = the default, expand per call), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
  * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL, rows staged through LDS for the other
  * formats with 4-byte-multiple blocks; 2 = staged rows for all of those; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* Counters of a context, for tests and reports: "launches" (kernel launches issued or recorded into a graph so far),
- * "graph.captures" (decode-step graphs captured so far), "profiler.attached" (1 when a rocprofiler tool library is
+ * "graph.captures" (decode-step graphs captured so far), "llama.expanded_bytes" (device bytes that the
+ * decoders of this context hold in expanded weight copies, see "llama.expand_weights"), "profiler.attached" (1 when a rocprofiler tool library is
  * loaded into the process: "llama.graph" is then 0 and cannot be set, every decode step is launched kernel by kernel). */
 int skn_get_stat(skn_ctx* ctx, const char* key, int64_t* value);
 /* HIP-event stopwatch on the context's stream: start, enqueue work, stop -> elapsed milliseconds. */
@@ -139,6 +142,16 @@ int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, c
  * A bf16 bits [m,k] row-major, C fp32 [m,n] row-major. */
 int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const uint16_t* a_bf16_dev, int m,
                float* c_dev);
+/* The same product (core/.../impl/DoublesTensor.kt:267-279) with the weight pass of the formats other than Q4_K done
+ * once instead of per call.  For those formats skn_gemm_q first rewrites W as an fp16 pair per weight in matrix-core
+ * operand order (4 bytes per weight, rows padded to a multiple of 64); a caller that multiplies with the same W
+ * again and has the memory keeps that copy: skn_gemm_expanded_bytes gives its size, skn_gemm_expand fills a device
+ * buffer of that size (16-byte aligned) from the blocks, skn_gemm_expanded multiplies with it -- the results are
+ * those of skn_gemm_q bit for bit.  Any SKN_TYPE_* weight type; k a multiple of 64. */
+int skn_gemm_expanded_bytes(skn_ctx* ctx, int ggml_type, int n, int k, size_t* bytes_out);
+int skn_gemm_expand(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, void* expanded_dev);
+int skn_gemm_expanded(skn_ctx* ctx, const void* expanded_dev, int n, int k, const uint16_t* a_bf16_dev, int m,
+                      float* c_dev);
 
 /* ---- paged KV cache -------------------------------------------------------------------------------- */
 

@@ -279,6 +279,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
         ctx->opt_llama_graph = value;
     }
     else if (!strcmp(key, "llama.fused")) ctx->opt_llama_fused = value;
+    else if (!strcmp(key, "llama.expand_weights")) ctx->opt_llama_expand = value;
     else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
     else if (!strcmp(key, "matvec.stage")) ctx->opt_matvec_stage = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
@@ -291,6 +292,7 @@ int skn_get_stat(skn_ctx* ctx, const char* key, int64_t* value) {
     SKN_REQUIRE(ctx, key && value, SKN_ERR_ARG, "skn_get_stat: null pointer");
     if (!strcmp(key, "launches")) *value = ctx->stat_launches;
     else if (!strcmp(key, "graph.captures")) *value = ctx->stat_captures;
+    else if (!strcmp(key, "llama.expanded_bytes")) *value = ctx->stat_expanded_bytes;
     else if (!strcmp(key, "profiler.attached")) *value = ctx->profiler_attached ? 1 : 0;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_get_stat: unknown counter '%s'", key);
     return SKN_OK;

@@ -28,10 +28,11 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0;
     int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
     bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
     long long stat_launches = 0, stat_captures = 0;  // kernel launches issued (or recorded) / decode-step graphs captured
+    long long stat_expanded_bytes = 0;               // device bytes held by the decoders' expanded weight copies
     // scratch for split-context attention partials, grown on demand
     void* attn_scratch = nullptr;
     size_t attn_scratch_bytes = 0;
@@ -151,6 +152,10 @@ struct skn_gemm_seg {
 int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m,
                        bool swiglu_pair = false);
 int skn_weights_hilo_frag(skn_ctx* ctx, int ggml_type, const uint8_t* w, int n, int k, void* bfrag);
+// The general GEMM path with weights expanded beforehand (skn_gemm_expand): one activation pass, then one launch per
+// matrix; seg.w is the expanded copy (skn_gemm_expanded_size bytes).
+size_t skn_gemm_expanded_size(int n, int k);
+int skn_gemm_expanded_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m);
 
 // ---- device helpers --------------------------------------------------------------------------------
 

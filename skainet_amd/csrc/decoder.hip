@@ -35,6 +35,10 @@ struct skn_llama {
     hipGraphExec_t graph_exec = nullptr;
     int graph_splits = 0;
     int graph_generation = -1;  // ctx->opt_generation at capture: every option decode_step reads, and the stream
+    // fp16-pair copies of the matrices that are not Q4_K, for the prompt GEMMs (made on first use when the option
+    // llama.expand_weights is set): seven per layer in the order q, k, v, o, gate, up, down
+    std::vector<void*> expanded;
+    long long expanded_bytes = 0;
     std::vector<void*> owned;
 };
 
@@ -537,6 +541,7 @@ int skn_llama_free(skn_ctx* ctx, skn_llama* m) {
     drop_graph(m);
     for (skn_kv* kv : m->kv) skn_kv_free(ctx, kv);
     for (void* p : m->owned) (void)hipFree(p);
+    ctx->stat_expanded_bytes -= m->expanded_bytes;
     delete m;
     return SKN_OK;
 }
@@ -546,6 +551,26 @@ int skn_llama_reset(skn_ctx* ctx, skn_llama* m) {
     SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_ARG, "skn_llama_reset: model is null");
     for (skn_kv* kv : m->kv) SKN_TRY(skn_kv_reset(ctx, kv, 0));
     m->pos = 0;
+    return SKN_OK;
+}
+
+// the expanded copy of matrix `which` of layer l, made on first use
+static int expanded_copy(skn_ctx* ctx, skn_llama* m, int l, int which, int type, const void* w, int n, int k, const void** out) {
+    if (m->expanded.empty()) m->expanded.assign((size_t)m->cfg.n_layer * 7, nullptr);
+    void*& slot = m->expanded[(size_t)l * 7 + which];
+    if (!slot) {
+        uint8_t* p = nullptr;
+        SKN_TRY(dev_alloc(ctx, m, &p, skn_gemm_expanded_size(n, k)));
+        const int rc = skn_gemm_expand(ctx, type, w, n, k, p);
+        if (rc != SKN_OK) {
+            dev_release(m, &p);
+            return rc;
+        }
+        slot = p;
+        m->expanded_bytes += (long long)skn_gemm_expanded_size(n, k);
+        ctx->stat_expanded_bytes += (long long)skn_gemm_expanded_size(n, k);
+    }
+    *out = slot;
     return SKN_OK;
 }
 
@@ -583,10 +608,31 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
         const bool q4k_gu = H <= 16384 && L.type_gate == SKN_TYPE_Q4_K && L.type_up == SKN_TYPE_Q4_K;
         const bool q4k_down = F <= 16384 && L.type_down == SKN_TYPE_Q4_K;
         SKN_TRY(skn_kv_reserve(ctx, kv, 0, pos0 + T));
+        // other formats with the option llama.expand_weights: their fp16-pair copies are kept, and the general GEMM
+        // takes the fp32 rows as the Q4_K one does (norm and rounding inside its activation pass, residual in its store)
+        const bool expand = ctx->opt_llama_expand != 0 && H % 64 == 0 && F % 64 == 0;
         if (q4k_qkv) {  // RMSNorm inside the activation pass, one launch for the three projections
             const skn_gemm_seg qkv[3] = {{L.wq, H, m->pq, 0}, {L.wk, KVD, m->pk, 0}, {L.wv, KVD, m->pv, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.attn_norm, c.rms_eps};
             SKN_TRY(skn_gemm_q4k_multi(ctx, qkv, 3, H, src, T));
+        } else if (expand) {  // Q4_K matrices of the group on their own kernel, the others through their kept copies
+            const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
+            const void* blocks[3] = {L.wq, L.wk, L.wv};
+            float* outs[3] = {m->pq, m->pk, m->pv};
+            skn_gemm_seg q4[3], ex[3];
+            int n4 = 0, nx = 0;
+            for (int i = 0; i < 3; i++) {
+                if (types[i] == SKN_TYPE_Q4_K && H <= 16384) {
+                    q4[n4++] = {blocks[i], rows[i], outs[i], 0};
+                } else {
+                    ex[nx] = {nullptr, rows[i], outs[i], 0};
+                    SKN_TRY(expanded_copy(ctx, m, l, i, types[i], blocks[i], rows[i], H, &ex[nx].w));
+                    nx++;
+                }
+            }
+            const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.attn_norm, c.rms_eps};
+            if (n4) SKN_TRY(skn_gemm_q4k_multi(ctx, q4, n4, H, src, T));
+            if (nx) SKN_TRY(skn_gemm_expanded_multi(ctx, ex, nx, H, src, T));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
@@ -608,6 +654,11 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             const skn_gemm_seg wo = {L.wo, H, m->px, 1};
             const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};
             SKN_TRY(skn_gemm_q4k_multi(ctx, &wo, 1, H, src, T));
+        } else if (expand) {
+            skn_gemm_seg wo = {nullptr, H, m->px, 1};
+            SKN_TRY(expanded_copy(ctx, m, l, 3, L.type_o, L.wo, H, H, &wo.w));
+            const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};
+            SKN_TRY(skn_gemm_expanded_multi(ctx, &wo, 1, H, src, T));
         } else {
             SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
             SKN_TRY(skn_gemm_q(ctx, L.type_o, L.wo, H, H, m->pb16, T, m->pproj));
@@ -619,6 +670,23 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pmid, 0}, {L.w_up, F, m->pmid, 0}};
             const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.ffn_norm, c.rms_eps};
             SKN_TRY(skn_gemm_q4k_multi(ctx, gu, 2, H, src, T, true));
+        } else if (expand) {
+            const int types[2] = {L.type_gate, L.type_up};
+            const void* blocks[2] = {L.w_gate, L.w_up};
+            float* outs[2] = {m->pgate, m->pup};
+            const skn_gemm_src src = {SKN_SRC_RMSNORM, m->px, L.ffn_norm, c.rms_eps};
+            for (int i = 0; i < 2; i++) {
+                skn_gemm_seg seg = {blocks[i], F, outs[i], 0};
+                if (types[i] == SKN_TYPE_Q4_K && H <= 16384) {
+                    SKN_TRY(skn_gemm_q4k_multi(ctx, &seg, 1, H, src, T));
+                } else {
+                    SKN_TRY(expanded_copy(ctx, m, l, 4 + i, types[i], blocks[i], F, H, &seg.w));
+                    SKN_TRY(skn_gemm_expanded_multi(ctx, &seg, 1, H, src, T));
+                }
+            }
+            skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
+                       (const float*)m->pup, m->pmid, (int64_t)T * F);
+            SKN_LAUNCH_CHECK(ctx);
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
@@ -633,6 +701,11 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             const skn_gemm_seg down = {L.w_down, H, m->px, 1};  // residual added by the store
             const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
             SKN_TRY(skn_gemm_q4k_multi(ctx, &down, 1, F, mid, T));
+        } else if (expand) {
+            skn_gemm_seg down = {nullptr, H, m->px, 1};
+            SKN_TRY(expanded_copy(ctx, m, l, 6, L.type_down, L.w_down, H, F, &down.w));
+            const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
+            SKN_TRY(skn_gemm_expanded_multi(ctx, &down, 1, F, mid, T));
         } else {
             SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
             SKN_TRY(skn_gemm_q(ctx, L.type_down, L.w_down, H, F, m->pb16, T, m->pproj));

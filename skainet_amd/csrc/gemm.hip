@@ -704,7 +704,7 @@ template <int MT, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void gemm_hilo_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ bfrag,
                            const float* __restrict__ inv_scale, float* __restrict__ c, int m, int n, int steps,
-                           int m_tiles, int n_tiles) {
+                           int m_tiles, int n_tiles, int accumulate) {
     extern __shared__ __align__(16) float red[];  // 2 MT tiles x 3 copies x 1024 floats
     const int lane = threadIdx.x & 63, kq = threadIdx.x >> 6;
     const int slot_in_xcd = blockIdx.x >> 3;
@@ -796,19 +796,31 @@ void gemm_hilo_frag_kernel(const u32x4* __restrict__ afrag, const u32x4* __restr
                 for (int o = 0; o < 3; o++)
 #pragma unroll
                     for (int x = 0; x < 16; x++) sum[x] += red[(t * 3 + o) * 1024 + 64 * x + lane];
-                store_tile(sum, c, n, (mt * MT + i) * 32, tn * kBN + 32 * j, m, n, inv_scale, lane);
+                store_tile(sum, c, n, (mt * MT + i) * 32, tn * kBN + 32 * j, m, n, inv_scale, lane, accumulate != 0);
             }
         }
 }
 
 template <int MT, int D>
-int launch_hilo_gemm(skn_ctx* ctx, const u32x4* afrag, const u32x4* bfrag, const float* isc, float* c, int m, int n, int k) {
+int launch_hilo_gemm(skn_ctx* ctx, const u32x4* afrag, const u32x4* bfrag, const float* isc, float* c, int m, int n, int k,
+                     int accumulate = 0) {
     constexpr int kLds = 2 * MT * 3 * 4096;
     const int m_tiles = (m + 32 * MT - 1) / (32 * MT), n_tiles = (n + kBN - 1) / kBN;
     const unsigned grid = (unsigned)(((n_tiles + 7) / 8) * 8 * m_tiles);
-    skn_launch(ctx, gemm_hilo_frag_kernel<MT, D>, dim3(grid), dim3(256), kLds, afrag, bfrag, isc, c, m, n, k >> 4, m_tiles, n_tiles);
+    skn_launch(ctx, gemm_hilo_frag_kernel<MT, D>, dim3(grid), dim3(256), kLds, afrag, bfrag, isc, c, m, n, k >> 4, m_tiles, n_tiles,
+               accumulate);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
+}
+
+// row blocks per tile of the general path: 32 MT rows
+inline int hilo_mt(int m) { return m <= 32 ? 1 : (m <= 64 ? 2 : 4); }
+
+int launch_hilo_gemm_mt(skn_ctx* ctx, int mt, const u32x4* afrag, const u32x4* bfrag, const float* isc, float* c, int m, int n,
+                        int k, int accumulate) {
+    if (mt == 1) return launch_hilo_gemm<1, 4>(ctx, afrag, bfrag, isc, c, m, n, k, accumulate);
+    if (mt == 2) return launch_hilo_gemm<2, 4>(ctx, afrag, bfrag, isc, c, m, n, k, accumulate);
+    return launch_hilo_gemm<4, 4>(ctx, afrag, bfrag, isc, c, m, n, k, accumulate);
 }
 
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
@@ -923,7 +935,7 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     // general path.  Workspace: activations in fragment order (rows padded to whole tiles) + row scales, then
     // the weights as an fp16 pair in fragment order (rows padded to whole 64-column tiles)
     SKN_REQUIRE(ctx, ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG, "skn_gemm_q: activations must be 8-byte aligned");
-    const int mt = m <= 32 ? 1 : (m <= 64 ? 2 : 4);
+    const int mt = hilo_mt(m);
     const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt), n_pad = (n + kBN - 1) / kBN * kBN;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
     uint8_t* ws;
@@ -938,7 +950,85 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     SKN_LAUNCH_CHECK(ctx);
     rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;
-    if (mt == 1) return launch_hilo_gemm<1, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
-    if (mt == 2) return launch_hilo_gemm<2, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
-    return launch_hilo_gemm<4, 4>(ctx, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k);
+    return launch_hilo_gemm_mt(ctx, mt, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k, 0);
+}
+
+// ---- expanded weights: the general path with its weight pass done once ------------------------------------
+// The fp16-pair copy of a weight matrix that the general path builds per call (4 bytes per weight, rows padded to
+// whole 64-column tiles) can be kept by the caller: skn_gemm_expand fills it, skn_gemm_expanded multiplies with it.
+
+size_t skn_gemm_expanded_size(int n, int k) { return (size_t)((n + kBN - 1) / kBN * kBN) * (size_t)k * 4; }
+
+int skn_gemm_expanded_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m) {
+    SKN_REQUIRE(ctx, nseg >= 1 && m > 0 && k > 0 && k % 64 == 0, SKN_ERR_ARG, "expanded GEMM: bad segment count or shape");
+    SKN_REQUIRE(ctx, src.a && ((uintptr_t)src.a & (src.kind == SKN_SRC_BF16 ? 7 : 15)) == 0, SKN_ERR_ARG,
+                "expanded GEMM: activations are null or misaligned");
+    SKN_REQUIRE(ctx, src.kind == SKN_SRC_BF16 || src.kind == SKN_SRC_F32 || (src.b && ((uintptr_t)src.b & 15) == 0),
+                SKN_ERR_ARG, "expanded GEMM: second activation operand is null or misaligned");
+    for (int i = 0; i < nseg; i++)
+        SKN_REQUIRE(ctx, segs[i].w && segs[i].c && segs[i].n > 0 && ((uintptr_t)segs[i].w & 15) == 0, SKN_ERR_ARG,
+                    "expanded GEMM: weights must be non-null and 16-byte aligned");
+    const int mt = hilo_mt(m);
+    const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt);
+    const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
+    SKN_REQUIRE(ctx, af_bytes < ((size_t)1 << 31), SKN_ERR_SHAPE,
+                "expanded GEMM: %d rows of %d activations exceed the 2^30 elements one call takes", m, k);
+    uint8_t* ws;
+    int rc = gemm_workspace(ctx, af_bytes + is_bytes, &ws);
+    if (rc != SKN_OK) return rc;
+    _Float16* afrag = (_Float16*)ws;
+    float* isc = (float*)(ws + af_bytes);
+    _Float16* no_sums = nullptr;
+    switch (src.kind) {
+        case SKN_SRC_BF16: launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        case SKN_SRC_F32: launch_prep<SKN_SRC_F32, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        case SKN_SRC_RMSNORM: launch_prep<SKN_SRC_RMSNORM, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        default: return skn_fail(ctx, SKN_ERR_ARG, "expanded GEMM: unknown activation source %d", src.kind);
+    }
+    SKN_LAUNCH_CHECK(ctx);
+    for (int i = 0; i < nseg; i++) {
+        rc = launch_hilo_gemm_mt(ctx, mt, (const u32x4*)afrag, (const u32x4*)segs[i].w, isc, segs[i].c, m, segs[i].n, k,
+                                 segs[i].accumulate);
+        if (rc != SKN_OK) return rc;
+    }
+    return SKN_OK;
+}
+
+extern "C" int skn_gemm_expanded_bytes(skn_ctx* ctx, int ggml_type, int n, int k, size_t* bytes_out) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_gemm_expanded_bytes: ctx is null");
+    SKN_REQUIRE(ctx, bytes_out != nullptr, SKN_ERR_ARG, "skn_gemm_expanded_bytes: bytes_out is null");
+    SKN_REQUIRE(ctx, skn_is_quant(ggml_type), SKN_ERR_TYPE, "skn_gemm_expanded_bytes: ggml type %d is not supported", ggml_type);
+    SKN_REQUIRE(ctx, n >= 0 && k >= 0, SKN_ERR_ARG, "skn_gemm_expanded_bytes: negative shape");
+    int be, bb;
+    skn_type_block(ggml_type, &be, &bb);
+    SKN_REQUIRE(ctx, k % be == 0, SKN_ERR_SHAPE, "Quantized tensor row size (%d) is not a multiple of block size (%d)", k,
+                be);
+    SKN_REQUIRE(ctx, k % 64 == 0, SKN_ERR_SHAPE, "skn_gemm_expanded_bytes: k (%d) must be a multiple of %d", k, 64);
+    *bytes_out = skn_gemm_expanded_size(n, k);
+    return SKN_OK;
+}
+
+extern "C" int skn_gemm_expand(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, void* expanded_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_gemm_expand: ctx is null");
+    size_t bytes = 0;
+    int rc = skn_gemm_expanded_bytes(ctx, ggml_type, n, k, &bytes);
+    if (rc != SKN_OK) return rc;
+    if (bytes == 0) return SKN_OK;
+    SKN_REQUIRE(ctx, w_dev && expanded_dev, SKN_ERR_ARG, "skn_gemm_expand: null pointer");
+    SKN_REQUIRE(ctx, ((uintptr_t)expanded_dev & 15) == 0, SKN_ERR_ARG, "skn_gemm_expand: the copy must be 16-byte aligned");
+    return skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, expanded_dev);
+}
+
+extern "C" int skn_gemm_expanded(skn_ctx* ctx, const void* expanded_dev, int n, int k, const uint16_t* a_bf16_dev, int m,
+                                 float* c_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_gemm_expanded: ctx is null");
+    SKN_REQUIRE(ctx, n >= 0 && k >= 0 && m >= 0, SKN_ERR_ARG, "skn_gemm_expanded: negative shape");
+    SKN_REQUIRE(ctx, k % 64 == 0, SKN_ERR_SHAPE, "skn_gemm_expanded: k (%d) must be a multiple of %d", k, 64);
+    if (n == 0 || m == 0) return SKN_OK;
+    SKN_REQUIRE(ctx, c_dev != nullptr, SKN_ERR_ARG, "skn_gemm_expanded: c is null");
+    if (k == 0) return skn_memset(ctx, c_dev, 0, (size_t)m * n * sizeof(float));
+    SKN_REQUIRE(ctx, expanded_dev && a_bf16_dev, SKN_ERR_ARG, "skn_gemm_expanded: null pointer");
+    const skn_gemm_seg seg = {expanded_dev, n, c_dev, 0};
+    const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
+    return skn_gemm_expanded_multi(ctx, &seg, 1, k, src, m);
 }

@@ -83,6 +83,9 @@ _SIGNATURES = {
     "skn_dequant": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_void_p]),
     "skn_matvec_q": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "skn_gemm_q": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+    "skn_gemm_expanded_bytes": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
+    "skn_gemm_expand": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "skn_gemm_expanded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
     "skn_kv_create": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "skn_kv_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_kv_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -350,6 +353,20 @@ class Context:
 
     def gemm_q(self, ggml_type, w_dev, n, k, a_bf16_dev, m, c_dev):
         self._check(self.lib.skn_gemm_q(self.handle, ggml_type, _ptr(w_dev), n, k, _ptr(a_bf16_dev), m, _ptr(c_dev)))
+
+    def gemm_expanded_bytes(self, ggml_type, n, k):
+        out = C.c_size_t(0)
+        self._check(self.lib.skn_gemm_expanded_bytes(self.handle, ggml_type, n, k, C.byref(out)))
+        return int(out.value)
+
+    def gemm_expand(self, ggml_type, w_dev, n, k):
+        """-> device buffer with the expanded copy of W [n, k] that gemm_expanded multiplies with."""
+        buf = self.alloc(max(self.gemm_expanded_bytes(ggml_type, n, k), 16))
+        self._check(self.lib.skn_gemm_expand(self.handle, ggml_type, _ptr(w_dev), n, k, _ptr(buf)))
+        return buf
+
+    def gemm_expanded(self, expanded_dev, n, k, a_bf16_dev, m, c_dev):
+        self._check(self.lib.skn_gemm_expanded(self.handle, _ptr(expanded_dev), n, k, _ptr(a_bf16_dev), m, _ptr(c_dev)))
 
     def rmsnorm(self, x_dev, w_dev, rows, n, eps, y_dev):
         self._check(self.lib.skn_rmsnorm(self.handle, _ptr(x_dev), _ptr(w_dev), rows, n, eps, _ptr(y_dev)))

@@ -49,6 +49,7 @@ class QuantizedTensor:
             raise ValueError("quantized weights are rank-2 [out, in] tensors")
         runtime.row_bytes(ggml_type, shape.dimensions[1])  # the reference's block-multiple check (Quants.kt:10-20)
         self.ctx, self.ggml_type, self._shape, self.buf, self.transposed = ctx, ggml_type, shape, buf, transposed
+        self.expanded = None  # device copy made by expand_for_gemm
 
     @classmethod
     def from_bytes(cls, ctx, ggml_type, n_out, n_in, raw):
@@ -71,7 +72,17 @@ class QuantizedTensor:
         return self._shape.volume
 
     def t(self):
-        return QuantizedTensor(self.ctx, self.ggml_type, self._shape, self.buf, not self.transposed)
+        v = QuantizedTensor(self.ctx, self.ggml_type, self._shape, self.buf, not self.transposed)
+        v.expanded = self.expanded
+        return v
+
+    def expand_for_gemm(self):
+        """Keeps the fp16-pair copy of the weights that rank-2 products multiply with (4 bytes per weight of device
+        memory), so that later products skip the per-call weight pass.  Q4_K has no such pass and is left as it is."""
+        if self.expanded is None and self.ggml_type != synth.Q4_K:
+            n_out, n_in = self._shape.dimensions
+            self.expanded = self.ctx.gemm_expand(self.ggml_type, self.buf, n_out, n_in)
+        return self
 
     def dequantize(self):
         """-> DeviceTensor [out, in] fp32 (bit-exact ggml dequantization)."""
@@ -128,7 +139,10 @@ class DeviceTensor:
         a16 = self.ctx.alloc(max(2 * m * n_in, 16))
         self.ctx.f32_to_bf16(self.buf, m * n_in, a16)
         c = DeviceTensor.empty(self.ctx, Shape(m, n_out))
-        self.ctx.gemm_q(other.ggml_type, other.buf, n_out, n_in, a16, m, c.buf)
+        if other.expanded is not None:
+            self.ctx.gemm_expanded(other.expanded, n_out, n_in, a16, m, c.buf)
+        else:
+            self.ctx.gemm_q(other.ggml_type, other.buf, n_out, n_in, a16, m, c.buf)
         return c
 
     def relu(self):

@@ -10,7 +10,7 @@ steps in fp32.  Stored: the prompt, the greedy token of every step, and for the 
 steps 0, 1, 63 and 127 every eighth logit together with the vector's largest magnitude, its arg max and its top-two
 margin (the error metric is relative to the largest magnitude).
 
-The run takes about 40 minutes on 8 cores (640 tokens x 3.75 GB of blocks); it keeps its state in --state every 32
+The run takes about 55 minutes on 8 cores (640 tokens x 3.75 GB of blocks); it keeps its state in --state every 32
 tokens and resumes from there.
 """
 from __future__ import annotations

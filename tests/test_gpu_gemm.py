@@ -215,6 +215,64 @@ def test_gemm_full_width_slice(hip):
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("qtype", [Q6_K, synth.Q8_0, synth.Q5_K, synth.Q4_0, Q4_K])
+@pytest.mark.parametrize("m,n,k", [(512, 320, 1024), (40, 100, 512), (3, 64, 256)])
+def test_gemm_with_expanded_weights_equals_the_per_call_path(hip, qtype, m, n, k):
+    """skn_gemm_expand + skn_gemm_expanded: the weight pass of the general path done once; same kernels, so the
+    product equals skn_gemm_q's bit for bit for every other format, and the oracle's to the tolerance (also for Q4_K,
+    which skn_gemm_q multiplies on its own path).  The copy serves any number of products."""
+    raw = synth.weight(qtype, n, k, seed=21)
+    w = hip.to_device(raw)
+    assert hip.gemm_expanded_bytes(qtype, n, k) == (n + 63) // 64 * 64 * k * 4
+    exp = hip.gemm_expand(qtype, w, n, k)
+    for seed in (22, 23):
+        a = synth.activation_bf16((m, k), seed=seed)
+        a_dev = hip.to_device(a)
+        c = hip.alloc(4 * m * n)
+        hip.memset(c, 0xFF, 4 * m * n)
+        hip.gemm_expanded(exp, n, k, a_dev, m, c)
+        got = c.download(np.float32, m * n).reshape(m, n)
+        assert oracle_np.rel_err(got, oracle_c.gemm_q(qtype, raw, n, k, a, m)) <= TOL
+        if qtype != Q4_K:
+            assert np.array_equal(got.view(np.uint32), hip.gemm_q_host(qtype, raw, n, k, a, m).view(np.uint32))
+        a_dev.free(), c.free()
+    exp.free(), w.free()
+
+
+def test_gemm_expanded_benchmark_shape_q6k(hip):
+    """M=512, K=4096, N=4096 with Q6_K weights through the kept copy, sampled columns."""
+    m, n, k = 512, 4096, 4096
+    raw = synth.weight(Q6_K, n, k, seed=11)
+    a = synth.activation_bf16((m, k), seed=12)
+    w, a_dev, c = hip.to_device(raw), hip.to_device(a), hip.alloc(4 * m * n)
+    exp = hip.gemm_expand(Q6_K, w, n, k)
+    hip.gemm_expanded(exp, n, k, a_dev, m, c)
+    got = c.download(np.float32, m * n).reshape(m, n)
+    rows = np.arange(0, n, 127)
+    want = oracle_c.gemm_q(Q6_K, raw.reshape(n, -1)[rows].reshape(-1), len(rows), k, a, m)
+    err = np.max(np.abs(got[:, rows] - want) / np.maximum(np.abs(want), 1e-3 * np.abs(got).max()))
+    assert err <= TOL, err
+    for b in (w, a_dev, c, exp):
+        b.free()
+
+
+def test_gemm_expanded_errors(hip):
+    buf = hip.alloc(1 << 16)
+    with pytest.raises(runtime.SknError, match="not a multiple of block size"):
+        hip.gemm_expanded_bytes(Q6_K, 4, 100)
+    with pytest.raises(runtime.SknError, match="multiple of 64"):
+        hip.gemm_expanded_bytes(synth.Q8_0, 4, 96)
+    with pytest.raises(runtime.SknError, match="not supported"):
+        hip.gemm_expanded_bytes(999, 4, 256)
+    with pytest.raises(runtime.SknError, match="null pointer"):
+        hip._check(hip.lib.skn_gemm_expand(hip.handle, Q6_K, None, 4, 256, runtime._ptr(buf)))
+    with pytest.raises(runtime.SknError, match="multiple of 64"):
+        hip.gemm_expanded(buf, 4, 96, buf, 2, buf)
+    assert hip.gemm_expanded_bytes(Q6_K, 0, 256) == 0
+    hip.gemm_expanded(buf, 0, 256, buf, 2, buf)  # nothing to do
+    buf.free()
+
+
 def test_gemm_errors(hip):
     buf = hip.alloc(1 << 16)
     with pytest.raises(runtime.SknError) as e:
