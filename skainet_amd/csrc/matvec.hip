@@ -167,7 +167,7 @@ struct Q5kLoads : Q4kLoads {
 // The four fifth bits that go with a dword of nibbles are spread to bit 0 of its four bytes by one multiply
 // ((bits * 0x00204081) & 0x01010101: bit k lands on 8k, no two partial products meet), those of the high nibbles
 // to bit 1, which is the form q5k_dot_dword takes.
-constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5, kFmtIQ4NL = 8;
+constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5, kFmtIQ4NL = 8, kFmtIQ4XS = 9;
 constexpr int kFmtQ6K = 6, kFmtQ80 = 7;  // (fused kernels only: the lane maps, staging and steps of matvec_q6k_kernel / matvec_q80_pairs_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
@@ -199,6 +199,17 @@ __device__ __forceinline__ float iq4nl_dot4(uint32_t t, const float4& x, float s
     return s;
 }
 
+//   IQ4_XS (136 bytes per 256: f16 d, u16 scales_h, scales_l[4], qs[128]; 8-byte aligned): a superblock of eight
+//     sub-blocks of 32 with the element order and the table of IQ4_NL, so lane (sub, p) takes sub-blocks 2p and 2p + 1
+//     as it takes blocks 2p and 2p + 1 there: their 32 bytes of qs (two 16-byte vectors) and the eight header bytes.
+//     Scale of sub-block ib: nibble ib % 2 of scales_l[ib / 2] with bits 2 ib, 2 ib + 1 of scales_h on top, minus 32.
+__device__ __forceinline__ void iq4xs_load(const uint8_t* block, int p, Q4xLoads& L) {
+    L.a = *reinterpret_cast<const u32x4_a4*>(block + 8 + 32 * p);
+    L.b = *reinterpret_cast<const u32x4_a4*>(block + 24 + 32 * p);
+    const u32x2_a4 t = *reinterpret_cast<const u32x2_a4*>(block);
+    L.c = u32x4{t.x, t.y, 0u, 0u};
+}
+
 // the lane's two blocks: two 16-byte vectors and the format's tail of one to four dwords
 template <int F>
 __device__ __forceinline__ void q4x_load(const uint8_t* bp, Q4xLoads& L) {
@@ -220,13 +231,19 @@ __device__ __forceinline__ void q4x_load(const uint8_t* bp, Q4xLoads& L) {
 
 // the fields of the lane's first (half 0) or second block: nibble dwords, fifth bits, scale and offset
 template <int F>
-__device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t (&q)[4], uint32_t& qh, float& d, float& m) {
+__device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, int p, uint32_t (&q)[4], uint32_t& qh, float& d, float& m) {
     const u32x4 &a = L.a, &b = L.b, &c = L.c;
     auto lo16 = [](uint32_t w) { return (float)__builtin_bit_cast(half2_t, w).x; };
     auto hi16 = [](uint32_t w) { return (float)__builtin_bit_cast(half2_t, w).y; };
     auto al = [](uint32_t hi, uint32_t lo) { return __builtin_amdgcn_alignbyte(hi, lo, 2); };
     qh = 0u, m = 0.f;
-    if (F == kFmtQ40 || F == kFmtIQ4NL) {
+    if (F == kFmtIQ4XS) {
+        const u32x4& v = half == 0 ? a : b;
+        q[0] = v.x, q[1] = v.y, q[2] = v.z, q[3] = v.w;
+        const int ib = 2 * p + half;
+        const int ls = (int)(((c.y >> (8 * p + 4 * half)) & 0xFu) | ((((c.x >> 16) >> (2 * ib)) & 3u) << 4)) - 32;
+        d = lo16(c.x) * (float)ls;
+    } else if (F == kFmtQ40 || F == kFmtIQ4NL) {
         if (half == 0) q[0] = al(a.y, a.x), q[1] = al(a.z, a.y), q[2] = al(a.w, a.z), q[3] = al(b.x, a.w), d = lo16(a.x);
         else q[0] = b.y, q[1] = b.z, q[2] = b.w, q[3] = c.x, d = hi16(b.x);
     } else if (F == kFmtQ41) {
@@ -244,7 +261,7 @@ __device__ __forceinline__ void q4x_fields(const Q4xLoads& L, int half, uint32_t
 template <int R, int F>
 __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
                                          int s, int lane, float (&acc)[R]) {
-    constexpr bool kFive = F == kFmtQ50 || F == kFmtQ51, kTable = F == kFmtIQ4NL;
+    constexpr bool kFive = F == kFmtQ50 || F == kFmtQ51, kTable = F == kFmtIQ4NL || F == kFmtIQ4XS;
     // the quant that stands for zero (IQ4_NL: the staged sums already carry the 128 of the table)
     constexpr float kZero = F == kFmtQ40 ? -8.0f : (F == kFmtQ50 ? -16.0f : (kTable ? -1.0f : 0.0f));
     const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // the sums of x over the two blocks (x 2^-24)
@@ -264,7 +281,7 @@ __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* _
         for (int r = 0; r < R; r++) {
             uint32_t q[4], qh;
             float d, m;
-            q4x_fields<F>(L[r], half, q, qh, d, m);
+            q4x_fields<F>(L[r], half, lane & 3, q, qh, d, m);
             float alo = 0.f, ahi = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -351,11 +368,11 @@ __device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restr
 template <int STEPS, int R, int F = kFmtQ4K>
 __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                          float* __restrict__ y, int n_rows, int nb) {
-    constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40;
+    constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40, kXS = F == kFmtIQ4XS;
     using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
     constexpr int kSmallBytes = (F == kFmtQ40 || F == kFmtIQ4NL) ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
-    constexpr bool kPlainX = F == kFmtIQ4NL;  // x staged unscaled, block sums times 128, results in true units
+    constexpr bool kPlainX = F == kFmtIQ4NL || kXS;  // x staged unscaled, block sums times 128, results in true units
     extern __shared__ float4 lds4[];
     const int steps = STEPS > 0 ? STEPS : (nb + 15) >> 4;
     float4* xs = lds4;
@@ -368,7 +385,8 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     const int row0 = (blockIdx.x * waves + wave) * R;
     const int sub = lane >> 2;  // superblock within the step
     const int p = lane & 3;     // sub-block pair within the superblock
-    const size_t row_chunks = kSmall ? (size_t)nb * (kSmallBytes / 2) : (size_t)nb * kChunks;  // (eight blocks: kSmallBytes / 2 chunks)
+    // bytes of a row (eight small blocks: 8 * kSmallBytes)
+    const size_t row_bytes = kXS ? (size_t)nb * 136 : kSmall ? (size_t)nb * (8 * kSmallBytes) : (size_t)nb * (16 * kChunks);
     const int n4 = nb * 64;  // float4 count of x
 
     // the first J float4 per thread go into registers now; J covers all of x in the unrolled kernels
@@ -385,13 +403,15 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
         acc[r] = 0.f;
         row_ok[r] = row0 + r < n_rows;
         // slots past the end of a row / past the last row read valid memory (clamped) and are masked at the end
-        rp[r] = reinterpret_cast<const u32x4*>(w) + (size_t)min(row0 + r, n_rows - 1) * row_chunks + (kSmall ? 0 : kFirst + 2 * p);
+        rp[r] = reinterpret_cast<const u32x4*>(w + (size_t)min(row0 + r, n_rows - 1) * row_bytes) + (kSmall ? 0 : kFirst + 2 * p);
     }
     auto issue = [&](int s, int tie, Loads (&L)[R]) __attribute__((always_inline)) {
         const int blk = s * 16 + sub;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if constexpr (kSmall) {
+            if constexpr (kXS) {
+                iq4xs_load(reinterpret_cast<const uint8_t*>(rp[r]) + (size_t)min(blk, nb - 1) * 136 + tie, p, L[r]);
+            } else if constexpr (kSmall) {
                 const uint8_t* bp = reinterpret_cast<const uint8_t*>(rp[r]) + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
                 q4x_load<F>(bp, L[r]);
             } else {
@@ -625,7 +645,9 @@ struct Q6kLoads {
     bool ok;
 };
 
-// float4 f of x -> (step, lane, slot) of the Q6_K lane order; also the run sums
+// float4 f of x -> (step, lane, slot) of the Q6_K lane order; also the run sums, times ZERO * 2^-24 (ZERO: the quant
+// that stands for zero -- 32 for Q6_K, 4 for Q3_K; 1 where the sums serve a separate minimum term, as in Q2_K)
+template <int ZERO = 32>
 __device__ __forceinline__ void q6k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
     const int e = 4 * f;
     const int b = e >> 8, r = e & 255;
@@ -637,7 +659,7 @@ __device__ __forceinline__ void q6k_stage_store_one(const float4& v, int f, floa
     float sum = (v.x + v.y) + (v.z + v.w);
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));  // lane ^ 1
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x4E, 0xF, 0xF, true));  // lane ^ 2
-    if ((f & 3) == 0) ss[(step * 64 + ln) * 4 + q] = sum * (32.0f * 5.9604644775390625e-08f);  // 32 * 2^-24
+    if ((f & 3) == 0) ss[(step * 64 + ln) * 4 + q] = sum * ((float)ZERO * 5.9604644775390625e-08f);  // ZERO * 2^-24
 }
 
 __device__ __forceinline__ float q6k_dot4(uint32_t v, const float4& x, float s) {
@@ -780,6 +802,187 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
     }
     acc = wave_sum(acc);
     if (lane == 0) y[row] = acc;
+}
+
+// ------------------------------------------------------------------------------------------ Q2_K, Q3_K
+//
+// The two-bit formats pack their superblock as Q6_K packs its low bits: byte qs[32n + l] holds, at bit pairs
+// j = 0..3, the elements 128n + 32j + l, and the scale of an element is the one of its run of sixteen
+// (8n + 2j + (l >= 16)).  So the Q6_K lane map carries over -- lane (b, jj) = (lane / 4, lane % 4) owns half
+// n = jj / 2, bytes l = 16 (jj % 2) .. + 15: sixteen bytes of qs = 64 weights = four runs of sixteen consecutive
+// activations under one scale each -- and with it the staging of x in lane order, the run sums, the one-step
+// lookahead and the reduction.
+//   Q2_K (84 bytes: scales[16], qs[64], f16 d, f16 dmin; 4-byte aligned): one 16-byte load of qs, the eight scale
+//     bytes of the half, the dword d | dmin.  y = d * sum_j sc_j * (q . x)_j - dmin * sum_j m_j * (sum x)_j.
+//   Q3_K (110 bytes: hmask[32], qs[64], scales[12], f16 d; 2-byte aligned): 16 bytes of qs, the 16 bytes of hmask
+//     at the same l (bit 4n + j of hmask[l] is the third bit of element 128n + 32j + l), the twelve scale bytes and
+//     d.  The three-bit value q | hbit << 2 stands for q - 4 + 4 hbit, so the zero point returns as 4 * sum(x of
+//     the run).  Scale of run j (index is = 8n + 2j + hsel): low four bits in nibble n of byte 2j + hsel, two more
+//     in bits 4n + 2 (j / 2) of byte 8 + (2j + hsel) % 4, stored with an offset of 32.
+// A byte of two or three bits masked out in pairs (v & 0x00FF00FF) is a pair of fp16 subnormals, as in Q6_K.
+constexpr int kRunsQ2K = 0, kRunsQ3K = 1;
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t u32x3_a2 __attribute__((ext_vector_type(3), aligned(2)));
+
+struct Q2kLoads {
+    u32x4 q;
+    u32x2 sc;
+    uint32_t dd;
+    bool ok;
+};
+
+struct Q3kLoads {
+    u32x4 q, hm;
+    u32x3 sc;
+    uint32_t d;
+    bool ok;
+};
+
+template <int R>
+__device__ __forceinline__ void q2k_step(const Q2kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, int hsel, float (&acc)[R]) {
+    float S[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) S[r][0] = S[r][1] = S[r][2] = S[r][3] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float4 xq[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) xq[q] = xs[(s * 16 + 4 * q + i) * kXPitch + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t dw = L[r].q[i];
+            S[r][0] = q6k_dot4(dw & 0x03030303u, xq[0], S[r][0]);
+            S[r][1] = q6k_dot4((dw >> 2) & 0x03030303u, xq[1], S[r][1]);
+            S[r][2] = q6k_dot4((dw >> 4) & 0x03030303u, xq[2], S[r][2]);
+            S[r][3] = q6k_dot4((dw >> 6) & 0x03030303u, xq[3], S[r][3]);
+        }
+    }
+    const float4 sx = reinterpret_cast<const float4*>(ss)[s * 64 + lane];  // sums of x over the four runs (x 2^-24)
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        // scale bytes hsel, hsel + 2, hsel + 4, hsel + 6 of the half's eight: low nibble scale, high nibble minimum
+        const uint32_t w0 = L[r].sc.x >> (8 * hsel), w1 = L[r].sc.y >> (8 * hsel);
+        float v = (float)(w0 & 0xF) * S[r][0];
+        v = fmaf((float)((w0 >> 16) & 0xF), S[r][1], v);
+        v = fmaf((float)(w1 & 0xF), S[r][2], v);
+        v = fmaf((float)((w1 >> 16) & 0xF), S[r][3], v);
+        float m = (float)((w0 >> 4) & 0xF) * sx.x;
+        m = fmaf((float)((w0 >> 20) & 0xF), sx.y, m);
+        m = fmaf((float)((w1 >> 4) & 0xF), sx.z, m);
+        m = fmaf((float)((w1 >> 20) & 0xF), sx.w, m);
+        const uint32_t dd = L[r].dd;
+        const float t = fmaf(h2f_bits(dd & 0xFFFF), v, -(h2f_bits(dd >> 16) * m));
+        acc[r] += L[r].ok ? t : 0.f;
+    }
+}
+
+template <int R>
+__device__ __forceinline__ void q3k_step(const Q3kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, int n, int hsel, float (&acc)[R]) {
+    float S[R][4];
+#pragma unroll
+    for (int r = 0; r < R; r++) S[r][0] = S[r][1] = S[r][2] = S[r][3] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float4 xq[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) xq[q] = xs[(s * 16 + 4 * q + i) * kXPitch + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t dw = L[r].q[i], hb = L[r].hm[i] >> (4 * n);  // third bits of the half: bit j of each byte
+            S[r][0] = q6k_dot4((dw & 0x03030303u) | ((hb << 2) & 0x04040404u), xq[0], S[r][0]);
+            S[r][1] = q6k_dot4(((dw >> 2) & 0x03030303u) | ((hb << 1) & 0x04040404u), xq[1], S[r][1]);
+            S[r][2] = q6k_dot4(((dw >> 4) & 0x03030303u) | (hb & 0x04040404u), xq[2], S[r][2]);
+            S[r][3] = q6k_dot4(((dw >> 6) & 0x03030303u) | ((hb >> 1) & 0x04040404u), xq[3], S[r][3]);
+        }
+    }
+    const float4 sx = reinterpret_cast<const float4*>(ss)[s * 64 + lane];  // 4 * 2^-24 * sums of x over the runs
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t w0 = L[r].sc.x >> (8 * hsel), w1 = L[r].sc.y >> (8 * hsel), w2 = L[r].sc.z >> (8 * hsel);
+        const int lo = 4 * n;
+        const float c0 = (float)((int)(((w0 >> lo) & 0xF) | (((w2 >> lo) & 3) << 4)) - 32);
+        const float c1 = (float)((int)(((w0 >> (16 + lo)) & 0xF) | (((w2 >> (16 + lo)) & 3) << 4)) - 32);
+        const float c2 = (float)((int)(((w1 >> lo) & 0xF) | (((w2 >> (lo + 2)) & 3) << 4)) - 32);
+        const float c3 = (float)((int)(((w1 >> (16 + lo)) & 0xF) | (((w2 >> (18 + lo)) & 3) << 4)) - 32);
+        float v = c0 * (S[r][0] - sx.x);
+        v = fmaf(c1, S[r][1] - sx.y, v);
+        v = fmaf(c2, S[r][2] - sx.z, v);
+        v = fmaf(c3, S[r][3] - sx.w, v);
+        acc[r] += L[r].ok ? h2f_bits(L[r].d) * v : 0.f;
+    }
+}
+
+template <int STEPS, int R, int F>
+__global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                          float* __restrict__ y, int n_rows, int nb) {
+    constexpr bool Q2 = F == kRunsQ2K;
+    constexpr int kBlock = Q2 ? 84 : 110;
+    using Loads = std::conditional_t<Q2, Q2kLoads, Q3kLoads>;
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);  // float4 per (step, lane)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 2, j = lane & 3, n = j >> 1, hsel = j & 1;
+    const int row0 = (blockIdx.x * 8 + wave) * R;
+    const int n4 = nb * 64;
+    constexpr int J = 2 * STEPS;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+
+    float acc[R];
+    const uint8_t* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        rp[r] = w + (size_t)min(row0 + r, n_rows - 1) * nb * kBlock;
+    }
+    Loads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int blk = s * 16 + sub;
+        const size_t off = (size_t)(min(blk, nb - 1) + tie) * kBlock;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t* bp = rp[r] + off;
+            if constexpr (Q2) {
+                L[s][r].q = *reinterpret_cast<const u32x4_a4*>(bp + 16 + 32 * n + 16 * hsel);
+                L[s][r].sc = *reinterpret_cast<const u32x2_a4*>(bp + 8 * n);
+                L[s][r].dd = *reinterpret_cast<const uint32_t*>(bp + 80);
+            } else {
+                L[s][r].q = *reinterpret_cast<const u32x4_a2*>(bp + 32 + 32 * n + 16 * hsel);
+                L[s][r].hm = *reinterpret_cast<const u32x4_a2*>(bp + 16 * hsel);
+                L[s][r].sc = *reinterpret_cast<const u32x3_a2*>(bp + 96);
+                L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 108);
+            }
+            L[s][r].ok = row_ok[r] && blk < nb;
+        }
+    };
+    issue(0, 0);
+#pragma unroll
+    for (int jj = 0; jj < J; jj++) {
+        // a float4 index past the end repeats the last one: same data to the same slot
+        const int f = min(tid + jj * 512, n4 - 1);
+        q6k_stage_store_one<Q2 ? 1 : 4>(st.v[jj], f, xs, ss);
+    }
+    __syncthreads();
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        if constexpr (Q2) q2k_step<R>(L[s], xs, ss, s, lane + tie, hsel, acc);
+        else q3k_step<R>(L[s], xs, ss, s, lane + tie, n, hsel, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]) * 16777216.0f;
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
+    }
 }
 
 // What the rotary epilogue needs beyond the row totals, formed at the top of the kernel so that its dependent
@@ -1102,6 +1305,33 @@ int launch_q6k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, fl
     return SKN_OK;
 }
 
+// Q2_K / Q3_K on the Q6_K lane map: two rows per wavefront while a row is one or two steps, one beyond
+template <int STEPS, int F>
+int launch_runs(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y) {
+    constexpr int R = STEPS <= 2 ? 2 : 1;
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float4));
+    dim3 grid((unsigned)((n + 8 * R - 1) / (8 * R))), block(512);
+    skn_launch(ctx, matvec_runs_kernel<STEPS, R, F>, grid, block, lds, w, x, y, n, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int F>
+int dispatch_runs(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y) {
+    switch ((nb + 15) / 16) {
+        case 1: return launch_runs<1, F>(ctx, w, n, nb, x, y);
+        case 2: return launch_runs<2, F>(ctx, w, n, nb, x, y);
+        case 3: return launch_runs<3, F>(ctx, w, n, nb, x, y);
+        default: return launch_runs<4, F>(ctx, w, n, nb, x, y);
+    }
+}
+
+template <int STEPS, int F>
+hipError_t allow_big_lds_runs() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_runs_kernel<STEPS, (STEPS <= 2 ? 2 : 1), F>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
 template <int STEPS>
 hipError_t allow_big_lds_q6k() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q6k_kernel<STEPS, 1>),
@@ -1134,13 +1364,22 @@ int skn_matvec_init(skn_ctx* ctx) {
         allow_big_lds<4, 1, F>, allow_big_lds<0, 2, F>, allow_big_lds<1, 2, F>, allow_big_lds<2, 2, F>,         \
         allow_big_lds<3, 2, F>, allow_big_lds<4, 2, F>
                              SKN_ALLOW_FMT(kFmtQ5K), SKN_ALLOW_FMT(kFmtQ40), SKN_ALLOW_FMT(kFmtQ41),
-                             SKN_ALLOW_FMT(kFmtQ50), SKN_ALLOW_FMT(kFmtQ51), SKN_ALLOW_FMT(kFmtIQ4NL)};
+                             SKN_ALLOW_FMT(kFmtQ50), SKN_ALLOW_FMT(kFmtQ51), SKN_ALLOW_FMT(kFmtIQ4NL),
+                             SKN_ALLOW_FMT(kFmtIQ4XS)};
 #undef SKN_ALLOW_FMT
     for (auto f : fns) SKN_HIP(ctx, f());
     SKN_HIP(ctx, allow_big_lds_q6k<1>());
     SKN_HIP(ctx, allow_big_lds_q6k<2>());
     SKN_HIP(ctx, allow_big_lds_q6k<3>());
     SKN_HIP(ctx, allow_big_lds_q6k<4>());
+    SKN_HIP(ctx, (allow_big_lds_runs<1, kRunsQ2K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsQ2K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsQ2K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsQ2K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<1, kRunsQ3K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsQ3K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsQ3K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsQ3K>()));
     SKN_HIP(ctx, allow_big_lds_q80<1>());
     SKN_HIP(ctx, allow_big_lds_q80<2>());
     SKN_HIP(ctx, allow_big_lds_q80<3>());
@@ -1287,6 +1526,14 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         }
 #undef SKN_SMALL
     }
+    // IQ4_XS: the superblock form of IQ4_NL on the same kernel (its blocks are 8-byte aligned)
+    if (ggml_type == SKN_TYPE_IQ4_XS && ((uintptr_t)w_dev & 7) == 0 && nb <= 144 && ctx->opt_matvec_stage == 1)
+        return nb > 32 ? dispatch_q4k<1, kFmtIQ4XS>(ctx, w, n, nb, x_dev, y_dev, 8) : dispatch_q4k<2, kFmtIQ4XS>(ctx, w, n, nb, x_dev, y_dev, 8);
+    // Q2_K / Q3_K on the lane map of the Q6_K kernel (rows of at most four steps)
+    if (ggml_type == SKN_TYPE_Q2_K && ((uintptr_t)w_dev & 3) == 0 && nb <= 64 && ctx->opt_matvec_stage == 1)
+        return dispatch_runs<kRunsQ2K>(ctx, w, n, nb, x_dev, y_dev);
+    if (ggml_type == SKN_TYPE_Q3_K && nb <= 64 && ctx->opt_matvec_stage == 1)
+        return dispatch_runs<kRunsQ3K>(ctx, w, n, nb, x_dev, y_dev);
     if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;

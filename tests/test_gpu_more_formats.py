@@ -60,7 +60,8 @@ def test_matvec_vs_oracle(hip, qtype, name, n, k):
     assert oracle_np.rel_err(got, want) <= TOL
 
 
-STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs")]
+STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"), (10, "q2_k"), (13, "q5_k"), (15, "q8_k"), (23, "iq4_xs"),
+          (11, "q3_k")]
 
 
 @pytest.mark.parametrize("qtype,name", STAGED)
@@ -68,8 +69,8 @@ STAGED = [(2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"), (1
 def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
     """The formats whose rows pass through LDS: several chunks per row with a short last one (k = 11008), the
     longest row, fewer rows than a workgroup takes -- every kernel the option selects (0: direct reads, 2: row
-    staged in LDS, 1: the default, which for Q5_K is the kernel on the Q4_K lane map) against the oracle and
-    against each other."""
+    staged in LDS, 1: the default, which for Q5_K, the small-block formats and IQ4_XS is the kernel on the Q4_K lane
+    map and for Q2_K / Q3_K the one on the Q6_K lane map) against the oracle and against each other."""
     raw = synth.weight(qtype, n, k, seed=3 * n + k + qtype)
     x = synth.activation_f32(k, seed=k + 1)
     want = oracle_c.matvec_q(qtype, raw, n, k, x)
@@ -85,12 +86,14 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
         assert np.abs(got[stage] - got[0]).max() <= 1e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl")])
+@pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"),
+                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
     eight small blocks, each), a partial last step, the rolled loop beyond four steps, the longest row the kernel
-    takes (144 superblocks) and one past it (direct kernel)."""
+    takes (144 superblocks) and one past it (direct kernel).  Q2_K and Q3_K (the Q6_K kernel's lane map): one to four
+    steps, then the kernels for longer rows."""
     raw = synth.weight(qtype, n, k, seed=n + k)
     x = synth.activation_f32(k, seed=k + 3)
     got = hip.matvec_q_host(qtype, raw, n, k, x)
@@ -162,6 +165,137 @@ def test_matvec_rows_not_16_byte_aligned(hip, qtype, name):
     xd, yd = hip.to_device(x), hip.alloc(4 * n)
     hip.matvec_q(qtype, buf.ptr + 4, n, k, xd, yd)
     assert oracle_np.rel_err(yd.download(np.float32, n), oracle_c.matvec_q(qtype, raw, n, k, x)) <= TOL
+
+
+def _against_oracle(hip, qtype, blocks, n, k, x):
+    got = hip.matvec_q_host(qtype, blocks.reshape(n, -1), n, k, x)
+    assert oracle_np.rel_err(got, oracle_c.matvec_q(qtype, blocks.reshape(n, -1), n, k, x)) <= TOL
+
+
+def test_q2k_matvec_fields_alone(hip):
+    """Q2_K (scales[16] @0, qs[64] @16, d @80, dmin @82) on the lane-map kernel, one field at a time: scales without
+    minimums and the reverse, each bit pair of qs alone, the bytes of either half of a run alone, one half of the
+    superblock alone -- a wrong scale index, shift or run sum shows at full scale."""
+    n, k = 16, 4096
+    raw = synth.weight(10, n, k, seed=41).reshape(n, k // 256, 84).copy()
+    x = synth.activation_f32(k, seed=42)
+    variants = []
+    for mask in (0x0F, 0xF0):
+        v = raw.copy()
+        v[:, :, :16] &= mask
+        variants.append(v)
+    for j in range(4):
+        v = raw.copy()
+        v[:, :, 16:80] &= 3 << (2 * j)
+        variants.append(v)
+    for lo in (0, 16):  # bytes l = lo .. lo + 15 of both halves
+        v = raw.copy()
+        keep = np.zeros(64, bool)
+        keep[lo:lo + 16] = keep[32 + lo:48 + lo] = True
+        v[:, :, 16:80][:, :, ~keep] = 0
+        v[:, :, :16] &= 0x0F  # (no minimums: the zeroed quants contribute nothing)
+        variants.append(v)
+    for half in (0, 1):
+        v = raw.copy()
+        v[:, :, 16 + 32 * (1 - half):48 + 32 * (1 - half)] = 0
+        v[:, :, 8 * (1 - half):8 + 8 * (1 - half)] = 0
+        variants.append(v)
+    for v in variants:
+        _against_oracle(hip, 10, v, n, k, x)
+
+
+def test_q3k_matvec_fields_alone(hip):
+    """Q3_K (hmask[32] @0, qs[64] @32, scales[12] @96, d @108): third bits all set (quants 0..3) or all clear (-4..-1)
+    or alone over zero low bits, each bit pair alone, each of the eight bit planes of hmask alone, the three parts of
+    the packed scales alone (low nibbles of bytes 0..7 = scales 0..7, high nibbles = 8..15, bytes 8..11 = the upper
+    two bits), one half alone."""
+    n, k = 16, 4096
+    rng = np.random.default_rng(6)
+    raw = synth.weight(11, n, k, seed=43).reshape(n, k // 256, 110).copy()
+    x = synth.activation_f32(k, seed=44)
+    variants = []
+    for fill in (0xFF, 0x00):
+        v = raw.copy()
+        v[:, :, :32] = fill
+        variants.append(v)
+    v = raw.copy()
+    v[:, :, 32:96] = 0
+    variants.append(v)
+    for j in range(4):
+        v = raw.copy()
+        v[:, :, 32:96] &= 3 << (2 * j)
+        variants.append(v)
+    for bit in range(8):
+        v = raw.copy()
+        v[:, :, :32] = (rng.integers(0, 2, size=(n, k // 256, 32), dtype=np.uint8) << bit) | (0xFF ^ (1 << bit))
+        v[:, :, 32:96] = 0  # quants: -4 where the plane's bit is clear, 0 elsewhere
+        variants.append(v)
+    for part in range(3):
+        v = raw.copy()
+        if part == 0:
+            v[:, :, 96:104] &= 0x0F
+            v[:, :, 104:108] = 0xAA  # upper bits 2: scales 32 + low nibble - 32
+        elif part == 1:
+            v[:, :, 96:104] &= 0xF0
+            v[:, :, 104:108] = 0xAA
+        else:
+            v[:, :, 96:104] = 0
+        variants.append(v)
+    for half in (0, 1):
+        v = raw.copy()
+        v[:, :, 32 + 32 * (1 - half):64 + 32 * (1 - half)] = 0
+        v[:, :, :32] |= 0x0F << (4 * (1 - half))  # the zeroed half's quants are 0, not -4
+        variants.append(v)
+    for v in variants:
+        _against_oracle(hip, 11, v, n, k, x)
+
+
+def test_iq4_xs_matvec_fields_alone(hip):
+    """IQ4_XS (d @0, scales_h @2, scales_l[4] @4, qs[128] @8): the upper scale bits alone and the lower alone, low
+    nibbles and high nibbles alone, each sub-block alone, and every table entry (all nibbles one index, scale 33 - 32)."""
+    n, k = 16, 4096
+    raw = synth.weight(23, n, k, seed=45).reshape(n, k // 256, 136).copy()
+    x = synth.activation_f32(k, seed=46)
+    variants = []
+    v = raw.copy()
+    v[:, :, 4:8] = 0
+    variants.append(v)
+    v = raw.copy()
+    v[:, :, 2:4] = 0
+    variants.append(v)
+    for mask in (0x0F, 0xF0):
+        v = raw.copy()
+        v[:, :, 8:] &= mask
+        v[:, :, 8:] |= 0x88 & ~mask  # index 8 of the table is the value 1, its smallest: the other nibbles nearly vanish
+        variants.append(v)
+    for ib in range(8):
+        v = raw.copy()
+        # scale 32 - 32 = 0 for every other sub-block: low bits 0, upper bits 2
+        sl = np.zeros(4, np.uint8)
+        sh = 0
+        for o in range(8):
+            val = 0x21 if o == ib else 0x20  # 33 or 32
+            sl[o // 2] |= (val & 0xF) << (4 * (o % 2))
+            sh |= (val >> 4) << (2 * o)
+        v[:, :, 4:8] = sl
+        v[:, :, 2] = sh & 0xFF
+        v[:, :, 3] = sh >> 8
+        variants.append(v)
+    for v in variants:
+        _against_oracle(hip, 23, v, n, k, x)
+    k = 1024
+    x = synth.activation_f32(k, seed=47)
+    blocks = np.zeros((16, k // 256, 136), np.uint8)
+    blocks[:, :, :2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    blocks[:, :, 2:4] = np.frombuffer(np.uint16(0xAAAA).tobytes(), np.uint8)  # upper bits 2 everywhere
+    blocks[:, :, 4:8] = 0x11                                                   # lower bits 1: scale 33 - 32 = 1
+    for i in range(16):
+        blocks[i, :, 8:] = i | (i << 4)
+    got = hip.matvec_q_host(23, blocks.reshape(16, -1), 16, k, x)
+    want = oracle_c.matvec_q(23, blocks.reshape(16, -1), 16, k, x)
+    table = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float64)
+    assert np.allclose(want, 0.5 * table * x.astype(np.float64).sum(), rtol=1e-5, atol=1e-4)
+    assert oracle_np.rel_err(got, want) <= TOL
 
 
 def test_iq4_nl_matvec_every_table_entry(hip):
