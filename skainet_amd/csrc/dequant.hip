@@ -27,64 +27,80 @@ __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t* __rest
 }
 
 // Q4_K: 144-byte superblock = f16 d @0, f16 dmin @2, 12 packed 6-bit scale/min bytes @4, 128 nibble bytes @16.
+// A thread takes one dword of nibbles and writes both of its quads -- the low nibbles (elements 64c + r .. + 3 of
+// sub-block 2c) and the high ones (the same positions of sub-block 2c + 1, 32 elements on): 32 threads per
+// superblock, one header load and one nibble load for two 16-byte stores; eight consecutive lanes still write one
+// whole 128-byte line per store.
 __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           int64_t n_quads) {
+                                                           int64_t n_pairs) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n_quads) return;
-    int64_t blk = t >> 6;    // 64 quads per 256-element superblock
-    int e = (int)(t & 63) * 4;  // first element of this quad inside the superblock
+    if (t >= n_pairs) return;
+    int64_t blk = t >> 5;        // 32 quad pairs per 256-element superblock
+    const int u = (int)(t & 31);
+    const int c = u >> 3, r = (u & 7) * 4;  // 64-element chunk, first position in its low half
     // superblocks are 16-byte aligned: the whole header (d, dmin, twelve scale / min bytes) is one 128-bit load
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     const u32x4* b128 = reinterpret_cast<const u32x4*>(w + blk * 144);
     const u32x4 hdr = b128[0];
-    float d = h2f_bits(hdr.x & 0xFFFF), dmin = h2f_bits(hdr.x >> 16);
-    int c = e >> 6, r = e & 63;
-    int j = 2 * c + (r >= 32);
+    const float d = h2f_bits(hdr.x & 0xFFFF), dmin = h2f_bits(hdr.x >> 16);
     // bytes 0..3 of the twelve: low scales, 4..7: low mins, 8..11: low nibbles of the high ones, whose top two
-    // bits sit in bits 6..7 of the first eight bytes
-    const int sh = 8 * (j & 3);
-    int sc, m;
-    if (j < 4) {
-        sc = (hdr.y >> sh) & 63;
-        m = (hdr.z >> sh) & 63;
-    } else {
-        sc = ((hdr.w >> sh) & 0x0F) | (((hdr.y >> (sh + 6)) & 3) << 4);
-        m = ((hdr.w >> (sh + 4)) & 0x0F) | (((hdr.z >> (sh + 6)) & 3) << 4);
+    // bits sit in bits 6..7 of the first eight bytes.  Sub-blocks j = 2c (low nibbles) and 2c + 1 (high nibbles)
+    int sc[2], m[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int j = 2 * c + i, sh = 8 * (j & 3);
+        if (j < 4) {
+            sc[i] = (hdr.y >> sh) & 63;
+            m[i] = (hdr.z >> sh) & 63;
+        } else {
+            sc[i] = ((hdr.w >> sh) & 0x0F) | (((hdr.y >> (sh + 6)) & 3) << 4);
+            m[i] = ((hdr.w >> (sh + 4)) & 0x0F) | (((hdr.z >> (sh + 6)) & 3) << 4);
+        }
     }
-    uint32_t q = reinterpret_cast<const uint32_t*>(b128)[4 + 8 * c + ((r & 31) >> 2)];
-    if (r >= 32) q >>= 4;
-    float d1 = __fmul_rn(d, (float)sc);
-    float m1 = __fmul_rn(dmin, (float)m);
-    float4 y;
-    y.x = __fsub_rn(__fmul_rn(d1, (float)(q & 0xF)), m1);
-    y.y = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xF)), m1);
-    y.z = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xF)), m1);
-    y.w = __fsub_rn(__fmul_rn(d1, (float)((q >> 24) & 0xF)), m1);
-    reinterpret_cast<float4*>(out)[t] = y;
+    const uint32_t q = reinterpret_cast<const uint32_t*>(b128)[4 + 8 * c + (r >> 2)];
+    float4* dst = reinterpret_cast<float4*>(out + blk * 256 + 64 * c + r);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const uint32_t qq = q >> (4 * i);
+        const float d1 = __fmul_rn(d, (float)sc[i]);
+        const float m1 = __fmul_rn(dmin, (float)m[i]);
+        float4 y;
+        y.x = __fsub_rn(__fmul_rn(d1, (float)(qq & 0xF)), m1);
+        y.y = __fsub_rn(__fmul_rn(d1, (float)((qq >> 8) & 0xF)), m1);
+        y.z = __fsub_rn(__fmul_rn(d1, (float)((qq >> 16) & 0xF)), m1);
+        y.w = __fsub_rn(__fmul_rn(d1, (float)((qq >> 24) & 0xF)), m1);
+        dst[8 * i] = y;  // + 32 elements
+    }
 }
 
 // Q6_K: 210-byte superblock = ql[128] @0 (low nibbles), qh[64] @128 (high bit pairs), int8 scales[16] @192, f16 d @208.
+// A thread takes one dword of ql and the dword of qh that goes with it and writes both quads that share them: the
+// low nibbles (quarter p = 0 or 1 of half n) and the high nibbles (quarter p + 2, 64 elements on).
 __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t* __restrict__ w, float* __restrict__ out,
-                                                           int64_t n_quads) {
+                                                           int64_t n_pairs) {
     int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= n_quads) return;
-    int64_t blk = t >> 6;
-    int e = (int)(t & 63) * 4;
+    if (t >= n_pairs) return;
+    int64_t blk = t >> 5;
+    const int u = (int)(t & 31);
     const uint8_t* b = w + blk * 210;  // only 2-byte aligned
-    int n = e >> 7, r = e & 127;
-    int quarter = r >> 5, l = r & 31;  // l is a multiple of 4
-    uint32_t lo = load_u32_a2(b + 64 * n + l + 32 * (quarter & 1));
-    if (quarter >= 2) lo >>= 4;
-    uint32_t hi = load_u32_a2(b + 128 + 32 * n + l) >> (2 * quarter);
-    float sc = (float)(int8_t)b[192 + 8 * n + 2 * quarter + (l >> 4)];
-    float d = h2f_bits(load_u16_a2(b + 208));
-    float ds = __fmul_rn(d, sc);
-    float4 y;
-    y.x = __fmul_rn(ds, (float)((int)((lo & 0xF) | ((hi & 3) << 4)) - 32));
-    y.y = __fmul_rn(ds, (float)((int)(((lo >> 8) & 0xF) | (((hi >> 8) & 3) << 4)) - 32));
-    y.z = __fmul_rn(ds, (float)((int)(((lo >> 16) & 0xF) | (((hi >> 16) & 3) << 4)) - 32));
-    y.w = __fmul_rn(ds, (float)((int)(((lo >> 24) & 0xF) | (((hi >> 24) & 3) << 4)) - 32));
-    reinterpret_cast<float4*>(out)[t] = y;
+    const int n = u >> 4, p = (u >> 3) & 1, l = (u & 7) * 4;
+    const uint32_t lo = load_u32_a2(b + 64 * n + 32 * p + l);
+    const uint32_t hi = load_u32_a2(b + 128 + 32 * n + l);
+    const float d = h2f_bits(load_u16_a2(b + 208));
+    float4* dst = reinterpret_cast<float4*>(out + blk * 256 + 128 * n + 32 * p + l);
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int quarter = p + 2 * i;
+        const uint32_t lq = lo >> (4 * i), hq = hi >> (2 * quarter);
+        const float sc = (float)(int8_t)b[192 + 8 * n + 2 * quarter + (l >> 4)];
+        const float ds = __fmul_rn(d, sc);
+        float4 y;
+        y.x = __fmul_rn(ds, (float)((int)((lq & 0xF) | ((hq & 3) << 4)) - 32));
+        y.y = __fmul_rn(ds, (float)((int)(((lq >> 8) & 0xF) | (((hq >> 8) & 3) << 4)) - 32));
+        y.z = __fmul_rn(ds, (float)((int)(((lq >> 16) & 0xF) | (((hq >> 16) & 3) << 4)) - 32));
+        y.w = __fmul_rn(ds, (float)((int)(((lq >> 24) & 0xF) | (((hq >> 24) & 3) << 4)) - 32));
+        dst[16 * i] = y;  // + 64 elements
+    }
 }
 
 }  // namespace
@@ -110,9 +126,9 @@ extern "C" int skn_dequant(skn_ctx* ctx, int ggml_type, const void* w_dev, int64
     if (ggml_type == SKN_TYPE_Q8_0)
         skn_launch(ctx, dequant_q8_0_kernel, grid, block, 0, w, out_dev, n_quads);
     else if (ggml_type == SKN_TYPE_Q4_K)
-        skn_launch(ctx, dequant_q4_k_kernel, grid, block, 0, w, out_dev, n_quads);
+        skn_launch(ctx, dequant_q4_k_kernel, dim3((unsigned)((n_quads / 2 + 255) / 256)), block, 0, w, out_dev, n_quads / 2);
     else
-        skn_launch(ctx, dequant_q6_k_kernel, grid, block, 0, w, out_dev, n_quads);
+        skn_launch(ctx, dequant_q6_k_kernel, dim3((unsigned)((n_quads / 2 + 255) / 256)), block, 0, w, out_dev, n_quads / 2);
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }
