@@ -62,7 +62,11 @@ class DeviceTensor internal constructor(
         try {
             ctx.check(SknLib.f32ToBf16.invokeExact(ctx.handle, dev, m.toLong() * k, a16) as Int)
             val c = ctx.newTensor(Shape(m, n))
-            ctx.check(SknLib.gemmQ.invokeExact(ctx.handle, other.ggmlType.value, other.dev, n, k, a16, m, c.dev) as Int)
+            val kept = other.expanded
+            if (kept != null)
+                ctx.check(SknLib.gemmExpanded.invokeExact(ctx.handle, kept, n, k, a16, m, c.dev) as Int)
+            else
+                ctx.check(SknLib.gemmQ.invokeExact(ctx.handle, other.ggmlType.value, other.dev, n, k, a16, m, c.dev) as Int)
             return c
         } finally {
             ctx.sync()      // the GEMM reads a16 asynchronously

@@ -44,7 +44,24 @@ class QuantizedTensor internal constructor(
         get() = if (transposed) Shape(inFeatures, outFeatures) else storedShape
     override val dataDescriptor: DataDescriptor get() = descriptor
 
-    override fun t(): Tensor = QuantizedTensor(ctx, ggmlType, storedShape, dev, !transposed, owner = false)
+    /** The fp16-pair copy that rank-2 products multiply with (skn_gemm_expand); shared by the views t() makes. */
+    internal var expanded: MemorySegment? = null
+
+    override fun t(): Tensor =
+        QuantizedTensor(ctx, ggmlType, storedShape, dev, !transposed, owner = false).also { it.expanded = expanded }
+
+    /**
+     * Keeps the expanded copy of the weights on the device (4 bytes per weight) so that rank-2 products skip the
+     * per-call weight pass of the formats other than Q4_K, which has none and is left as it is.
+     */
+    fun expandForGemm(): QuantizedTensor {
+        if (expanded == null && ggmlType != GGMLQuantizationType.Q4_K) {
+            val copy = ctx.malloc(ctx.gemmExpandedBytes(ggmlType.value, outFeatures, inFeatures))
+            ctx.check(SknLib.gemmExpand.invokeExact(ctx.handle, ggmlType.value, dev, outFeatures, inFeatures, copy) as Int)
+            expanded = copy
+        }
+        return this
+    }
 
     /** skn_dequant: the dequantizer the reference leaves as a TODO (gguf/.../Quants.kt:8), bit-exact ggml values. */
     fun dequantize(): DeviceTensor {
@@ -92,7 +109,10 @@ class QuantizedTensor internal constructor(
     override fun flatten(startDim: Int, endDim: Int): Tensor = toDoubles().flatten(startDim, endDim)
 
     override fun close() {
-        if (owner) ctx.free(dev)
+        if (owner) {
+            expanded?.let { ctx.free(it) }
+            ctx.free(dev)
+        }
     }
 }
 

@@ -9,6 +9,7 @@ import java.lang.foreign.MemorySegment
 import java.lang.foreign.ValueLayout.ADDRESS
 import java.lang.foreign.ValueLayout.JAVA_BYTE
 import java.lang.foreign.ValueLayout.JAVA_FLOAT
+import java.lang.foreign.ValueLayout.JAVA_LONG
 
 class SknException(val code: Int, message: String) : IllegalStateException(message)
 
@@ -79,6 +80,13 @@ class SknContext(device: Int = 0) : AutoCloseable {
         val host = arena.allocate(JAVA_FLOAT, count.toLong())
         download(host, dev, 4L * count)
         host.toArray(JAVA_FLOAT)
+    }
+
+    /** Size of the expanded copy of an [n, k] weight matrix (skn_gemm_expanded_bytes; size_t is 64 bits here). */
+    fun gemmExpandedBytes(type: Int, n: Int, k: Int): Long = Arena.ofConfined().use { arena ->
+        val out = arena.allocate(JAVA_LONG)
+        check(SknLib.gemmExpandedBytes.invokeExact(handle, type, n, k, out) as Int)
+        out.get(JAVA_LONG, 0)
     }
 
     fun newTensor(shape: Shape): DeviceTensor = DeviceTensor(this, shape, malloc(4L * shape.volume))
