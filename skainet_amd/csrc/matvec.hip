@@ -590,6 +590,92 @@ __global__ __launch_bounds__(512) void matvec_q80_pairs_kernel(const uint8_t* __
     }
 }
 
+// Q8_K (292 bytes per 256: f32 d @0, int8 qs[256] @4, int16 sums of sixteen @260, unused here; 4-byte aligned) on the
+// same scheme with the Q4_K lane map: lane (b, p) = (lane / 4, lane % 4) of a step owns the 64 quants 64p .. 64p + 63
+// of superblock b -- four 16-byte loads -- and its 64 consecutive activations; d is one more dword.
+struct Q8kLoads {
+    u32x4 w[4];
+    float d;
+    bool ok;
+};
+
+template <int R>
+__device__ __forceinline__ void q8k_step(const Q8kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, float (&acc)[R]) {
+    float sa[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) sa[r] = 0.f;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {  // sixteen quants at a time: one of the lane's four vectors
+        float4 xv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) xv[j] = xs[(s * 16 + 4 * q + j) * kXPitch + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) sa[r] = q80_dot_dword(L[r].w[q][j], xv[j], sa[r]);
+        }
+    }
+    const float2 sx = reinterpret_cast<const float2*>(ss)[s * 64 + lane];  // 128 * the sums of x over the two halves
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] += L[r].ok ? L[r].d * (sa[r] - (sx.x + sx.y)) : 0.f;
+}
+
+template <int STEPS, int R>
+__global__ __launch_bounds__(512) void matvec_q8k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ y, int n_rows, int nb) {
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 2, p = lane & 3;
+    const int row0 = (blockIdx.x * 8 + wave) * R;
+    const int n4 = nb * 64;  // float4 count of x
+    constexpr int J = 2 * STEPS;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+
+    float acc[R];
+    const uint8_t* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        rp[r] = w + (size_t)min(row0 + r, n_rows - 1) * nb * 292;
+    }
+    Q8kLoads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int blk = s * 16 + sub;
+        const size_t off = (size_t)(min(blk, nb - 1) + tie) * 292;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const u32x4_a4* bp = reinterpret_cast<const u32x4_a4*>(rp[r] + off + 4 + 64 * p);
+#pragma unroll
+            for (int i = 0; i < 4; i++) L[s][r].w[i] = bp[i];
+            L[s][r].d = *reinterpret_cast<const float*>(rp[r] + off);
+            L[s][r].ok = row_ok[r] && blk < nb;
+        }
+    };
+    issue(0, 0);
+    q4k_stage_store<J, false>(st, n4, tid, 512, xs, ss);
+    __syncthreads();
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        q8k_step<R>(L[s], xs, ss, s, lane + tie, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
+    }
+}
+
 // General form (any alignment, any block count): one wavefront per row; lane l takes blocks l, l+64, ...  The
 // lane's 34 bytes are fetched as seventeen 16-bit loads (consecutive lanes read consecutive blocks, so the
 // wavefront still walks one contiguous range) and x as eight aligned float4.
@@ -1333,6 +1419,22 @@ hipError_t allow_big_lds_runs() {
 }
 
 template <int STEPS>
+int launch_q8k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y) {
+    constexpr int R = STEPS <= 2 ? 2 : 1;
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
+    dim3 grid((unsigned)((n + 8 * R - 1) / (8 * R))), block(512);
+    skn_launch(ctx, matvec_q8k_kernel<STEPS, R>, grid, block, lds, w, x, y, n, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int STEPS>
+hipError_t allow_big_lds_q8k() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q8k_kernel<STEPS, (STEPS <= 2 ? 2 : 1)>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
+template <int STEPS>
 hipError_t allow_big_lds_q6k() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q6k_kernel<STEPS, 1>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1380,6 +1482,10 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsQ3K>()));
     SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsQ3K>()));
     SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsQ3K>()));
+    SKN_HIP(ctx, allow_big_lds_q8k<1>());
+    SKN_HIP(ctx, allow_big_lds_q8k<2>());
+    SKN_HIP(ctx, allow_big_lds_q8k<3>());
+    SKN_HIP(ctx, allow_big_lds_q8k<4>());
     SKN_HIP(ctx, allow_big_lds_q80<1>());
     SKN_HIP(ctx, allow_big_lds_q80<2>());
     SKN_HIP(ctx, allow_big_lds_q80<3>());
@@ -1534,6 +1640,15 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         return dispatch_runs<kRunsQ2K>(ctx, w, n, nb, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q3_K && nb <= 64 && ctx->opt_matvec_stage == 1)
         return dispatch_runs<kRunsQ3K>(ctx, w, n, nb, x_dev, y_dev);
+    // Q8_K: the Q8_0 arithmetic on the Q4_K lane map (blocks are 4-byte aligned)
+    if (ggml_type == SKN_TYPE_Q8_K && ((uintptr_t)w_dev & 3) == 0 && nb <= 64 && ctx->opt_matvec_stage == 1) {
+        switch ((nb + 15) / 16) {
+            case 1: return launch_q8k<1>(ctx, w, n, nb, x_dev, y_dev);
+            case 2: return launch_q8k<2>(ctx, w, n, nb, x_dev, y_dev);
+            case 3: return launch_q8k<3>(ctx, w, n, nb, x_dev, y_dev);
+            default: return launch_q8k<4>(ctx, w, n, nb, x_dev, y_dev);
+        }
+    }
     if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;

@@ -87,13 +87,13 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"),
-                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k")])
+                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
     eight small blocks, each), a partial last step, the rolled loop beyond four steps, the longest row the kernel
-    takes (144 superblocks) and one past it (direct kernel).  Q2_K and Q3_K (the Q6_K kernel's lane map): one to four
-    steps, then the kernels for longer rows."""
+    takes (144 superblocks) and one past it (direct kernel).  Q2_K and Q3_K (the Q6_K kernel's lane map) and Q8_K: one
+    to four steps, then the kernels for longer rows."""
     raw = synth.weight(qtype, n, k, seed=n + k)
     x = synth.activation_f32(k, seed=k + 3)
     got = hip.matvec_q_host(qtype, raw, n, k, x)
@@ -248,6 +248,30 @@ def test_q3k_matvec_fields_alone(hip):
         variants.append(v)
     for v in variants:
         _against_oracle(hip, 11, v, n, k, x)
+
+
+def test_q8k_matvec_ignores_the_block_sums(hip):
+    """Q8_K (f32 d @0, int8 qs[256] @4, int16 sums @260) on the lane-map kernel: the stored sums of sixteen are not part
+    of the values (random bytes there change nothing); each quarter of a superblock alone; the extreme quants."""
+    n, k = 16, 4096
+    rng = np.random.default_rng(9)
+    raw = synth.weight(15, n, k, seed=51).reshape(n, k // 256, 292).copy()
+    x = synth.activation_f32(k, seed=52)
+    base = hip.matvec_q_host(15, raw.reshape(n, -1), n, k, x)
+    _against_oracle(hip, 15, raw, n, k, x)
+    v = raw.copy()
+    v[:, :, 260:] = rng.integers(0, 256, size=(n, k // 256, 32), dtype=np.uint8)
+    assert np.array_equal(hip.matvec_q_host(15, v.reshape(n, -1), n, k, x), base)
+    for quarter in range(4):
+        v = raw.copy()
+        keep = np.zeros(256, bool)
+        keep[64 * quarter:64 * quarter + 64] = True
+        v[:, :, 4:260][:, :, ~keep] = 0
+        _against_oracle(hip, 15, v, n, k, x)
+    for fill in (0x80, 0x7F):  # -128 and 127 everywhere
+        v = raw.copy()
+        v[:, :, 4:260] = fill
+        _against_oracle(hip, 15, v, n, k, x)
 
 
 def test_iq4_xs_matvec_fields_alone(hip):
