@@ -103,12 +103,13 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel; a captured
  * step is dropped and captured again after any change of an option or of the stream),
  * "llama.fused" (1 = fused per-layer kernels in the decode step, the default: for every group of matrices whose
- * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0), "llama.expand_weights" (1 = the prompt pass of a decoder keeps an expanded
+ * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K), "llama.expand_weights" (1 = the prompt pass of a decoder keeps an expanded
  * copy, see skn_gemm_expand, of every layer matrix that is not Q4_K, made at the first prompt: 4 bytes per weight of
  * device memory on top of the blocks; 0 = the default, expand per call), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
- * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL, rows staged through LDS for the other
- * formats with 4-byte-multiple blocks; 2 = staged rows for all of those; 0 = direct reads).  The knobs exist for
+ * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / Q8_K, the Q6_K kernel's for
+ * Q2_K / Q3_K, rows staged through LDS for what is left with 4-byte-multiple blocks; 2 = staged rows for all
+ * formats with such blocks; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
 /* Counters of a context, for tests and reports: "launches" (kernel launches issued or recorded into a graph so far),

@@ -169,6 +169,7 @@ struct Q5kLoads : Q4kLoads {
 // to bit 1, which is the form q5k_dot_dword takes.
 constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5, kFmtIQ4NL = 8, kFmtIQ4XS = 9;
 constexpr int kFmtQ6K = 6, kFmtQ80 = 7;  // (fused kernels only: the lane maps, staging and steps of matvec_q6k_kernel / matvec_q80_pairs_kernel)
+constexpr int kFmtQ2K = 10, kFmtQ3K = 11, kFmtQ8K = 12;  // (fused kernels only: those of matvec_runs_kernel / matvec_q8k_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
@@ -1148,15 +1149,19 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                                                                float* __restrict__ y, int n_out, int nb,
                                                                skn_rope_epilogue rope) {
     constexpr int R = 2;
-    constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, Q8 = F == kFmtQ80, kSmall = F >= kFmtQ40 && !Q6 && !Q8;
-    using Loads = std::conditional_t<Q8, Q80Loads, std::conditional_t<Q6, Q6kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>;
+    constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, Q8 = F == kFmtQ80, Q2 = F == kFmtQ2K, Q3 = F == kFmtQ3K, Q8K = F == kFmtQ8K;
+    constexpr bool kRuns = Q6 || Q2 || Q3;  // the Q6_K lane map: four runs of sixteen per lane, a float4 of run sums
+    constexpr bool kXS = F == kFmtIQ4XS;
+    constexpr bool kSmall = F >= kFmtQ40 && F <= kFmtIQ4XS && !Q6 && !Q8;
+    using Loads = std::conditional_t<Q8, Q80Loads, std::conditional_t<Q6, Q6kLoads, std::conditional_t<Q2, Q2kLoads, std::conditional_t<Q3, Q3kLoads,
+                  std::conditional_t<Q8K, Q8kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>>>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
     constexpr int kSmallBytes = (F == kFmtQ40 || F == kFmtIQ4NL) ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
-    constexpr bool kPlainX = F == kFmtIQ4NL;  // x staged unscaled, block sums times 128, results in true units
+    constexpr bool kPlainX = F == kFmtIQ4NL || kXS;  // x staged unscaled, block sums times 128, results in true units
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
     float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);
-    float* red = ss + STEPS * (Q6 ? 256 : 128);  // eight partial sums of x^2 (all LDS here is dynamic)
+    float* red = ss + STEPS * (kRuns ? 256 : 128);  // eight partial sums of x^2 (all LDS here is dynamic)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int sub = lane >> 2, p = lane & 3;
     const int n4 = nb * 64;
@@ -1179,7 +1184,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int unit = blockIdx.x * 8 + wave;
     const uint8_t* rowp[R];
     bool row_ok[R];
-    const size_t row_bytes = (size_t)nb * (Q8 ? 272 : Q6 ? 210 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
+    const size_t row_bytes = (size_t)nb * (Q8 ? 272 : Q6 ? 210 : Q2 ? 84 : Q3 ? 110 : Q8K ? 292 : kXS ? 136 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
     if (EPI == SKN_EPI_SWIGLU) {
         const int i = min(unit, n_out - 1);
         row_ok[0] = row_ok[1] = unit < n_out;
@@ -1223,6 +1228,26 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                 L[s][r].h = *reinterpret_cast<const u32x4_a2*>(bp + 128 + 32 * n + 16 * hsel);
                 L[s][r].sc = *reinterpret_cast<const u32x2_a2*>(bp + 192 + 8 * n);
                 L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 208);
+            } else if constexpr (Q2) {
+                const int n = p >> 1, hsel = p & 1;
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 84;
+                L[s][r].q = *reinterpret_cast<const u32x4_a4*>(bp + 16 + 32 * n + 16 * hsel);
+                L[s][r].sc = *reinterpret_cast<const u32x2_a4*>(bp + 8 * n);
+                L[s][r].dd = *reinterpret_cast<const uint32_t*>(bp + 80);
+            } else if constexpr (Q3) {
+                const int n = p >> 1, hsel = p & 1;
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 110;
+                L[s][r].q = *reinterpret_cast<const u32x4_a2*>(bp + 32 + 32 * n + 16 * hsel);
+                L[s][r].hm = *reinterpret_cast<const u32x4_a2*>(bp + 16 * hsel);
+                L[s][r].sc = *reinterpret_cast<const u32x3_a2*>(bp + 96);
+                L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 108);
+            } else if constexpr (Q8K) {
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 292;
+#pragma unroll
+                for (int i = 0; i < 4; i++) L[s][r].w[i] = reinterpret_cast<const u32x4_a4*>(bp + 4 + 64 * p)[i];
+                L[s][r].d = *reinterpret_cast<const float*>(bp);
+            } else if constexpr (kXS) {
+                iq4xs_load(rowp[r] + (size_t)min(blk, nb - 1) * 136 + tie, p, L[s][r]);
             } else if constexpr (kSmall) {
                 const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) * 8 + 2 * p) * kSmallBytes + tie;
                 q4x_load<F>(bp, L[s][r]);
@@ -1261,11 +1286,11 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
     }
-    if constexpr (Q8) {
+    if constexpr (Q8 || Q8K) {
         q4k_stage_store<J, false>(st, n4, tid, 512, xs, ss);
-    } else if constexpr (Q6) {
+    } else if constexpr (kRuns) {
 #pragma unroll
-        for (int jj = 0; jj < J; jj++) q6k_stage_store_one(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
+        for (int jj = 0; jj < J; jj++) q6k_stage_store_one<Q6 ? 32 : Q3 ? 4 : 1>(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
     } else {
         q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, 512, xs, ss);
     }
@@ -1287,12 +1312,15 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         if (s + 1 < STEPS) issue(s + 1, tie);
         asm volatile("" ::: "memory");
         if constexpr (Q8) q80_step<R>(L[s], xs, ss, s, lane + tie, acc);
+        else if constexpr (Q8K) q8k_step<R>(L[s], xs, ss, s, lane + tie, acc);
         else if constexpr (Q6) q6k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
+        else if constexpr (Q2) q2k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
+        else if constexpr (Q3) q3k_step<R>(L[s], xs, ss, s, lane + tie, p >> 1, p & 1, acc);
         else if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
         else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
-    const float back = (Q8 || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
+    const float back = (Q8 || Q8K || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
     const float t0 = wave_sum(acc[0]) * back;
     const float t1 = wave_sum(acc[1]) * back;
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
@@ -1301,7 +1329,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
 template <int STEPS, int EPI, bool NORM, int F>
 int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
                      float eps, float* y, const skn_rope_epilogue& rope) {
-    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * (F == kFmtQ6K ? sizeof(float4) : sizeof(float2))) + 8 * sizeof(float);
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * ((F == kFmtQ6K || F == kFmtQ2K || F == kFmtQ3K) ? sizeof(float4) : sizeof(float2))) + 8 * sizeof(float);
     const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
     dim3 grid((unsigned)((units + 7) / 8)), block(512);
     skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM, F>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
@@ -1504,6 +1532,10 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_ALLOW_FUSED(kFmtQ6K);
     SKN_ALLOW_FUSED(kFmtQ80);
     SKN_ALLOW_FUSED(kFmtIQ4NL);
+    SKN_ALLOW_FUSED(kFmtIQ4XS);
+    SKN_ALLOW_FUSED(kFmtQ2K);
+    SKN_ALLOW_FUSED(kFmtQ3K);
+    SKN_ALLOW_FUSED(kFmtQ8K);
 #undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
@@ -1511,7 +1543,8 @@ int skn_matvec_init(skn_ctx* ctx) {
 bool skn_matvec_fusable(int ggml_type) {
     return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
            ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
-           ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_IQ4_NL;
+           ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_IQ4_NL ||
+           ggml_type == SKN_TYPE_IQ4_XS || ggml_type == SKN_TYPE_Q2_K || ggml_type == SKN_TYPE_Q3_K || ggml_type == SKN_TYPE_Q8_K;
 }
 
 // Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
@@ -1520,7 +1553,9 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
                          float eps, float* y, int epi, const skn_rope_epilogue* rope_in, int ggml_type) {
     SKN_REQUIRE(ctx, skn_matvec_fusable(ggml_type), SKN_ERR_TYPE, "fused matvec: ggml type %d has no fused kernel", ggml_type);
     {
-        const uintptr_t mask = ggml_type == SKN_TYPE_Q6_K ? 1 : ggml_type == SKN_TYPE_Q8_0 ? 3 : 15;
+        const uintptr_t mask = (ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q3_K) ? 1
+                               : (ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_Q2_K || ggml_type == SKN_TYPE_Q8_K) ? 3
+                               : ggml_type == SKN_TYPE_IQ4_XS ? 7 : 15;
         for (int i = 0; i < 3; i++)
             SKN_REQUIRE(ctx, seg.rows[i] == 0 || (seg.w[i] && ((uintptr_t)seg.w[i] & mask) == 0), SKN_ERR_ARG,
                         "fused matvec: weights of type %d must be %d-byte aligned", ggml_type, (int)mask + 1);
@@ -1555,6 +1590,10 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         case SKN_TYPE_Q6_K: SKN_FUSED(kFmtQ6K)
         case SKN_TYPE_Q8_0: SKN_FUSED(kFmtQ80)
         case SKN_TYPE_IQ4_NL: SKN_FUSED(kFmtIQ4NL)
+        case SKN_TYPE_IQ4_XS: SKN_FUSED(kFmtIQ4XS)
+        case SKN_TYPE_Q2_K: SKN_FUSED(kFmtQ2K)
+        case SKN_TYPE_Q3_K: SKN_FUSED(kFmtQ3K)
+        case SKN_TYPE_Q8_K: SKN_FUSED(kFmtQ8K)
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED

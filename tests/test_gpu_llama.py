@@ -389,7 +389,7 @@ def _decode_against_oracle(hip, cfg, w, n_steps, modes=(1, 0), tol=TOL):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (14, "q6_k"),
-                                        (8, "q8_0"), (20, "iq4_nl")])
+                                        (8, "q8_0"), (20, "iq4_nl"), (10, "q2_k")])
 @pytest.mark.parametrize("group", ["qkv", "o", "gu", "down"])
 def test_fused_groups_of_further_formats(hip, qtype, name, group):
     """The fused decode kernels take Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, Q6_K and Q8_0 as well: one group of matrices at a time in
@@ -421,7 +421,7 @@ def test_fused_groups_of_further_formats(hip, qtype, name, group):
 
 
 @pytest.mark.parametrize("qtype,name", [(12, "q4_k"), (13, "q5_k"), (2, "q4_0"), (6, "q5_0"), (14, "q6_k"), (8, "q8_0"),
-                                        (20, "iq4_nl")])
+                                        (20, "iq4_nl"), (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k")])
 @pytest.mark.parametrize("ffn", [8192, 11008, 14336])
 def test_fused_down_projection_of_two_to_four_steps(hip, qtype, name, ffn):
     """Rows of 8192, 11008 and 14336 weights take two, three and four unrolled steps of the fused kernel (4096
@@ -444,10 +444,10 @@ def test_fused_groups_of_two_steps(hip, group, qtype):
     _decode_against_oracle(hip, cfg, w, 3)
 
 
-@pytest.mark.parametrize("tq,tk,tv", [(12, 12, 14), (13, 2, 14), (14, 12, 12), (12, 8, 14), (12, 10, 12)])
+@pytest.mark.parametrize("tq,tk,tv", [(12, 12, 14), (13, 2, 14), (14, 12, 12), (12, 8, 14), (12, 10, 12), (12, 35, 12)])
 def test_qkv_of_mixed_formats(hip, tq, tk, tv):
     """q, k and v of different formats (value projections with more bits, as mixed quantizations have them): one
-    fused launch per format, each carrying the rows of its matrices only; a format without a fused kernel (Q2_K)
+    fused launch per format, each carrying the rows of its matrices only; a format without a fused kernel (TQ2_0)
     sends the group to the separate kernels.  Layer 1 keeps Q4_K; down projections Q6_K as in such files."""
     cfg = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=2, head_dim=128, vocab=512, max_tokens=64,
                        page_tokens=16, matrix_types={"l0.wq": tq, "l0.wk": tk, "l0.wv": tv, "l0.w_down": 14})
