@@ -252,7 +252,8 @@ typedef struct skn_llama_weights {
 } skn_llama_weights;
 
 /* The module graph the reference would express as nested Module.forward calls (core/.../nn/Module.kt:6-16,
- * core/.../nn/topology/MLP.kt:13-19) for a Llama block stack; weights stay owned by the caller. */
+ * core/.../nn/topology/MLP.kt:13-19) for a Llama block stack; weights stay owned by the caller.  Every layer matrix and
+ * norm vector must be 16-byte aligned on the device (what skn_malloc returns is). */
 int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_weights* w, skn_llama** out);
 int skn_llama_free(skn_ctx* ctx, skn_llama* m);
 int skn_llama_reset(skn_ctx* ctx, skn_llama* m);

@@ -483,6 +483,10 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
                     skn_is_quant(L.type_q) && skn_is_quant(L.type_k) && skn_is_quant(L.type_v) && skn_is_quant(L.type_o) &&
                         skn_is_quant(L.type_gate) && skn_is_quant(L.type_up) && skn_is_quant(L.type_down),
                     SKN_ERR_TYPE, "skn_llama_create: layer %d has an unsupported weight type", l);
+        // (the fused kernels and the GEMMs read 16-byte vectors from these)
+        const uintptr_t all = (uintptr_t)L.wq | (uintptr_t)L.wk | (uintptr_t)L.wv | (uintptr_t)L.wo | (uintptr_t)L.w_gate |
+                              (uintptr_t)L.w_up | (uintptr_t)L.w_down | (uintptr_t)L.attn_norm | (uintptr_t)L.ffn_norm;
+        SKN_REQUIRE(ctx, (all & 15) == 0, SKN_ERR_ARG, "skn_llama_create: the weights of layer %d must be 16-byte aligned", l);
     }
     skn_llama* m = new (std::nothrow) skn_llama();
     SKN_REQUIRE(ctx, m != nullptr, SKN_ERR_OOM, "skn_llama_create: host allocation failed");

@@ -520,3 +520,16 @@ def test_llama_argument_errors(hip):
     with pytest.raises(runtime.SknError) as e:
         llama.LlamaModel(hip, bad, weights=llama.random_weights(bad, seed=1))
     assert e.value.code == runtime.ERR_SHAPE and "must divide" in e.value.message
+    # a layer matrix off the 16-byte grid is refused when the model is made, not when a kernel first reads it
+    import ctypes as C
+    model = llama.LlamaModel(hip, SMALL, weights=w)
+    model._layers[1].wo = model._layers[1].wo + 4
+    wts = llama.LlamaWeights(model.bufs["tok_embd"].ptr, model.bufs["out_norm"].ptr, model.bufs["out_head"].ptr,
+                             w["tok_embd"][0], w["out_head"][0], model._layers)
+    c = llama.LlamaConfig(SMALL.n_layer, SMALL.hidden, SMALL.ffn, SMALL.n_head, SMALL.head_dim, SMALL.vocab, SMALL.max_tokens,
+                          SMALL.page_tokens, SMALL.rope_base, SMALL.rms_eps, SMALL.n_kv_head)
+    h = C.c_void_p()
+    with pytest.raises(runtime.SknError) as e:
+        hip._check(hip.lib.skn_llama_create(hip.handle, C.byref(c), C.byref(wts), C.byref(h)))
+    assert e.value.code == runtime.ERR_ARG and "16-byte aligned" in e.value.message
+    model.free()
