@@ -107,13 +107,17 @@ def test_mixed_matrix_types_match_oracle(hip):
     model.free()
 
 
-def test_prompt_pass_with_kept_expanded_weights(hip):
+@pytest.mark.parametrize("n_kv_head,types", [(4, None), (2, {"l0.wk": 14, "l0.wv": 8, "l1.w_up": 13, "l1.w_down": 14})])
+def test_prompt_pass_with_kept_expanded_weights(hip, n_kv_head, types):
     """llama.expand_weights = 1: the matrices that are not Q4_K keep their fp16-pair copies from the first prompt on and
     the general GEMM takes the fp32 rows itself (norm and bf16 rounding in its activation pass, residual in its
     store).  Same operands and same matrix instructions as the per-call route: the logits agree to the rounding of
     the residual add (one fused multiply-add instead of a multiply and an add), and with the oracle to the usual
     bound; a second prompt reuses the copies."""
-    cfg = MIXED
+    # (the second case: grouped K / V heads with their projections among the expanded matrices, and a gate / up pair
+    # of which only one is Q4_K)
+    cfg = MIXED if types is None else llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=n_kv_head, head_dim=128,
+                                                   vocab=512, max_tokens=96, page_tokens=16, matrix_types=types)
     w = llama.random_weights(cfg, seed=21)
     prompt = np.random.default_rng(2).integers(0, cfg.vocab, size=41).tolist()
     model = llama.LlamaModel(hip, cfg, weights=w)
@@ -126,8 +130,10 @@ def test_prompt_pass_with_kept_expanded_weights(hip):
         assert model.prefill(prompt) == first or not _margin_ok(base, 1e-4 * np.abs(base).max())
         kept = model.logits()
         assert oracle_np.rel_err(kept, base) <= 1e-4
-        # l0: wq, w_down; l1: wo, w_gate -- 4 bytes per weight; the Q4_K matrices beside them keep their own kernel
-        want = 4 * (512 * 512 + 512 * 768 + 512 * 512 + 768 * 512)
+        # 4 bytes per weight of the matrices that are not Q4_K (MIXED: l0 wq, w_down; l1 wo, w_gate); the Q4_K matrices
+        # beside them keep their own kernel
+        kvd = n_kv_head * 128
+        want = 4 * (512 * 512 + 512 * 768 + 512 * 512 + 768 * 512) if types is None else 4 * (2 * kvd * 512 + 768 * 512 + 512 * 768)
         assert hip.stat("llama.expanded_bytes") == want
         model.reset()
         model.prefill(prompt)
