@@ -108,7 +108,7 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * device memory on top of the blocks; 0 = the default, expand per call), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
  * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / Q8_K, the Q6_K kernel's for
- * Q2_K / Q3_K, rows staged through LDS for what is left with 4-byte-multiple blocks; 2 = staged rows for all
+ * Q2_K / Q3_K / TQ2_0, rows staged through LDS for what is left with 4-byte-multiple blocks; 2 = staged rows for all
  * formats with such blocks; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);

@@ -906,8 +906,10 @@ __global__ __launch_bounds__(256) void matvec_q6_k_kernel(const uint8_t* __restr
 //     d.  The three-bit value q | hbit << 2 stands for q - 4 + 4 hbit, so the zero point returns as 4 * sum(x of
 //     the run).  Scale of run j (index is = 8n + 2j + hsel): low four bits in nibble n of byte 2j + hsel, two more
 //     in bits 4n + 2 (j / 2) of byte 8 + (2j + hsel) % 4, stored with an offset of 32.
+//   TQ2_0 (66 bytes: qs[64], f16 d; 2-byte aligned; ternary): the packing of Q2_K's qs with one scale, y = d (q - 1):
+//     sixteen bytes of qs and d; the zero point returns as 1 * sum(x of the run).
 // A byte of two or three bits masked out in pairs (v & 0x00FF00FF) is a pair of fp16 subnormals, as in Q6_K.
-constexpr int kRunsQ2K = 0, kRunsQ3K = 1;
+constexpr int kRunsQ2K = 0, kRunsQ3K = 1, kRunsTQ2 = 2;
 typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
 typedef uint32_t u32x3_a2 __attribute__((ext_vector_type(3), aligned(2)));
 
@@ -964,6 +966,38 @@ __device__ __forceinline__ void q2k_step(const Q2kLoads (&L)[R], const float4* _
     }
 }
 
+struct Tq2Loads {
+    u32x4 q;
+    uint32_t d;
+    bool ok;
+};
+
+template <int R>
+__device__ __forceinline__ void tq2_step(const Tq2Loads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
+                                         int s, int lane, float (&acc)[R]) {
+    float S[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) S[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float4 xq[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) xq[q] = xs[(s * 16 + 4 * q + i) * kXPitch + lane];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint32_t dw = L[r].q[i];
+            S[r] = q6k_dot4(dw & 0x03030303u, xq[0], S[r]);
+            S[r] = q6k_dot4((dw >> 2) & 0x03030303u, xq[1], S[r]);
+            S[r] = q6k_dot4((dw >> 4) & 0x03030303u, xq[2], S[r]);
+            S[r] = q6k_dot4((dw >> 6) & 0x03030303u, xq[3], S[r]);
+        }
+    }
+    const float4 sx = reinterpret_cast<const float4*>(ss)[s * 64 + lane];  // 2^-24 * sums of x over the four runs
+    const float zero = (sx.x + sx.y) + (sx.z + sx.w);
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] += L[r].ok ? h2f_bits(L[r].d) * (S[r] - zero) : 0.f;
+}
+
 template <int R>
 __device__ __forceinline__ void q3k_step(const Q3kLoads (&L)[R], const float4* __restrict__ xs, const float* __restrict__ ss,
                                          int s, int lane, int n, int hsel, float (&acc)[R]) {
@@ -1004,9 +1038,9 @@ __device__ __forceinline__ void q3k_step(const Q3kLoads (&L)[R], const float4* _
 template <int STEPS, int R, int F>
 __global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                           float* __restrict__ y, int n_rows, int nb) {
-    constexpr bool Q2 = F == kRunsQ2K;
-    constexpr int kBlock = Q2 ? 84 : 110;
-    using Loads = std::conditional_t<Q2, Q2kLoads, Q3kLoads>;
+    constexpr bool Q2 = F == kRunsQ2K, T2 = F == kRunsTQ2;
+    constexpr int kBlock = Q2 ? 84 : T2 ? 66 : 110;
+    using Loads = std::conditional_t<Q2, Q2kLoads, std::conditional_t<T2, Tq2Loads, Q3kLoads>>;
     extern __shared__ float4 lds4[];
     float4* xs = lds4;
     float* ss = reinterpret_cast<float*>(lds4 + STEPS * 16 * kXPitch);  // float4 per (step, lane)
@@ -1038,6 +1072,9 @@ __global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restr
                 L[s][r].q = *reinterpret_cast<const u32x4_a4*>(bp + 16 + 32 * n + 16 * hsel);
                 L[s][r].sc = *reinterpret_cast<const u32x2_a4*>(bp + 8 * n);
                 L[s][r].dd = *reinterpret_cast<const uint32_t*>(bp + 80);
+            } else if constexpr (T2) {
+                L[s][r].q = *reinterpret_cast<const u32x4_a2*>(bp + 32 * n + 16 * hsel);
+                L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 64);
             } else {
                 L[s][r].q = *reinterpret_cast<const u32x4_a2*>(bp + 32 + 32 * n + 16 * hsel);
                 L[s][r].hm = *reinterpret_cast<const u32x4_a2*>(bp + 16 * hsel);
@@ -1052,7 +1089,7 @@ __global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restr
     for (int jj = 0; jj < J; jj++) {
         // a float4 index past the end repeats the last one: same data to the same slot
         const int f = min(tid + jj * 512, n4 - 1);
-        q6k_stage_store_one<Q2 ? 1 : 4>(st.v[jj], f, xs, ss);
+        q6k_stage_store_one<(Q2 || T2) ? 1 : 4>(st.v[jj], f, xs, ss);
     }
     __syncthreads();
     int tie = 0;
@@ -1062,6 +1099,7 @@ __global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restr
         if (s + 1 < STEPS) issue(s + 1, tie);
         asm volatile("" ::: "memory");
         if constexpr (Q2) q2k_step<R>(L[s], xs, ss, s, lane + tie, hsel, acc);
+        else if constexpr (T2) tq2_step<R>(L[s], xs, ss, s, lane + tie, acc);
         else q3k_step<R>(L[s], xs, ss, s, lane + tie, n, hsel, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
@@ -1510,6 +1548,10 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsQ3K>()));
     SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsQ3K>()));
     SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsQ3K>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<1, kRunsTQ2>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsTQ2>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsTQ2>()));
+    SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsTQ2>()));
     SKN_HIP(ctx, allow_big_lds_q8k<1>());
     SKN_HIP(ctx, allow_big_lds_q8k<2>());
     SKN_HIP(ctx, allow_big_lds_q8k<3>());
@@ -1679,6 +1721,8 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         return dispatch_runs<kRunsQ2K>(ctx, w, n, nb, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_Q3_K && nb <= 64 && ctx->opt_matvec_stage == 1)
         return dispatch_runs<kRunsQ3K>(ctx, w, n, nb, x_dev, y_dev);
+    if (ggml_type == SKN_TYPE_TQ2_0 && nb <= 64 && ctx->opt_matvec_stage == 1)
+        return dispatch_runs<kRunsTQ2>(ctx, w, n, nb, x_dev, y_dev);
     // Q8_K: the Q8_0 arithmetic on the Q4_K lane map (blocks are 4-byte aligned)
     if (ggml_type == SKN_TYPE_Q8_K && ((uintptr_t)w_dev & 3) == 0 && nb <= 64 && ctx->opt_matvec_stage == 1) {
         switch ((nb + 15) / 16) {

@@ -87,13 +87,13 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"),
-                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k")])
+                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k"), (35, "tq2_0")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
     eight small blocks, each), a partial last step, the rolled loop beyond four steps, the longest row the kernel
     takes (144 superblocks) and one past it (direct kernel).  Q2_K and Q3_K (the Q6_K kernel's lane map) and Q8_K: one
-    to four steps, then the kernels for longer rows."""
+    to four steps, then the kernels for longer rows; TQ2_0 likewise (the packing of Q2_K's quants)."""
     raw = synth.weight(qtype, n, k, seed=n + k)
     x = synth.activation_f32(k, seed=k + 3)
     got = hip.matvec_q_host(qtype, raw, n, k, x)
@@ -248,6 +248,33 @@ def test_q3k_matvec_fields_alone(hip):
         variants.append(v)
     for v in variants:
         _against_oracle(hip, 11, v, n, k, x)
+
+
+def test_tq2_0_matvec_bit_pairs_alone(hip):
+    """TQ2_0 (qs[64] @0, d @64; y = d (q - 1)) on the lane-map kernel: each bit pair alone, each half alone, all quants 2
+    (y = d sum x) and all quants 1 (every weight zero)."""
+    n, k = 16, 4096
+    raw = synth.weight(35, n, k, seed=61).reshape(n, k // 256, 66).copy()
+    x = synth.activation_f32(k, seed=62)
+    variants = [raw]
+    for j in range(4):
+        v = raw.copy()
+        v[:, :, :64] &= 3 << (2 * j)
+        variants.append(v)
+    for half in (0, 1):
+        v = raw.copy()
+        v[:, :, 32 * (1 - half):32 * (1 - half) + 32] = 0x55  # the other half: quants 1, weights 0
+        variants.append(v)
+    v = raw.copy()
+    v[:, :, :64] = 0xAA
+    variants.append(v)
+    for v in variants:
+        _against_oracle(hip, 35, v, n, k, x)
+    # all quants 1: every weight is zero, and what is left of sum(q x) - sum(x) is rounding noise
+    v = raw.copy()
+    v[:, :, :64] = 0x55
+    got = hip.matvec_q_host(35, v.reshape(n, -1), n, k, x)
+    assert np.abs(got).max() <= 1e-5 * np.abs(x).sum() * 0.05
 
 
 def test_q8k_matvec_ignores_the_block_sums(hip):
