@@ -16,6 +16,7 @@ class DeviceTensor internal constructor(
     val ctx: SknContext,
     override val shape: Shape,
     internal val dev: MemorySegment,
+    private val owner: Boolean = true,   // false: a view of another tensor's buffer (a reshape)
 ) : Tensor, AutoCloseable {
 
     companion object {
@@ -38,10 +39,19 @@ class DeviceTensor internal constructor(
 
     /**
      * x.matmul(W.t()) with W a quantized [out, in] weight: rank 1 -> skn_matvec_q (DoublesTensor.kt:255-264 semantics),
-     * rank 2 -> skn_gemm_q on bf16 rows (DoublesTensor.kt:267-279 semantics).  Anything else: the reference's matmul on
-     * host values, including its error messages.
+     * rank 2 -> skn_gemm_q on bf16 rows (DoublesTensor.kt:267-279 semantics); ranks 3 and 4 multiply every [.., in] row
+     * (DoublesTensor.kt:281-357), i.e. the same GEMM with the leading dimensions as its rows.  Anything else: the
+     * reference's matmul on host values, including its error messages.
      */
     override fun matmul(other: Tensor): Tensor {
+        if (other is QuantizedTensor && other.transposed && (rank == 3 || rank == 4)) {
+            val k = shape.dimensions.last()
+            if (k != other.inFeatures) throw IllegalArgumentException("Shapes do not align.")
+            val rows = DeviceTensor(ctx, Shape(shape.volume / k, k), dev, owner = false)
+            val out = rows.matmul(other) as DeviceTensor
+            val lead = shape.dimensions.dropLast(1).toIntArray()
+            return out.reshaped(Shape(*lead, other.outFeatures))  // (out itself is not closed: the result owns its buffer)
+        }
         if (other !is QuantizedTensor || !other.transposed || (rank != 1 && rank != 2)) {
             if (other is QuantizedTensor && (rank == 1 || rank == 2))
                 throw IllegalArgumentException(
@@ -126,5 +136,13 @@ class DeviceTensor internal constructor(
     override fun ln(): Tensor = toDoubles().ln()
     override fun flatten(startDim: Int, endDim: Int): Tensor = toDoubles().flatten(startDim, endDim)
 
-    override fun close() = ctx.free(dev)
+    /** The same buffer under another shape of the same volume; the receiver gives up ownership to the result. */
+    internal fun reshaped(to: Shape): DeviceTensor {
+        require(to.volume == shape.volume) { "a reshape keeps the element count" }
+        return DeviceTensor(ctx, to, dev, owner)
+    }
+
+    override fun close() {
+        if (owner) ctx.free(dev)
+    }
 }

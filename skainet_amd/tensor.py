@@ -122,7 +122,16 @@ class DeviceTensor:
         return self.buf.download(np.float32, self.shape.volume).reshape(self.shape.dimensions)
 
     def matmul(self, other):
-        """x.matmul(W.t()) for a transposed quantized weight: rank 1 -> matvec, rank 2 -> GEMM."""
+        """x.matmul(W.t()) for a transposed quantized weight: rank 1 -> matvec, rank 2 -> GEMM; ranks 3 and 4 multiply
+        every [.., in] row, as the reference does for a 3-D or 4-D tensor times a matrix
+        (core/.../impl/DoublesTensor.kt:281-357; TensorTest.kt:393-538): the leading dimensions are the GEMM's rows."""
+        if isinstance(other, QuantizedTensor) and other.transposed and self.rank in (3, 4):
+            lead = self.shape.dimensions[:-1]
+            if self.shape.dimensions[-1] != other._shape.dimensions[1]:
+                raise ValueError("Shapes do not align.")
+            rows = DeviceTensor(self.ctx, Shape(self.shape.volume // self.shape.dimensions[-1], self.shape.dimensions[-1]), self.buf)
+            out = rows.matmul(other)
+            return DeviceTensor(self.ctx, Shape(*lead, other._shape.dimensions[0]), out.buf)
         if not isinstance(other, QuantizedTensor) or not other.transposed or self.rank not in (1, 2):
             raise ValueError(
                 f"Unsupported tensor shapes for multiplication: {list(self.shape.dimensions)} and "

@@ -54,6 +54,31 @@ def test_reference_matmul_known_answers_through_quantized_weights(hip, golden_di
     assert got.shape == Shape(2, 2) and got.numpy().reshape(-1).tolist() == c["expected"]
 
 
+@pytest.mark.parametrize("case", ["matmulOf3DTensorAnd2DMatrix", "matmulOf4DNCHWTensorAnd2DMatrix"])
+def test_reference_3d_and_4d_inputs_through_the_gemm(hip, golden_dir, case):
+    """TensorTest.kt:393-538: a [3, 2, 4] and a [2, 3, 2, 4] tensor times a [4, 3] matrix -- every row of four times
+    the matrix, the leading dimensions kept.  The rows are small integers (exact in the bf16 the GEMM rounds them to),
+    the matrix 0.1 .. 1.2 as dense F32 weights W = B^T (k padded to the GEMM's 64-element granule): the reference's
+    expected values (it lists the first 18) to fp32 accuracy."""
+    c = json.load(open(os.path.join(golden_dir, "tensor_test_vectors.json")))["cases"][case]
+    x = np.array(c["tensors"][0]["values"]).reshape(c["tensors"][0]["shape"])
+    b = np.array(c["tensors"][1]["values"]).reshape(c["tensors"][1]["shape"])
+    kp = 64
+    wt = np.zeros((b.shape[1], kp), dtype=np.float32)
+    wt[:, : b.shape[0]] = b.T
+    w = QuantizedTensor.from_bytes(hip, synth.F32, b.shape[1], kp, wt.view(np.uint8))
+    xp = np.zeros(x.shape[:-1] + (kp,), dtype=np.float32)
+    xp[..., : x.shape[-1]] = x
+    got = DeviceTensor.from_numpy(hip, xp).matmul(w.t())
+    assert got.shape == Shape(*x.shape[:-1], b.shape[1])
+    want = np.array(c["expected"], dtype=np.float64)
+    flat = got.numpy().reshape(-1).astype(np.float64)
+    assert np.max(np.abs(flat[: want.size] - want) / np.abs(want)) < 1e-6
+    assert np.max(np.abs(flat - (x @ b).reshape(-1)) / np.abs((x @ b).reshape(-1))) < 1e-6
+    with pytest.raises(ValueError, match="Shapes do not align"):
+        DeviceTensor.from_numpy(hip, xp[..., :32]).matmul(w.t())
+
+
 def test_reference_1x16_times_16x16_through_the_matvec(hip, golden_dir):
     """TensorTest.kt:72-391: the 1x16 row times the 16x16 matrix, expected row within 1e-4 -- as Linear computes it,
     x.matmul(W.t()) with W = B^T held as dense F32 rows on the device."""
