@@ -195,6 +195,47 @@ def bench_gemm(ctx, qtype, m, n, k, reps=20, expanded=False):
             "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
+def matvec_timeline(ctx, n, k, reps=20, queued=12):
+    """In-kernel timeline of the headline kernel (its measuring build, skn_test_matvec_q4k_stamps): `queued` launches back
+    to back over rotating weight copies, the stamps of the last one; percentiles over its wavefronts, averaged over
+    `reps` such launches.  Times in microseconds after the first wavefront of the launch started (100 MHz clock)."""
+    ws = [ctx.to_device(synth.weight(Q4_K, n, k, seed=1234 + c)) for c in range(N_COPIES)]
+    x = ctx.to_device(synth.activation_f32(k, seed=5))
+    y = ctx.alloc(4 * n)
+    stamps = ctx.alloc(8 * 8 * n)
+    names = ["wavefront starts", "x and step-0 weights requested", "x stored to LDS", "barrier passed", "step 0 done",
+             "step 1 done", "step 2 done"]
+    acc = np.zeros((7, 5))
+    end_by_block = np.zeros(n // 8)
+    end_by_xcc = {}
+    for r in range(reps):
+        for j in range(queued):
+            ctx.test_matvec_q4k_stamps(ws[(r * queued + j) % N_COPIES], n, k, x, y, stamps)
+        ctx.sync()
+        t = stamps.download(np.uint64, 8 * n).reshape(n, 8)
+        rel = (t[:, :7] - t[:, 0].min()).astype(np.float64) * 0.01
+        for e in range(7):
+            v = np.sort(rel[:, e])
+            acc[e] += [v[0], v[n // 10], v[n // 2], v[n * 9 // 10], v[-1]]
+        end_by_block += rel[:, 6].reshape(n // 8, 8).mean(axis=1)
+        xcc = (t[:, 7] >> np.uint64(32)).astype(np.int64) & 7
+        for q in range(8):
+            if np.any(xcc == q):
+                end_by_xcc.setdefault(q, []).append(float(rel[xcc == q, 6].mean()))
+    acc /= reps
+    end_by_block /= reps
+    half = (n // 8) // 2
+    out = {"mode": "timeline", "workload": f"Q4_K matvec N={n} K={k}", "wavefronts": n, "launches_averaged": reps,
+           "queued_back_to_back": queued, "columns": ["min", "p10", "median", "p90", "max"],
+           "events_us": {names[e]: [round(float(a), 2) for a in acc[e]] for e in range(7)},
+           "mean_end_us_first_half_of_workgroups": round(float(end_by_block[:half].mean()), 2),
+           "mean_end_us_second_half_of_workgroups": round(float(end_by_block[half:].mean()), 2),
+           "mean_end_us_by_xcd": {str(q): round(float(np.mean(v)), 2) for q, v in sorted(end_by_xcc.items())}}
+    for b in ws + [x, y, stamps]:
+        b.free()
+    return out
+
+
 def gemm_expanded_rows(ctx):
     """The Q6_K shapes of the GEMM leg with their expanded weights kept between calls."""
     return {f"q6_k_expanded_{mm}x{nn}x{kk}": bench_gemm(ctx, Q6_K, mm, nn, kk, expanded=True)
@@ -304,8 +345,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats"], default="bench",
-                    help="decode / attention / gemm: only that leg (for kernel traces).  copy: run --steps plain device copies of the headline weight size instead (the known-size "
+    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline"], default="bench",
+                    help="decode / attention / gemm: only that leg (for kernel traces).  timeline: the headline kernel's in-kernel time stamps.  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode without the captured step graph (kernel tracers that cannot follow graph launches)")
@@ -319,6 +360,10 @@ def main():
     if args.no_graph:
         ctx.set_option("llama.graph", 0)
     n, k = 4096, 11008
+    if args.mode == "timeline":
+        print(json.dumps(matvec_timeline(ctx, n, k)))
+        ctx.close()
+        return
     if args.mode == "copy":
         nbytes = n * (k // 256) * 144
         srcs = [ctx.to_device(synth.weight(Q4_K, n, k, seed=1234 + c)) for c in range(N_COPIES)]

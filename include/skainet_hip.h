@@ -273,10 +273,18 @@ int skn_llama_logits(skn_ctx* ctx, skn_llama* m, const float** logits_dev);
  * (norm_w_dev, eps), and an epilogue: 0 store y, 1 y +=, 2 y[i] = silu(w0 row i . x) * (w1 row i . x), 3 rotary
  * embedding of q (rows0, to y as fp32) and k (rows1) with k and v (rows2) stored as fp16 at the end of sequence 0 of the
  * one-sequence cache `kv` (its position is written to *pos_dev, a device int the caller provides).  No reference
- * counterpart.  Types: Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, Q6_K, Q8_0; k a multiple of 256, at most 16384. */
+ * counterpart.  Types: Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K; k a multiple of 256,
+ * at most 16384. */
 int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const void* w0, int rows0, const void* w1, int rows1,
                           const void* w2, int rows2, int k, const float* x_dev, const float* norm_w_dev, float eps,
                           float* y_dev, skn_kv* kv, int32_t* pos_dev, float rope_base);
+/* The Q4_K matvec of skn_matvec_q for a row of three steps (8192 < k <= 12288, one row per wavefront) run with the
+ * kernel's measuring build: y as usual, and eight 64-bit words per row (= per wavefront) in stamps_dev -- the 100 MHz
+ * wall clock at the wavefront's start, after its first requests are issued, after its stores of x, after the
+ * barrier, after each of the three steps, and (XCC_ID << 32 | HW_ID).  For `bench.py --mode timeline`.  No
+ * reference counterpart. */
+int skn_test_matvec_q4k_stamps(skn_ctx* ctx, const void* w_dev, int n, int k, const float* x_dev, float* y_dev,
+                               uint64_t* stamps_dev);
 
 #ifdef __cplusplus
 }

@@ -366,9 +366,17 @@ __device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restr
 // x stores (and with them every wavefront at the barrier) would sit behind the issue of a whole row.
 // F: Q4_K; Q5_K blocks (eleven chunks, the quants from the fourth on) with the same lane map, staging and scales;
 // Q4_0 / Q4_1, eight blocks for a superblock (nb counts groups of eight).
-template <int STEPS, int R, int F = kFmtQ4K>
+// TS: a measuring build (skn_test_matvec_q4k_stamps).  Every wavefront records the wall clock (100 MHz) at its start,
+// after its first requests are issued, after its x stores, after the barrier and after each step, plus its hardware
+// ids, into the buffer g_matvec_stamps points at: eight 64-bit words per wavefront.  The shipped instantiations have
+// TS = false and contain none of it.
+__device__ unsigned long long* g_matvec_stamps = nullptr;
+
+template <int STEPS, int R, int F = kFmtQ4K, bool TS = false>
 __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                                          float* __restrict__ y, int n_rows, int nb) {
+    unsigned long long ts[8] = {};
+    if constexpr (TS) ts[0] = wall_clock64();
     constexpr bool Q5 = F == kFmtQ5K, kSmall = F >= kFmtQ40, kXS = F == kFmtIQ4XS;
     using Loads = std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;  // chunks per block, first chunk of quants
@@ -436,8 +444,17 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     if constexpr (STEPS > 0) {
         Loads L[STEPS][R];
         issue(0, 0, L[0]);
+        if constexpr (TS) {
+            asm volatile("" ::: "memory");
+            ts[1] = wall_clock64();
+        }
         q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, blockDim.x, xs, ss);
+        if constexpr (TS) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            ts[2] = wall_clock64();
+        }
         __syncthreads();
+        if constexpr (TS) ts[3] = wall_clock64();
         // `tie` is always 0; an empty asm after each step makes it look rewritten from the finished accumulator,
         // which pins the loads of step s+1 between the arithmetic of steps s-1 and s (one step of lookahead) and
         // the LDS reads of step s below the arithmetic of step s-1 (bounded registers)
@@ -449,6 +466,15 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
             asm volatile("" ::: "memory");  // the loads above stay above the LDS reads below
             step(L[s], s, lane + tie);
             asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+            if constexpr (TS && STEPS <= 3) ts[4 + s] = wall_clock64();
+        }
+        if constexpr (TS) {
+            // hardware ids: HW_ID (wave, SIMD, compute unit, shader array, shader engine) and XCC_ID
+            ts[7] = ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32) | (unsigned)__builtin_amdgcn_s_getreg(63492);
+            if (lane == 0 && g_matvec_stamps) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) g_matvec_stamps[(size_t)(blockIdx.x * waves + wave) * 8 + i] = ts[i];
+            }
         }
     } else {
         Loads bufa[R], bufb[R];
@@ -1674,6 +1700,32 @@ extern "C" int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const
     rc = skn_matvec_q4k_fused(ctx, seg, n_out, k, x_dev, norm_w_dev, eps, y_dev, SKN_EPI_ROPE, &rope, ggml_type);
     if (rc != SKN_OK) return rc;
     return skn_kv_advance_len(ctx, kv, 0, 1);
+}
+
+// Test / measurement hook: the Q4_K matvec of a three-step row (8192 < k <= 12288) with the kernel's measuring build.
+extern "C" int skn_test_matvec_q4k_stamps(skn_ctx* ctx, const void* w_dev, int n, int k, const float* x_dev, float* y_dev,
+                                          uint64_t* stamps_dev) {
+    SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_test_matvec_q4k_stamps: ctx is null");
+    SKN_REQUIRE(ctx, w_dev && x_dev && y_dev && stamps_dev, SKN_ERR_ARG, "skn_test_matvec_q4k_stamps: null pointer");
+    SKN_REQUIRE(ctx, n > 0 && k % 256 == 0 && k > 8192 && k <= 12288, SKN_ERR_SHAPE,
+                "skn_test_matvec_q4k_stamps: k (%d) must be a multiple of 256 in (8192, 12288]", k);
+    SKN_REQUIRE(ctx, (((uintptr_t)w_dev | (uintptr_t)x_dev) & 15) == 0 && ((uintptr_t)stamps_dev & 7) == 0, SKN_ERR_ARG,
+                "skn_test_matvec_q4k_stamps: misaligned pointer");
+    auto kern = matvec_q4k_kernel<3, 1, kFmtQ4K, true>;
+    static bool lds_allowed[64] = {};
+    int dev = 0;
+    SKN_HIP(ctx, hipGetDevice(&dev));
+    if (dev >= 0 && dev < 64 && !lds_allowed[dev]) {
+        SKN_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        lds_allowed[dev] = true;
+    }
+    unsigned long long* p = reinterpret_cast<unsigned long long*>(stamps_dev);
+    SKN_HIP(ctx, hipMemcpyToSymbolAsync(HIP_SYMBOL(g_matvec_stamps), &p, sizeof(p), 0, hipMemcpyHostToDevice, ctx->stream));
+    const int nb = k / 256;
+    const size_t lds = (size_t)3 * (16 * kXPitch * sizeof(float4) + 64 * sizeof(float2));
+    skn_launch(ctx, kern, dim3((unsigned)((n + 7) / 8)), dim3(512), lds, (const uint8_t*)w_dev, x_dev, y_dev, n, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
 }
 
 extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n, int k, const float* x_dev,

@@ -86,6 +86,7 @@ _SIGNATURES = {
     "skn_gemm_expanded_bytes": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t)]),
     "skn_gemm_expand": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "skn_gemm_expanded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
+    "skn_test_matvec_q4k_stamps": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "skn_kv_create": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "skn_kv_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_kv_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -367,6 +368,10 @@ class Context:
 
     def gemm_expanded(self, expanded_dev, n, k, a_bf16_dev, m, c_dev):
         self._check(self.lib.skn_gemm_expanded(self.handle, _ptr(expanded_dev), n, k, _ptr(a_bf16_dev), m, _ptr(c_dev)))
+
+    def test_matvec_q4k_stamps(self, w_dev, n, k, x_dev, y_dev, stamps_dev):
+        """The Q4_K matvec with the kernel's measuring build: eight 64-bit stamps per row in stamps_dev."""
+        self._check(self.lib.skn_test_matvec_q4k_stamps(self.handle, _ptr(w_dev), n, k, _ptr(x_dev), _ptr(y_dev), _ptr(stamps_dev)))
 
     def rmsnorm(self, x_dev, w_dev, rows, n, eps, y_dev):
         self._check(self.lib.skn_rmsnorm(self.handle, _ptr(x_dev), _ptr(w_dev), rows, n, eps, _ptr(y_dev)))
