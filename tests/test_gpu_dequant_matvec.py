@@ -178,3 +178,22 @@ def test_matvec_errors_and_empty(hip):
     y = hip.to_device(np.ones(4, dtype=np.float32))
     hip.matvec_q(Q4_K, buf, 4, 0, buf, y)  # k = 0: the empty sum
     assert np.all(y.download(np.float32, 4) == 0.0)
+
+
+def test_measuring_build_of_the_q4k_matvec(hip):
+    """skn_test_matvec_q4k_stamps (what `bench.py --mode timeline` runs): the same result as skn_matvec_q bit for bit, and
+    per wavefront seven clock readings in program order plus its hardware ids."""
+    n, k = 72, 11008
+    raw = synth.weight(Q4_K, n, k, seed=91)
+    x = synth.activation_f32(k, seed=92)
+    w, xd, y, stamps = hip.to_device(raw), hip.to_device(x), hip.alloc(4 * n), hip.alloc(64 * n)
+    hip.test_matvec_q4k_stamps(w, n, k, xd, y, stamps)
+    got = y.download(np.float32, n)
+    assert np.array_equal(got.view(np.uint32), hip.matvec_q_host(Q4_K, raw, n, k, x).view(np.uint32))
+    t = stamps.download(np.uint64, 8 * n).reshape(n, 8)
+    assert np.all(t[:, 0] > 0) and np.all(np.diff(t[:, :7].astype(np.int64), axis=1) >= 0)
+    assert np.all((t[:, 7] >> np.uint64(32)) < 8)  # XCC_ID
+    with pytest.raises(runtime.SknError, match="multiple of 256 in"):
+        hip.test_matvec_q4k_stamps(w, n, 4096, xd, y, stamps)
+    for b in (w, xd, y, stamps):
+        b.free()
