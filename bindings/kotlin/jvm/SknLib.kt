@@ -86,6 +86,8 @@ object SknLib {
     val llamaLogits: MethodHandle = h("skn_llama_logits", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
     val testFusedMatvec: MethodHandle = h("skn_test_fused_matvec", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, JAVA_FLOAT, ADDRESS, ADDRESS, ADDRESS, JAVA_FLOAT))
     val testMatvecQ4kStamps: MethodHandle = h("skn_test_matvec_q4k_stamps", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
+    val testMfmaValuOverlap: MethodHandle = h("skn_test_mfma_valu_overlap", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS))
+    val testFragmentDelivery: MethodHandle = h("skn_test_fragment_delivery", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, ADDRESS))
 
     init {
         val v = abiVersion.invokeExact() as Int

@@ -285,6 +285,16 @@ int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const void* w0, 
  * reference counterpart. */
 int skn_test_matvec_q4k_stamps(skn_ctx* ctx, const void* w_dev, int n, int k, const float* x_dev, float* y_dev,
                                uint64_t* stamps_dev);
+/* Two measurements of the machine that the kernel designs lean on (`bench.py --mode machine`); no reference
+ * counterpart.  (1) Nanoseconds per v_mfma_f32_32x32x16_f16 and SIMD when every matrix instruction is followed by
+ * valu_per_mfma (0, 2, 4, 6, 7, 8 or 12) independent vector instructions, at one or two wavefronts per SIMD;
+ * scratch_dev: 512 KiB of device memory.  (2) GB/s per compute unit at which 1 KiB operand fragments (one 16-byte load
+ * per lane, eight in flight per wavefront, eight wavefronts per compute unit) arrive in registers when `share` (1, 2, 4
+ * or 8) wavefronts of a workgroup read the same fragments; data_dev: data_mib MiB of device memory, flag_dev: one
+ * device word. */
+int skn_test_mfma_valu_overlap(skn_ctx* ctx, int waves_per_simd, int valu_per_mfma, float* scratch_dev, double* ns_out);
+int skn_test_fragment_delivery(skn_ctx* ctx, int share, const void* data_dev, int data_mib, unsigned* flag_dev,
+                               double* gbs_out);
 
 #ifdef __cplusplus
 }

@@ -87,6 +87,8 @@ _SIGNATURES = {
     "skn_gemm_expand": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "skn_gemm_expanded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
     "skn_test_matvec_q4k_stamps": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "skn_test_mfma_valu_overlap": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
+    "skn_test_fragment_delivery": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
     "skn_kv_create": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "skn_kv_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_kv_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -372,6 +374,16 @@ class Context:
     def test_matvec_q4k_stamps(self, w_dev, n, k, x_dev, y_dev, stamps_dev):
         """The Q4_K matvec with the kernel's measuring build: eight 64-bit stamps per row in stamps_dev."""
         self._check(self.lib.skn_test_matvec_q4k_stamps(self.handle, _ptr(w_dev), n, k, _ptr(x_dev), _ptr(y_dev), _ptr(stamps_dev)))
+
+    def test_mfma_valu_overlap(self, waves_per_simd, valu_per_mfma, scratch_dev):
+        out = C.c_double()
+        self._check(self.lib.skn_test_mfma_valu_overlap(self.handle, waves_per_simd, valu_per_mfma, _ptr(scratch_dev), C.byref(out)))
+        return out.value
+
+    def test_fragment_delivery(self, share, data_dev, data_mib, flag_dev):
+        out = C.c_double()
+        self._check(self.lib.skn_test_fragment_delivery(self.handle, share, _ptr(data_dev), data_mib, _ptr(flag_dev), C.byref(out)))
+        return out.value
 
     def rmsnorm(self, x_dev, w_dev, rows, n, eps, y_dev):
         self._check(self.lib.skn_rmsnorm(self.handle, _ptr(x_dev), _ptr(w_dev), rows, n, eps, _ptr(y_dev)))

@@ -273,6 +273,26 @@ def test_gemm_expanded_errors(hip):
     buf.free()
 
 
+def test_machine_measurements_run(hip):
+    """The two machine figures of `bench.py --mode machine`: they run, and come out in the range the design argues from
+    (a matrix instruction of 32 clocks, vector instructions that hide only up to a point, fragment rates of a compute
+    unit between L2 and vector-cache speed)."""
+    scratch, flag, data = hip.alloc(512 * 1024), hip.alloc(16), hip.alloc(8 << 20)
+    hip.memset(data, 1, 8 << 20)
+    alone = hip.test_mfma_valu_overlap(2, 0, scratch)
+    loaded = hip.test_mfma_valu_overlap(2, 12, scratch)
+    assert 10.0 < alone < 25.0 and alone < loaded < 4 * alone
+    distinct = hip.test_fragment_delivery(1, data, 8, flag)
+    shared = hip.test_fragment_delivery(8, data, 8, flag)
+    assert 50.0 < distinct < 400.0 and shared > 0.9 * distinct
+    with pytest.raises(runtime.SknError, match="not built"):
+        hip.test_mfma_valu_overlap(1, 5, scratch)
+    with pytest.raises(runtime.SknError, match="share must be"):
+        hip.test_fragment_delivery(3, data, 8, flag)
+    for b in (scratch, flag, data):
+        b.free()
+
+
 def test_gemm_errors(hip):
     buf = hip.alloc(1 << 16)
     with pytest.raises(runtime.SknError) as e:
