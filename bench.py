@@ -196,8 +196,9 @@ def bench_gemm(ctx, qtype, m, n, k, reps=20, expanded=False):
 
 
 def machine_figures(ctx):
-    """Two figures of the machine that the GEMM's design argument uses: time per matrix instruction with independent
-    vector instructions behind it, and the rate at which operand fragments arrive in a compute unit's registers."""
+    """Figures of the machine that the GEMM's design argument uses: time per matrix instruction with independent
+    vector instructions behind it, the rate at which operand fragments arrive in a compute unit's registers, and the
+    cost of each part of the Q4_K GEMM's loop next to its matrix instructions."""
     scratch = ctx.alloc(512 * 1024)
     flag = ctx.alloc(16)
     overlap = {f"{w}_wavefronts_per_simd": {str(nv): round(ctx.test_mfma_valu_overlap(w, nv, scratch), 2) for nv in (0, 2, 4, 6, 7, 8, 12)}
@@ -208,11 +209,21 @@ def machine_figures(ctx):
         ctx.memset(data, 1, mib << 20)
         delivery[f"{mib}_mib_of_distinct_data"] = {str(sh): round(ctx.test_fragment_delivery(sh, data, mib, flag), 1) for sh in (1, 2, 4, 8)}
         data.free()
+    # the Q4_K GEMM's loop with parts left out (two passes: the clock of a box moves under such a load)
+    data = ctx.alloc(64 << 20)
+    ctx.memset(data, 0x3c, 64 << 20)
+    parts = (("matrix instructions only", 0), ("+ nibble decode from LDS", 3), ("+ activation fragments from memory", 7),
+             ("+ header unpack per superblock", 15), ("+ accumulator rescale", 31), ("+ min term (the whole loop)", 63),
+             ("whole loop without the fragments from memory", 59), ("whole loop without the rescale", 47),
+             ("whole loop without the header unpack", 55), ("matrix instructions and fragments only", 4))
+    loop = {name: [round(ctx.test_q4k_gemm_loop(p, data, scratch), 1) for _ in range(2)] for name, p in parts}
+    data.free()
     scratch.free()
     flag.free()
     return {"mode": "machine",
             "ns_per_mfma_32x32x16_f16_and_simd_by_vector_instructions_behind_it": overlap,
-            "fragment_gbs_per_compute_unit_by_wavefronts_sharing_a_stream": delivery}
+            "fragment_gbs_per_compute_unit_by_wavefronts_sharing_a_stream": delivery,
+            "q4k_gemm_loop_ns_per_k_step_and_simd": loop}
 
 
 def matvec_timeline(ctx, n, k, reps=20, queued=12):

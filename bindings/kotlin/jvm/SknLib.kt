@@ -88,6 +88,7 @@ object SknLib {
     val testMatvecQ4kStamps: MethodHandle = h("skn_test_matvec_q4k_stamps", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
     val testMfmaValuOverlap: MethodHandle = h("skn_test_mfma_valu_overlap", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS))
     val testFragmentDelivery: MethodHandle = h("skn_test_fragment_delivery", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, ADDRESS))
+    val testQ4kGemmLoop: MethodHandle = h("skn_test_q4k_gemm_loop", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
 
     init {
         val v = abiVersion.invokeExact() as Int

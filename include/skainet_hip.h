@@ -295,6 +295,12 @@ int skn_test_matvec_q4k_stamps(skn_ctx* ctx, const void* w_dev, int n, int k, co
 int skn_test_mfma_valu_overlap(skn_ctx* ctx, int waves_per_simd, int valu_per_mfma, float* scratch_dev, double* ns_out);
 int skn_test_fragment_delivery(skn_ctx* ctx, int share, const void* data_dev, int data_mib, unsigned* flag_dev,
                                double* gbs_out);
+/* Nanoseconds per k-step and SIMD (two wavefronts, eight matrix instructions) of a model of the Q4_K GEMM's inner loop
+ * with some of its parts left out (`bench.py --mode machine`); parts, bit by bit: 1 nibble decode, 2 nibbles from LDS
+ * and scale unpack, 4 activation fragments from memory, 8 header unpack per superblock, 16 accumulator rescale, 32 the
+ * "- dmin * m" term; built: 0, 3, 4, 7, 15, 31, 47, 55, 59, 63.  data_dev: 64 MiB of device memory, scratch_dev:
+ * 512 KiB.  No reference counterpart. */
+int skn_test_q4k_gemm_loop(skn_ctx* ctx, int parts, const void* data_dev, float* scratch_dev, double* ns_out);
 
 #ifdef __cplusplus
 }

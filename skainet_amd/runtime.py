@@ -89,6 +89,7 @@ _SIGNATURES = {
     "skn_test_matvec_q4k_stamps": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
     "skn_test_mfma_valu_overlap": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
     "skn_test_fragment_delivery": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
+    "skn_test_q4k_gemm_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]),
     "skn_kv_create": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "skn_kv_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_kv_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -383,6 +384,11 @@ class Context:
     def test_fragment_delivery(self, share, data_dev, data_mib, flag_dev):
         out = C.c_double()
         self._check(self.lib.skn_test_fragment_delivery(self.handle, share, _ptr(data_dev), data_mib, _ptr(flag_dev), C.byref(out)))
+        return out.value
+
+    def test_q4k_gemm_loop(self, parts, data_dev, scratch_dev):
+        out = C.c_double()
+        self._check(self.lib.skn_test_q4k_gemm_loop(self.handle, parts, _ptr(data_dev), _ptr(scratch_dev), C.byref(out)))
         return out.value
 
     def rmsnorm(self, x_dev, w_dev, rows, n, eps, y_dev):

@@ -285,6 +285,13 @@ def test_machine_measurements_run(hip):
     distinct = hip.test_fragment_delivery(1, data, 8, flag)
     shared = hip.test_fragment_delivery(8, data, 8, flag)
     assert 50.0 < distinct < 400.0 and shared > 0.9 * distinct
+    big = hip.alloc(64 << 20)
+    hip.memset(big, 0x3c, 64 << 20)
+    bare, whole = hip.test_q4k_gemm_loop(0, big, scratch), hip.test_q4k_gemm_loop(63, big, scratch)
+    assert 80.0 < bare < 250.0 and bare < whole < 5 * bare
+    with pytest.raises(runtime.SknError, match="not built"):
+        hip.test_q4k_gemm_loop(5, big, scratch)
+    big.free()
     with pytest.raises(runtime.SknError, match="not built"):
         hip.test_mfma_valu_overlap(1, 5, scratch)
     with pytest.raises(runtime.SknError, match="share must be"):
