@@ -281,14 +281,14 @@ def test_machine_measurements_run(hip):
     hip.memset(data, 1, 8 << 20)
     alone = hip.test_mfma_valu_overlap(2, 0, scratch)
     loaded = hip.test_mfma_valu_overlap(2, 12, scratch)
-    assert 10.0 < alone < 25.0 and alone < loaded < 4 * alone
+    assert 5.0 < alone < 60.0 and alone < loaded < 6 * alone
     distinct = hip.test_fragment_delivery(1, data, 8, flag)
     shared = hip.test_fragment_delivery(8, data, 8, flag)
-    assert 50.0 < distinct < 400.0 and shared > 0.9 * distinct
+    assert 20.0 < distinct < 1000.0 and shared > 0.7 * distinct
     big = hip.alloc(64 << 20)
     hip.memset(big, 0x3c, 64 << 20)
     bare, whole = hip.test_q4k_gemm_loop(0, big, scratch), hip.test_q4k_gemm_loop(63, big, scratch)
-    assert 80.0 < bare < 250.0 and bare < whole < 5 * bare
+    assert 40.0 < bare < 600.0 and bare < whole < 8 * bare
     with pytest.raises(runtime.SknError, match="not built"):
         hip.test_q4k_gemm_loop(5, big, scratch)
     big.free()
