@@ -362,7 +362,7 @@ def bench_other_formats(ctx):
     for nn, kk in ((4096, 4096), (4096, 11008)):
         res = {}
         for name, qt in (("q4_0", 2), ("q4_1", 3), ("q5_0", 6), ("q5_1", 7), ("q2_k", 10), ("q3_k", 11), ("q5_k", 13),
-                         ("q8_k", 15), ("iq4_nl", 20), ("iq4_xs", 23), ("f16", 1)):
+                         ("q8_k", 15), ("iq4_nl", 20), ("iq4_xs", 23), ("tq1_0", 34), ("tq2_0", 35), ("f16", 1)):
             r = bench_matvec(ctx, qt, nn, kk, 200, 20, copies=24, seed=7000 + qt)
             res[name] = {"kernel_us": round(r["kernel_us"], 2), "kernel_gbs": round(r["kernel_gbs"], 1)}
         out[f"{nn}x{kk}"] = res

@@ -1136,6 +1136,155 @@ __global__ __launch_bounds__(512) void matvec_runs_kernel(const uint8_t* __restr
     }
 }
 
+// TQ1_0 (54 bytes per 256: qs u8[48] @0, qh u8[4] @48, f16 d @52; blocks 2-byte aligned).  A byte packs five trits, a qh
+// byte four: trit n = ((byte * 3^n mod 256) * 3) >> 8, y = d (t - 1).  Lane (b, jj) = (lane / 4, lane % 4) of a step owns,
+// of superblock b, bytes 8 jj .. 8 jj + 7 (elements 32 n + 8 jj + 0..7 for n < 5), bytes 32 + 4 jj .. + 3 (elements
+// 160 + 16 n + 4 jj + 0..3) and qh byte jj (elements 240 + 4 n + jj for n < 4): 64 elements from 13 bytes.  x is staged in
+// that order -- slot 2 n + h of a lane: the h-th four of its eight elements under trit n; slot 10 + n: its four of the
+// second region; slot 15: its four of the third -- so a step reads sixteen float4 per lane without bank conflicts.
+// Two bytes are decoded at a time in the halves of a dword: (b0 | b2 << 16) * 3^n stays inside its halves
+// (255 * 81 < 2^16), so does the product with 3 after the mask, and the two trits are bytes 1 and 3 of the result
+// (v_cvt_f32_ubyte1 / 3): 3.5 vector instructions per weight, the "- 1" comes back out as the sum of the lane's x.
+typedef uint32_t u32_a2 __attribute__((aligned(2)));
+
+struct Tq1Loads {
+    u32x2 qa;      // bytes 8 jj .. 8 jj + 7
+    uint32_t qb;   // bytes 32 + 4 jj .. + 3
+    uint32_t qh;   // qh byte jj
+    uint32_t d;    // f16 bits
+    bool ok;
+};
+
+__device__ __forceinline__ void tq1_stage_store_one(const float4& v, int f, float4* xs) {
+    const int blk = f >> 6, w = f & 63;
+    const int step = blk >> 4, ln4 = (blk & 15) * 4;
+    if (w < 40) {
+        const int n = w >> 3, jj = (w & 7) >> 1, h = w & 1;
+        xs[(step * 16 + 2 * n + h) * kXPitch + ln4 + jj] = v;
+    } else if (w < 60) {
+        const int n = (w - 40) >> 2, jj = (w - 40) & 3;
+        xs[(step * 16 + 10 + n) * kXPitch + ln4 + jj] = v;
+    } else {
+        // elements 240 + 4 n + jj: component jj of this float4 is element n of lane jj's last slot
+        float* last = reinterpret_cast<float*>(xs + (step * 16 + 15) * kXPitch + ln4) + (w - 60);
+        last[0] = v.x, last[4] = v.y, last[8] = v.z, last[12] = v.w;
+    }
+}
+
+// sum over the four bytes of q (as trit n) times the four components of x
+template <int N>
+__device__ __forceinline__ float tq1_dot_dword(uint32_t lo, uint32_t hi, const float4& x, float sa) {
+    constexpr uint32_t kPow3 = N == 0 ? 1u : N == 1 ? 3u : N == 2 ? 9u : N == 3 ? 27u : 81u;
+    const uint32_t tl = N == 0 ? lo : __umul24(lo, kPow3) & 0x00FF00FFu;
+    const uint32_t th = N == 0 ? hi : __umul24(hi, kPow3) & 0x00FF00FFu;
+    const uint32_t ml = __umul24(tl, 3u), mh = __umul24(th, 3u);
+    sa = fmaf((float)((ml >> 8) & 0xFFu), x.x, sa);
+    sa = fmaf((float)((mh >> 8) & 0xFFu), x.y, sa);
+    sa = fmaf((float)(ml >> 24), x.z, sa);
+    sa = fmaf((float)(mh >> 24), x.w, sa);
+    return sa;
+}
+
+template <int R>
+__device__ __forceinline__ void tq1_step(const Tq1Loads (&L)[R], const float4* __restrict__ xs, int s, int lane, float (&acc)[R]) {
+    float4 xv[16];
+    float sx = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        xv[i] = xs[(s * 16 + i) * kXPitch + lane];
+        sx += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float sa = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t q = L[r].qa[h], lo = q & 0x00FF00FFu, hi = (q >> 8) & 0x00FF00FFu;
+            sa = tq1_dot_dword<0>(lo, hi, xv[0 + h], sa);
+            sa = tq1_dot_dword<1>(lo, hi, xv[2 + h], sa);
+            sa = tq1_dot_dword<2>(lo, hi, xv[4 + h], sa);
+            sa = tq1_dot_dword<3>(lo, hi, xv[6 + h], sa);
+            sa = tq1_dot_dword<4>(lo, hi, xv[8 + h], sa);
+        }
+        {
+            const uint32_t q = L[r].qb, lo = q & 0x00FF00FFu, hi = (q >> 8) & 0x00FF00FFu;
+            sa = tq1_dot_dword<0>(lo, hi, xv[10], sa);
+            sa = tq1_dot_dword<1>(lo, hi, xv[11], sa);
+            sa = tq1_dot_dword<2>(lo, hi, xv[12], sa);
+            sa = tq1_dot_dword<3>(lo, hi, xv[13], sa);
+            sa = tq1_dot_dword<4>(lo, hi, xv[14], sa);
+        }
+        {
+            // the qh byte: trits 0..3 against the four components of the last slot
+            const uint32_t b = L[r].qh;
+            const uint32_t t01 = (b | (__umul24(b, 3u) << 16)) & 0x00FF00FFu;      // b, 3 b mod 256
+            const uint32_t t23 = (__umul24(b, 9u) & 0xFFu) | ((__umul24(b, 27u) & 0xFFu) << 16);
+            const uint32_t m01 = __umul24(t01, 3u), m23 = __umul24(t23, 3u);
+            sa = fmaf((float)((m01 >> 8) & 0xFFu), xv[15].x, sa);
+            sa = fmaf((float)(m01 >> 24), xv[15].y, sa);
+            sa = fmaf((float)((m23 >> 8) & 0xFFu), xv[15].z, sa);
+            sa = fmaf((float)(m23 >> 24), xv[15].w, sa);
+        }
+        acc[r] += L[r].ok ? h2f_bits((uint16_t)L[r].d) * (sa - sx) : 0.f;
+    }
+}
+
+template <int STEPS, int R>
+__global__ __launch_bounds__(512) void matvec_tq1_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                         float* __restrict__ y, int n_rows, int nb) {
+    extern __shared__ float4 lds4[];
+    float4* xs = lds4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int sub = lane >> 2, jj = lane & 3;
+    const int row0 = (blockIdx.x * 8 + wave) * R;
+    const int n4 = nb * 64;  // float4 count of x
+    constexpr int J = 2 * STEPS;
+    Q4kStage<J> st;
+    q4k_stage_load<J>(x, n4, tid, 512, st);
+
+    float acc[R];
+    const uint8_t* rp[R];
+    bool row_ok[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.f;
+        row_ok[r] = row0 + r < n_rows;
+        rp[r] = w + (size_t)min(row0 + r, n_rows - 1) * nb * 54;
+    }
+    Tq1Loads L[STEPS][R];
+    auto issue = [&](int s, int tie) __attribute__((always_inline)) {
+        const int blk = s * 16 + sub;
+        const size_t off = (size_t)(min(blk, nb - 1) + tie) * 54;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint8_t* bp = rp[r] + off;
+            L[s][r].qa = *reinterpret_cast<const u32x2_a2*>(bp + 8 * jj);
+            L[s][r].qb = *reinterpret_cast<const u32_a2*>(bp + 32 + 4 * jj);
+            L[s][r].qh = bp[48 + jj];
+            L[s][r].d = load_u16_a2(bp + 52);
+            L[s][r].ok = row_ok[r] && blk < nb;
+        }
+    };
+    issue(0, 0);
+#pragma unroll
+    for (int j = 0; j < J; j++) tq1_stage_store_one(st.v[j], min(tid + j * 512, n4 - 1), xs);
+    __syncthreads();
+    int tie = 0;
+    asm volatile("" : "+v"(tie));
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        if (s + 1 < STEPS) issue(s + 1, tie);
+        asm volatile("" ::: "memory");
+        tq1_step<R>(L[s], xs, s, lane + tie, acc);
+        asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float total = wave_sum(acc[r]);
+        if (lane == 0 && row_ok[r]) y[row0 + r] = total;
+    }
+}
+
 // What the rotary epilogue needs beyond the row totals, formed at the top of the kernel so that its dependent
 // loads (position, then page id) and the sine / cosine are off the tail of the wavefront.
 struct Q4kRopeCtx {
@@ -1521,6 +1670,22 @@ int launch_q8k(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, fl
 }
 
 template <int STEPS>
+int launch_tq1(skn_ctx* ctx, const uint8_t* w, int n, int nb, const float* x, float* y) {
+    constexpr int R = STEPS <= 2 ? 2 : 1;
+    const size_t lds = (size_t)STEPS * 16 * kXPitch * sizeof(float4);
+    dim3 grid((unsigned)((n + 8 * R - 1) / (8 * R))), block(512);
+    skn_launch(ctx, matvec_tq1_kernel<STEPS, R>, grid, block, lds, w, x, y, n, nb);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+template <int STEPS>
+hipError_t allow_big_lds_tq1() {
+    return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_tq1_kernel<STEPS, (STEPS <= 2 ? 2 : 1)>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+
+template <int STEPS>
 hipError_t allow_big_lds_q8k() {
     return hipFuncSetAttribute(reinterpret_cast<const void*>(matvec_q8k_kernel<STEPS, (STEPS <= 2 ? 2 : 1)>),
                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -1578,6 +1743,10 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_HIP(ctx, (allow_big_lds_runs<2, kRunsTQ2>()));
     SKN_HIP(ctx, (allow_big_lds_runs<3, kRunsTQ2>()));
     SKN_HIP(ctx, (allow_big_lds_runs<4, kRunsTQ2>()));
+    SKN_HIP(ctx, allow_big_lds_tq1<1>());
+    SKN_HIP(ctx, allow_big_lds_tq1<2>());
+    SKN_HIP(ctx, allow_big_lds_tq1<3>());
+    SKN_HIP(ctx, allow_big_lds_tq1<4>());
     SKN_HIP(ctx, allow_big_lds_q8k<1>());
     SKN_HIP(ctx, allow_big_lds_q8k<2>());
     SKN_HIP(ctx, allow_big_lds_q8k<3>());
@@ -1775,6 +1944,15 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         return dispatch_runs<kRunsQ3K>(ctx, w, n, nb, x_dev, y_dev);
     if (ggml_type == SKN_TYPE_TQ2_0 && nb <= 64 && ctx->opt_matvec_stage == 1)
         return dispatch_runs<kRunsTQ2>(ctx, w, n, nb, x_dev, y_dev);
+    // TQ1_0: its own lane map (blocks are 2-byte aligned)
+    if (ggml_type == SKN_TYPE_TQ1_0 && ((uintptr_t)w_dev & 1) == 0 && nb <= 64 && ctx->opt_matvec_stage == 1) {
+        switch ((nb + 15) / 16) {
+            case 1: return launch_tq1<1>(ctx, w, n, nb, x_dev, y_dev);
+            case 2: return launch_tq1<2>(ctx, w, n, nb, x_dev, y_dev);
+            case 3: return launch_tq1<3>(ctx, w, n, nb, x_dev, y_dev);
+            default: return launch_tq1<4>(ctx, w, n, nb, x_dev, y_dev);
+        }
+    }
     // Q8_K: the Q8_0 arithmetic on the Q4_K lane map (blocks are 4-byte aligned)
     if (ggml_type == SKN_TYPE_Q8_K && ((uintptr_t)w_dev & 3) == 0 && nb <= 64 && ctx->opt_matvec_stage == 1) {
         switch ((nb + 15) / 16) {

@@ -87,13 +87,14 @@ def test_matvec_staged_and_plain_kernels(hip, qtype, name, n, k):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (20, "iq4_nl"),
-                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k"), (35, "tq2_0")])
+                                        (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k"), (35, "tq2_0"), (34, "tq1_0")])
 @pytest.mark.parametrize("n,k", [(33, 256), (16, 4096), (17, 8192), (9, 8448), (5, 12288), (3, 16384), (2, 36864), (1, 37120)])
 def test_lane_map_matvec_every_step_count(hip, qtype, name, n, k):
     """The formats on the Q4_K kernel's lane map: rows of one to four unrolled steps (16 superblocks, or 16 groups of
     eight small blocks, each), a partial last step, the rolled loop beyond four steps, the longest row the kernel
     takes (144 superblocks) and one past it (direct kernel).  Q2_K and Q3_K (the Q6_K kernel's lane map) and Q8_K: one
-    to four steps, then the kernels for longer rows; TQ2_0 likewise (the packing of Q2_K's quants)."""
+    to four steps, then the kernels for longer rows; TQ2_0 likewise (the packing of Q2_K's quants) and TQ1_0 (a lane map
+    of its own)."""
     raw = synth.weight(qtype, n, k, seed=n + k)
     x = synth.activation_f32(k, seed=k + 3)
     got = hip.matvec_q_host(qtype, raw, n, k, x)
@@ -274,6 +275,39 @@ def test_tq2_0_matvec_bit_pairs_alone(hip):
     v = raw.copy()
     v[:, :, :64] = 0x55
     got = hip.matvec_q_host(35, v.reshape(n, -1), n, k, x)
+    assert np.abs(got).max() <= 1e-5 * np.abs(x).sum() * 0.05
+
+
+def test_tq1_0_matvec_regions_alone(hip):
+    """TQ1_0 (qs[48] @0, qh[4] @48, d @52; five trits per byte, four per qh byte; y = d (t - 1)) on its lane-map kernel:
+    each of the three regions of a block alone and each lane's bytes alone (every other byte 0x80: all its trits 1, its
+    weights zero), all trits 2 (byte 255: y = d sum x), all trits 0 (byte 0: y = -d sum x), odd rows (2-byte aligned)."""
+    n, k = 15, 4096 + 256
+    raw = synth.weight(34, n, k, seed=71).reshape(n, k // 256, 54).copy()
+    x = synth.activation_f32(k, seed=72)
+    variants = [raw]
+    for lo, hi in ((0, 32), (32, 48), (48, 52)):
+        v = raw.copy()
+        keep = np.zeros(52, bool)
+        keep[lo:hi] = True
+        v[:, :, :52][:, :, ~keep] = 0x80
+        variants.append(v)
+    for jj in range(4):
+        v = raw.copy()
+        keep = np.zeros(52, bool)
+        keep[8 * jj:8 * jj + 8] = keep[32 + 4 * jj:36 + 4 * jj] = keep[48 + jj] = True
+        v[:, :, :52][:, :, ~keep] = 0x80
+        variants.append(v)
+    for fill in (255, 0):
+        v = raw.copy()
+        v[:, :, :52] = fill
+        variants.append(v)
+    for v in variants:
+        _against_oracle(hip, 34, v, n, k, x)
+    # all trits 1: every weight is zero, and what is left of sum(t x) - sum(x) is rounding noise
+    v = raw.copy()
+    v[:, :, :52] = 0x80
+    got = hip.matvec_q_host(34, v.reshape(n, -1), n, k, x)
     assert np.abs(got).max() <= 1e-5 * np.abs(x).sum() * 0.05
 
 
