@@ -103,12 +103,12 @@ int skn_set_stream(skn_ctx* ctx, void* hip_stream);
  * "llama.graph" (1 = replay a captured HIP graph per decode step, the default; 0 = launch every kernel; a captured
  * step is dropped and captured again after any change of an option or of the stream),
  * "llama.fused" (1 = fused per-layer kernels in the decode step, the default: for every group of matrices whose
- * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K), "llama.expand_weights" (1 = the prompt pass of a decoder keeps an expanded
+ * formats have one -- Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K, TQ1_0, TQ2_0), "llama.expand_weights" (1 = the prompt pass of a decoder keeps an expanded
  * copy, see skn_gemm_expand, of every layer matrix that is not Q4_K, made at the first prompt: 4 bytes per weight of
  * device memory on top of the blocks; 0 = the default, expand per call), "gemm.tile" (0 = choose, 1 = 64-row tiles,
  * 2 = 128-row tiles of the Q4_K GEMM), "matvec.stage" (kernel family of the further formats' matvec: 1 = the
  * default -- the Q4_K kernel's lane map for Q5_K / Q4_0 / Q4_1 / Q5_0 / Q5_1 / IQ4_NL / IQ4_XS / Q8_K, the Q6_K kernel's for
- * Q2_K / Q3_K / TQ2_0, rows staged through LDS for what is left with 4-byte-multiple blocks; 2 = staged rows for all
+ * Q2_K / Q3_K / TQ2_0, its own for TQ1_0, rows staged through LDS for what is left with 4-byte-multiple blocks; 2 = staged rows for all
  * formats with such blocks; 0 = direct reads).  The knobs exist for
  * measurements and tests; every setting computes the same results to the tolerance of the operation. */
 int skn_set_option(skn_ctx* ctx, const char* key, int value);
@@ -273,7 +273,7 @@ int skn_llama_logits(skn_ctx* ctx, skn_llama* m, const float** logits_dev);
  * (norm_w_dev, eps), and an epilogue: 0 store y, 1 y +=, 2 y[i] = silu(w0 row i . x) * (w1 row i . x), 3 rotary
  * embedding of q (rows0, to y as fp32) and k (rows1) with k and v (rows2) stored as fp16 at the end of sequence 0 of the
  * one-sequence cache `kv` (its position is written to *pos_dev, a device int the caller provides).  No reference
- * counterpart.  Types: Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K; k a multiple of 256,
+ * counterpart.  Types: Q4_K, Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q6_K, Q8_0, Q2_K, Q3_K, Q8_K, TQ1_0, TQ2_0; k a multiple of 256,
  * at most 16384. */
 int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const void* w0, int rows0, const void* w1, int rows1,
                           const void* w2, int rows2, int k, const float* x_dev, const float* norm_w_dev, float eps,

@@ -169,7 +169,7 @@ struct Q5kLoads : Q4kLoads {
 // to bit 1, which is the form q5k_dot_dword takes.
 constexpr int kFmtQ4K = 0, kFmtQ5K = 1, kFmtQ40 = 2, kFmtQ41 = 3, kFmtQ50 = 4, kFmtQ51 = 5, kFmtIQ4NL = 8, kFmtIQ4XS = 9;
 constexpr int kFmtQ6K = 6, kFmtQ80 = 7;  // (fused kernels only: the lane maps, staging and steps of matvec_q6k_kernel / matvec_q80_pairs_kernel)
-constexpr int kFmtQ2K = 10, kFmtQ3K = 11, kFmtQ8K = 12;  // (fused kernels only: those of matvec_runs_kernel / matvec_q8k_kernel)
+constexpr int kFmtQ2K = 10, kFmtQ3K = 11, kFmtQ8K = 12, kFmtTQ2 = 13, kFmtTQ1 = 14;  // (fused kernels only: those of matvec_runs_kernel / matvec_q8k_kernel / matvec_tq1_kernel)
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
@@ -1363,11 +1363,13 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                                                                skn_rope_epilogue rope) {
     constexpr int R = 2;
     constexpr bool Q5 = F == kFmtQ5K, Q6 = F == kFmtQ6K, Q8 = F == kFmtQ80, Q2 = F == kFmtQ2K, Q3 = F == kFmtQ3K, Q8K = F == kFmtQ8K;
-    constexpr bool kRuns = Q6 || Q2 || Q3;  // the Q6_K lane map: four runs of sixteen per lane, a float4 of run sums
+    constexpr bool T2 = F == kFmtTQ2, T1 = F == kFmtTQ1;
+    constexpr bool kRuns = Q6 || Q2 || Q3 || T2;  // the Q6_K lane map: four runs of sixteen per lane, a float4 of run sums
     constexpr bool kXS = F == kFmtIQ4XS;
     constexpr bool kSmall = F >= kFmtQ40 && F <= kFmtIQ4XS && !Q6 && !Q8;
     using Loads = std::conditional_t<Q8, Q80Loads, std::conditional_t<Q6, Q6kLoads, std::conditional_t<Q2, Q2kLoads, std::conditional_t<Q3, Q3kLoads,
-                  std::conditional_t<Q8K, Q8kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>>>>;
+                  std::conditional_t<T2, Tq2Loads, std::conditional_t<T1, Tq1Loads,
+                  std::conditional_t<Q8K, Q8kLoads, std::conditional_t<kSmall, Q4xLoads, std::conditional_t<Q5, Q5kLoads, Q4kLoads>>>>>>>>>;
     constexpr int kChunks = Q5 ? 11 : 9, kFirst = Q5 ? 3 : 1;
     constexpr int kSmallBytes = (F == kFmtQ40 || F == kFmtIQ4NL) ? 18 : (F == kFmtQ41 ? 20 : (F == kFmtQ50 ? 22 : 24)), kHi = kSmall ? 4 : 8;
     constexpr bool kPlainX = F == kFmtIQ4NL || kXS;  // x staged unscaled, block sums times 128, results in true units
@@ -1397,7 +1399,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const int unit = blockIdx.x * 8 + wave;
     const uint8_t* rowp[R];
     bool row_ok[R];
-    const size_t row_bytes = (size_t)nb * (Q8 ? 272 : Q6 ? 210 : Q2 ? 84 : Q3 ? 110 : Q8K ? 292 : kXS ? 136 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
+    const size_t row_bytes = (size_t)nb * (Q8 ? 272 : Q6 ? 210 : Q2 ? 84 : Q3 ? 110 : T2 ? 66 : T1 ? 54 : Q8K ? 292 : kXS ? 136 : kSmall ? 8 * kSmallBytes : 16 * kChunks);
     if (EPI == SKN_EPI_SWIGLU) {
         const int i = min(unit, n_out - 1);
         row_ok[0] = row_ok[1] = unit < n_out;
@@ -1454,6 +1456,17 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
                 L[s][r].hm = *reinterpret_cast<const u32x4_a2*>(bp + 16 * hsel);
                 L[s][r].sc = *reinterpret_cast<const u32x3_a2*>(bp + 96);
                 L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 108);
+            } else if constexpr (T2) {
+                const int n = p >> 1, hsel = p & 1;
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 66;
+                L[s][r].q = *reinterpret_cast<const u32x4_a2*>(bp + 32 * n + 16 * hsel);
+                L[s][r].d = *reinterpret_cast<const uint16_t*>(bp + 64);
+            } else if constexpr (T1) {
+                const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 54;
+                L[s][r].qa = *reinterpret_cast<const u32x2_a2*>(bp + 8 * p);
+                L[s][r].qb = *reinterpret_cast<const u32_a2*>(bp + 32 + 4 * p);
+                L[s][r].qh = bp[48 + p];
+                L[s][r].d = load_u16_a2(bp + 52);
             } else if constexpr (Q8K) {
                 const uint8_t* bp = rowp[r] + (size_t)(min(blk, nb - 1) + tie) * 292;
 #pragma unroll
@@ -1504,6 +1517,9 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     } else if constexpr (kRuns) {
 #pragma unroll
         for (int jj = 0; jj < J; jj++) q6k_stage_store_one<Q6 ? 32 : Q3 ? 4 : 1>(st.v[jj], min(tid + jj * 512, n4 - 1), xs, ss);
+    } else if constexpr (T1) {
+#pragma unroll
+        for (int jj = 0; jj < J; jj++) tq1_stage_store_one(st.v[jj], min(tid + jj * 512, n4 - 1), xs);
     } else {
         q4k_stage_store<J, !kPlainX, kHi>(st, n4, tid, 512, xs, ss);
     }
@@ -1529,11 +1545,13 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         else if constexpr (Q6) q6k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
         else if constexpr (Q2) q2k_step<R>(L[s], xs, ss, s, lane + tie, p & 1, acc);
         else if constexpr (Q3) q3k_step<R>(L[s], xs, ss, s, lane + tie, p >> 1, p & 1, acc);
+        else if constexpr (T2) tq2_step<R>(L[s], xs, ss, s, lane + tie, acc);
+        else if constexpr (T1) tq1_step<R>(L[s], xs, s, lane + tie, acc);
         else if constexpr (kSmall) q4x_step<R, F>(L[s], xs, ss, s, lane + tie, acc);
         else q4k_step<R>(L[s], xs, ss, s, lane + tie, p, acc);
         asm volatile("" : "+v"(tie), "+v"(acc[R - 1]));
     }
-    const float back = (Q8 || Q8K || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
+    const float back = (Q8 || Q8K || T1 || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
     const float t0 = wave_sum(acc[0]) * back;
     const float t1 = wave_sum(acc[1]) * back;
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
@@ -1542,7 +1560,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
 template <int STEPS, int EPI, bool NORM, int F>
 int launch_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int nb, const float* x, const float* norm_w,
                      float eps, float* y, const skn_rope_epilogue& rope) {
-    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * ((F == kFmtQ6K || F == kFmtQ2K || F == kFmtQ3K) ? sizeof(float4) : sizeof(float2))) + 8 * sizeof(float);
+    const size_t lds = (size_t)STEPS * (16 * kXPitch * sizeof(float4) + 64 * ((F == kFmtQ6K || F == kFmtQ2K || F == kFmtQ3K || F == kFmtTQ2) ? sizeof(float4) : sizeof(float2))) + 8 * sizeof(float);
     const int units = EPI == SKN_EPI_SWIGLU ? n_out : (n_out + 1) / 2;
     dim3 grid((unsigned)((units + 7) / 8)), block(512);
     skn_launch(ctx, matvec_q4k_fused_kernel<STEPS, EPI, NORM, F>, grid, block, lds, seg, x, norm_w, eps, y, n_out, nb, rope);
@@ -1773,6 +1791,8 @@ int skn_matvec_init(skn_ctx* ctx) {
     SKN_ALLOW_FUSED(kFmtQ2K);
     SKN_ALLOW_FUSED(kFmtQ3K);
     SKN_ALLOW_FUSED(kFmtQ8K);
+    SKN_ALLOW_FUSED(kFmtTQ2);
+    SKN_ALLOW_FUSED(kFmtTQ1);
 #undef SKN_ALLOW_FUSED
     return SKN_OK;
 }
@@ -1781,7 +1801,8 @@ bool skn_matvec_fusable(int ggml_type) {
     return ggml_type == SKN_TYPE_Q4_K || ggml_type == SKN_TYPE_Q5_K || ggml_type == SKN_TYPE_Q4_0 ||
            ggml_type == SKN_TYPE_Q4_1 || ggml_type == SKN_TYPE_Q5_0 || ggml_type == SKN_TYPE_Q5_1 ||
            ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_IQ4_NL ||
-           ggml_type == SKN_TYPE_IQ4_XS || ggml_type == SKN_TYPE_Q2_K || ggml_type == SKN_TYPE_Q3_K || ggml_type == SKN_TYPE_Q8_K;
+           ggml_type == SKN_TYPE_IQ4_XS || ggml_type == SKN_TYPE_Q2_K || ggml_type == SKN_TYPE_Q3_K || ggml_type == SKN_TYPE_Q8_K ||
+           ggml_type == SKN_TYPE_TQ1_0 || ggml_type == SKN_TYPE_TQ2_0;
 }
 
 // Fused matvec for the decoder, all matrices of one of the formats above; k <= 16384 (four unrolled steps).
@@ -1790,7 +1811,7 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
                          float eps, float* y, int epi, const skn_rope_epilogue* rope_in, int ggml_type) {
     SKN_REQUIRE(ctx, skn_matvec_fusable(ggml_type), SKN_ERR_TYPE, "fused matvec: ggml type %d has no fused kernel", ggml_type);
     {
-        const uintptr_t mask = (ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q3_K) ? 1
+        const uintptr_t mask = (ggml_type == SKN_TYPE_Q6_K || ggml_type == SKN_TYPE_Q3_K || ggml_type == SKN_TYPE_TQ1_0 || ggml_type == SKN_TYPE_TQ2_0) ? 1
                                : (ggml_type == SKN_TYPE_Q8_0 || ggml_type == SKN_TYPE_Q2_K || ggml_type == SKN_TYPE_Q8_K) ? 3
                                : ggml_type == SKN_TYPE_IQ4_XS ? 7 : 15;
         for (int i = 0; i < 3; i++)
@@ -1831,6 +1852,8 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         case SKN_TYPE_Q2_K: SKN_FUSED(kFmtQ2K)
         case SKN_TYPE_Q3_K: SKN_FUSED(kFmtQ3K)
         case SKN_TYPE_Q8_K: SKN_FUSED(kFmtQ8K)
+        case SKN_TYPE_TQ2_0: SKN_FUSED(kFmtTQ2)
+        case SKN_TYPE_TQ1_0: SKN_FUSED(kFmtTQ1)
         default: SKN_FUSED(kFmtQ4K)
     }
 #undef SKN_FUSED

@@ -11,7 +11,7 @@ from skainet_amd import synth
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
 FUSED_TYPES = [synth.Q4_K, synth.Q5_K, synth.Q4_0, synth.Q4_1, synth.Q5_0, synth.Q5_1, synth.IQ4_NL, synth.Q6_K, synth.Q8_0,
-               synth.IQ4_XS, synth.Q2_K, synth.Q3_K, synth.Q8_K]
+               synth.IQ4_XS, synth.Q2_K, synth.Q3_K, synth.Q8_K, synth.TQ2_0, synth.TQ1_0]
 STORE, ADD, SWIGLU, ROPE = 0, 1, 2, 3
 
 

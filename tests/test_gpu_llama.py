@@ -364,12 +364,17 @@ def test_longer_prompt_releases_the_shorter_prompt_buffers(hip):
     model.free()
 
 
+def _scale_d(raw, block_bytes, d_offset, factor):
+    """Block bytes with every d (fp16 at byte d_offset of each block) multiplied by a power of two."""
+    blocks = raw.reshape(-1, block_bytes).copy()
+    d = blocks[:, d_offset:d_offset + 2].copy().view(np.float16).astype(np.float32) * factor
+    blocks[:, d_offset:d_offset + 2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return blocks.reshape(raw.shape)
+
+
 def _scale_q6k(raw, factor):
     """Q6_K block bytes with every d (fp16 at byte 208 of the 210) multiplied by a power of two."""
-    blocks = raw.reshape(-1, 210).copy()
-    d = blocks[:, 208:210].copy().view(np.float16).astype(np.float32) * factor
-    blocks[:, 208:210] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
-    return blocks.reshape(raw.shape)
+    return _scale_d(raw, 210, 208, factor)
 
 
 def _decode_against_oracle(hip, cfg, w, n_steps, modes=(1, 0), tol=TOL):
@@ -395,7 +400,7 @@ def _decode_against_oracle(hip, cfg, w, n_steps, modes=(1, 0), tol=TOL):
 
 
 @pytest.mark.parametrize("qtype,name", [(13, "q5_k"), (2, "q4_0"), (3, "q4_1"), (6, "q5_0"), (7, "q5_1"), (14, "q6_k"),
-                                        (8, "q8_0"), (20, "iq4_nl"), (10, "q2_k")])
+                                        (8, "q8_0"), (20, "iq4_nl"), (10, "q2_k"), (34, "tq1_0")])
 @pytest.mark.parametrize("group", ["qkv", "o", "gu", "down"])
 def test_fused_groups_of_further_formats(hip, qtype, name, group):
     """The fused decode kernels take Q5_K, Q4_0, Q4_1, Q5_0, Q5_1, Q6_K and Q8_0 as well: one group of matrices at a time in
@@ -418,6 +423,13 @@ def test_fused_groups_of_further_formats(hip, qtype, name, group):
                 w[f"l{l}.{m}"] = (14, _scale_q6k(w[f"l{l}.{m}"][1], 2.0 ** -8))
         _decode_against_oracle(hip, cfg, w, 5, tol=2e-2)
         return
+    if group == "qkv" and qtype == 34:
+        # (ternary, zero-centred queries, keys and values: on this stack the separate kernels reach 1.7e-3 at the third
+        # step and 8e-3 at the fifth, the fused ones 2.7e-3 and 1.4e-2 -- it is the stack that amplifies; each fused
+        # launch of this format holds 1e-3 as an operation in test_gpu_fused_ops.py.  Three steps, at the bound of
+        # the Q8_0 case below.)
+        _decode_against_oracle(hip, cfg, w, 3, tol=5e-3)
+        return
     if group == "qkv" and qtype == 8:
         # (zero-centred queries and keys again, at a tenth of the Q6_K magnitudes: the separate kernels reach
         # 1.4e-3 on this stack at one step or another, the fused ones 2.2e-3)
@@ -427,7 +439,7 @@ def test_fused_groups_of_further_formats(hip, qtype, name, group):
 
 
 @pytest.mark.parametrize("qtype,name", [(12, "q4_k"), (13, "q5_k"), (2, "q4_0"), (6, "q5_0"), (14, "q6_k"), (8, "q8_0"),
-                                        (20, "iq4_nl"), (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k")])
+                                        (20, "iq4_nl"), (23, "iq4_xs"), (10, "q2_k"), (11, "q3_k"), (15, "q8_k"), (35, "tq2_0"), (34, "tq1_0")])
 @pytest.mark.parametrize("ffn", [8192, 11008, 14336])
 def test_fused_down_projection_of_two_to_four_steps(hip, qtype, name, ffn):
     """Rows of 8192, 11008 and 14336 weights take two, three and four unrolled steps of the fused kernel (4096
@@ -450,10 +462,11 @@ def test_fused_groups_of_two_steps(hip, group, qtype):
     _decode_against_oracle(hip, cfg, w, 3)
 
 
-@pytest.mark.parametrize("tq,tk,tv", [(12, 12, 14), (13, 2, 14), (14, 12, 12), (12, 8, 14), (12, 10, 12), (12, 35, 12)])
+@pytest.mark.parametrize("tq,tk,tv", [(12, 12, 14), (13, 2, 14), (14, 12, 12), (12, 8, 14), (12, 10, 12), (12, 35, 12),
+                                      (34, 12, 35), (12, 1, 12)])
 def test_qkv_of_mixed_formats(hip, tq, tk, tv):
     """q, k and v of different formats (value projections with more bits, as mixed quantizations have them): one
-    fused launch per format, each carrying the rows of its matrices only; a format without a fused kernel (TQ2_0)
+    fused launch per format, each carrying the rows of its matrices only; a format without a fused kernel (F16)
     sends the group to the separate kernels.  Layer 1 keeps Q4_K; down projections Q6_K as in such files."""
     cfg = llama.Config(n_layer=2, hidden=512, ffn=768, n_head=4, n_kv_head=2, head_dim=128, vocab=512, max_tokens=64,
                        page_tokens=16, matrix_types={"l0.wq": tq, "l0.wk": tk, "l0.wv": tv, "l0.w_down": 14})
