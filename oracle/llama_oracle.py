@@ -1,7 +1,13 @@
 """CPU oracle of the Llama-style decoder (test infrastructure only): the same module graph evaluated with the C
 oracle's kernels (fp64 accumulation), token by token.  Prompt tokens can be run either exactly like decode steps
 (`bf16_gemm=False`) or with the activations of every projection rounded to bf16 first (`bf16_gemm=True`), which is
-what the batched prompt path of the library feeds its GEMMs with."""
+what the batched prompt path of the library feeds its GEMMs with.
+
+`mutation` swaps in one deliberately wrong piece (tests use it to show that a model's logits react to that piece, i.e.
+that a parity test on that model could catch such a mistake): "no_rope" (rotary embedding skipped), "pos_plus_one"
+(the query rotated for the next position, the key for its own: relative positions off by one -- shifting queries and
+keys alike would change nothing, the rotary embedding being relative), "ctx_minus_one" (the attention leaves out the newest token), "last_only" (the attention
+sees the newest token only), "kv_head_mod" (query head i reads cached head i % kv heads instead of i // group)."""
 from __future__ import annotations
 
 import numpy as np
@@ -9,9 +15,13 @@ import numpy as np
 from . import oracle_c, oracle_np
 
 
+MUTATIONS = ("no_rope", "pos_plus_one", "ctx_minus_one", "last_only", "kv_head_mod")
+
+
 class OracleLlama:
-    def __init__(self, cfg, weights):
-        self.cfg, self.w = cfg, weights
+    def __init__(self, cfg, weights, mutation=None):
+        assert mutation is None or mutation in MUTATIONS, mutation
+        self.cfg, self.w, self.mutation = cfg, weights, mutation
         c = cfg
         self.kvh = getattr(c, "n_kv_head", 0) or c.n_head  # grouped-query attention: heads of k / v
         self.k = np.zeros((c.n_layer, c.max_tokens, self.kvh, c.head_dim), dtype=np.uint16)
@@ -32,22 +42,32 @@ class OracleLlama:
         be, bb = oracle_c.type_sizes(t)
         rb = h // be * bb
         x = oracle_c.dequant(t, raw[token * rb:(token + 1) * rb], h)
-        pos = self.pos
+        pos, mut = self.pos, self.mutation
         for l in range(c.n_layer):
             xn = oracle_c.rmsnorm(x, self.w[f"l{l}.attn_norm"][1], c.rms_eps)
             q = self._lin(f"l{l}.wq", h, h, xn, bf16_gemm).reshape(c.n_head, c.head_dim)
             kvd = self.kvh * c.head_dim
             k = self._lin(f"l{l}.wk", kvd, h, xn, bf16_gemm).reshape(self.kvh, c.head_dim)
             v = self._lin(f"l{l}.wv", kvd, h, xn, bf16_gemm).reshape(self.kvh, c.head_dim)
-            q = oracle_c.rope(q, pos, c.rope_base)
-            k = oracle_c.rope(k, pos, c.rope_base)
+            if mut != "no_rope":
+                q = oracle_c.rope(q, pos + 1 if mut == "pos_plus_one" else pos, c.rope_base)
+                k = oracle_c.rope(k, pos, c.rope_base)
             self.k[l, pos] = oracle_c.f2h(k)
             self.v[l, pos] = oracle_c.f2h(v)
             # query head i reads cached head i // (n_head / kv heads)
             rep = c.n_head // self.kvh
-            att = oracle_c.attn_decode(q[None], np.repeat(self.k[l][None, : pos + 1], rep, axis=2),
-                                       np.repeat(self.v[l][None, : pos + 1], rep, axis=2), [pos + 1],
-                                       1.0 / np.sqrt(c.head_dim))[0].reshape(h)
+            lo, hi = 0, pos + 1
+            if mut == "ctx_minus_one" and pos > 0:
+                hi = pos
+            if mut == "last_only":
+                lo = pos
+            kc, vc = self.k[l][None, lo:hi], self.v[l][None, lo:hi]
+            if mut == "kv_head_mod":
+                heads = np.arange(c.n_head) % self.kvh
+                kc, vc = kc[:, :, heads], vc[:, :, heads]
+            else:
+                kc, vc = np.repeat(kc, rep, axis=2), np.repeat(vc, rep, axis=2)
+            att = oracle_c.attn_decode(q[None], kc, vc, [hi - lo], 1.0 / np.sqrt(c.head_dim))[0].reshape(h)
             x = x + self._lin(f"l{l}.wo", h, h, att, bf16_gemm)
             xn = oracle_c.rmsnorm(x, self.w[f"l{l}.ffn_norm"][1], c.rms_eps)
             g = self._lin(f"l{l}.w_gate", f, h, xn, bf16_gemm)

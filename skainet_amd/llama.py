@@ -70,6 +70,34 @@ def random_weights(cfg: Config, seed: int):
     return w
 
 
+# Gains of the conditioned model: queries and keys of rms 2 give attention logits of spread about 4, the attention
+# branch (values 1, output projection 1.5) outweighs the feed-forward branch (gate / up 1, down 1 on a SwiGLU of rms
+# about 0.4), and the residual stream stays of order one through the stack.
+_GAINS = {"wq": 2.0, "wk": 2.0, "wv": 1.0, "wo": 1.5, "w_gate": 1.0, "w_up": 1.0, "w_down": 1.0}
+
+
+def conditioned_weights(cfg: Config, seed: int):
+    """Like random_weights, with every matrix drawn by synth.conditioned_weight: zero-centred values and a power-of-two
+    scale per matrix, so that the logits depend on positions, on the cache and on the attention (the benchmark's
+    Q4_K draws have a mean that buries those under the feed-forward output).  The model for decoder parity tests."""
+    h, f, v = cfg.hidden, cfg.ffn, cfg.vocab
+    w = {}
+    rng = np.random.default_rng(seed)
+    w["tok_embd"] = (cfg.type_embd, synth.conditioned_weight(cfg.type_embd, v, h, seed + 1, gain=np.sqrt(h)))
+    w["out_head"] = (cfg.type_head, synth.conditioned_weight(cfg.type_head, v, h, seed + 2, gain=1.0))
+    w["out_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+    kvd = cfg.kv_heads * cfg.head_dim
+    shapes = {"wq": (h, h), "wk": (kvd, h), "wv": (kvd, h), "wo": (h, h), "w_gate": (f, h), "w_up": (f, h), "w_down": (h, f)}
+    for l in range(cfg.n_layer):
+        s = seed + 100 * (l + 1)
+        for i, (name, (rows, cols)) in enumerate(shapes.items()):
+            t = cfg.matrix_type(l, name)
+            w[f"l{l}.{name}"] = (t, synth.conditioned_weight(t, rows, cols, s + i, gain=_GAINS[name]))
+        w[f"l{l}.attn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+        w[f"l{l}.ffn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
+    return w
+
+
 class LlamaModel:
     """Device-resident model: owns the uploaded weights and the skn_llama handle."""
 

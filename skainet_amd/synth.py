@@ -168,3 +168,40 @@ def checksum(arr):
     for byte in a[::step].tolist():
         h = ((h ^ byte) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
     return f"{h:016x}:{a.size}"
+
+
+# ---- conditioned weights -------------------------------------------------------------------------------------
+# The benchmark's Q4_K draws (d * sc * q - dmin * m with independent scales and minima) have a positive mean about
+# two thirds of their spread: stacked into a decoder they drown the attention path in the feed-forward output.  The
+# generator below keeps the block formats and their full field ranges but centres the values on zero and scales
+# every d by a power of two, so that a matrix maps a unit-rms vector to a vector of a chosen rms ("gain").  It is
+# what decoder tests use when the result must depend on positions, cache contents and attention.
+
+# rms of a weight drawn by the base generators after centring, per format, at their stated d scales
+# (Q8_0: d * q, q uniform in [-127, 127], d = |N| * 0.02; Q6_K: d * sc * (q - 32); the offset formats centred as below)
+_CENTRED_RMS = {Q8_0: 1.4722, Q6_K: 3.4150, Q4_K: 1.6834, Q5_K: 3.3717, Q4_0: 0.046368, Q5_0: 0.092466}
+_D_FIELDS = {Q8_0: (34, (0,)), Q6_K: (210, (208,)), Q4_K: (144, (0, 2)), Q5_K: (176, (0, 2)), Q4_0: (18, (0,)),
+             Q5_0: (22, (0,))}
+
+
+def conditioned_weight(qtype, n_rows, k, seed, gain=1.0):
+    """Raw block bytes of an [n_rows, k] weight whose values are centred on zero and whose rows map a unit-rms
+    vector to outputs of rms about `gain` (to the nearest power of two in d).  Q4_K / Q5_K: every sub-block gets
+    m = sc and the superblock dmin = f16(7.5 d) / f16(15.5 d), i.e. values d * sc * (q - 7.5) / (q - 15.5)."""
+    if qtype not in _CENTRED_RMS:
+        raise ValueError(f"no conditioned generator for ggml type {qtype}")
+    raw = weight(qtype, n_rows, k, seed)
+    nbytes, d_at = _D_FIELDS[qtype]
+    b = raw.reshape(-1, nbytes).copy()
+    factor = 2.0 ** np.round(np.log2(gain / (_CENTRED_RMS[qtype] * np.sqrt(k))))
+    d = b[:, d_at[0]:d_at[0] + 2].copy().view(np.float16).astype(np.float32).reshape(-1) * np.float32(factor)
+    b[:, d_at[0]:d_at[0] + 2] = _f16_bytes(d)
+    if qtype in (Q4_K, Q5_K):
+        d = b[:, 0:2].copy().view(np.float16).astype(np.float32).reshape(-1)  # as stored
+        b[:, 2:4] = _f16_bytes(d * np.float32(7.5 if qtype == Q4_K else 15.5))
+        packed = b[:, 4:16]
+        sc = np.empty((b.shape[0], 8), dtype=np.uint8)  # the scales as drawn; the minima become copies of them
+        sc[:, 0:4] = packed[:, 0:4] & 63
+        sc[:, 4:8] = (packed[:, 8:12] & 0x0F) | ((packed[:, 0:4] >> 6) << 4)
+        b[:, 4:16] = pack_q4k_scales(sc, sc)
+    return b.reshape(-1)
