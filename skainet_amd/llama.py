@@ -70,17 +70,19 @@ def random_weights(cfg: Config, seed: int):
     return w
 
 
-# Gains of the conditioned model: queries and keys of rms 2 give attention logits of spread about 4, the attention
-# branch (values 1, output projection 1.5) outweighs the feed-forward branch (gate / up 1, down 1 on a SwiGLU of rms
-# about 0.4), and the residual stream stays of order one through the stack.
-_GAINS = {"wq": 2.0, "wk": 2.0, "wv": 1.0, "wo": 1.5, "w_gate": 1.0, "w_up": 1.0, "w_down": 1.0}
+# Gains of the conditioned model: queries and keys of rms about 1 give attention scores of order one (larger ones make
+# the logits hang on single fp16 roundings of cached keys), the attention branch (values 1, output projection 1.5)
+# outweighs the feed-forward branch (gate / up 1, down 1 on a SwiGLU of rms about 0.4), and the residual stream stays
+# of order one through the stack.
+_GAINS = {"wq": 1.0, "wk": 1.0, "wv": 1.0, "wo": 1.5, "w_gate": 1.0, "w_up": 1.0, "w_down": 1.0}
 
 
-def conditioned_weights(cfg: Config, seed: int):
+def conditioned_weights(cfg: Config, seed: int, gains=None):
     """Like random_weights, with every matrix drawn by synth.conditioned_weight: zero-centred values and a power-of-two
     scale per matrix, so that the logits depend on positions, on the cache and on the attention (the benchmark's
     Q4_K draws have a mean that buries those under the feed-forward output).  The model for decoder parity tests."""
     h, f, v = cfg.hidden, cfg.ffn, cfg.vocab
+    gains = {**_GAINS, **(gains or {})}
     w = {}
     rng = np.random.default_rng(seed)
     w["tok_embd"] = (cfg.type_embd, synth.conditioned_weight(cfg.type_embd, v, h, seed + 1, gain=np.sqrt(h)))
@@ -92,7 +94,7 @@ def conditioned_weights(cfg: Config, seed: int):
         s = seed + 100 * (l + 1)
         for i, (name, (rows, cols)) in enumerate(shapes.items()):
             t = cfg.matrix_type(l, name)
-            w[f"l{l}.{name}"] = (t, synth.conditioned_weight(t, rows, cols, s + i, gain=_GAINS[name]))
+            w[f"l{l}.{name}"] = (t, synth.conditioned_weight(t, rows, cols, s + i, gain=gains[name]))
         w[f"l{l}.attn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
         w[f"l{l}.ffn_norm"] = (None, (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float32))
     return w

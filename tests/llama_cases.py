@@ -23,6 +23,17 @@ DECODE_TOL = 2e-3   # the decoder tests' bound for two layers (1e-3 per operatio
 PROMPT_TOL = 5e-3   # prompt pass: bf16 activations in every projection
 
 
+def logit_err(got, want):
+    """max |got - want| / max |want|.  The logits of these models are centred on zero, so some are always within
+    rounding of it and an error relative to each logit's own size measures nothing but those; and the cached keys
+    and values are fp16, so a difference in the last bit of an fp32 key flips an fp16 rounding now and then, which
+    moves every later logit by about 1e-4 of the largest (test_oracle_llama_sensitivity.py measures both)."""
+    import numpy as np
+
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    return float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+
+
 def tokens(n, vocab, seed=1):
     import numpy as np
 

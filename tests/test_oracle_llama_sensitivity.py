@@ -1,14 +1,19 @@
-"""That the decoder parity tests can fail: on the conditioned models of tests/llama_cases.py every deliberately wrong
-piece of the oracle (rotary embedding dropped, relative position off by one, attention without the newest token,
-attention over the newest token only, the wrong cached head for a query head) moves the logits by at least ten times
-the tolerance the GPU tests hold -- at every step from the third on, in the metric those tests use.  On the
-benchmark's own Q4_K draws (positive mean) the same mistakes are invisible, which is why those models only check
-the matvec / GEMM / norm chain.  CPU only."""
+"""That the decoder parity tests can fail.
+
+On the conditioned models of tests/llama_cases.py every deliberately wrong piece of the oracle -- rotary embedding
+dropped, relative position off by one, attention without the newest token, attention over the newest token only, the
+wrong cached head for a query head -- moves the logits by at least ten times the tolerance of the GPU tests at every
+step from the third on (prompt path, whose tolerance is wider: at nine steps in ten, and by five tolerances at every
+step), in the metric those tests use.  In the other direction, an oracle whose every operation carries fp32-sized
+noise stays a factor of four inside the tolerance: the tolerance separates rounding from mistakes with room on both
+sides.  On the benchmark's own Q4_K draws (positive mean) the same mistakes are nearly invisible, which is why those
+models only check the matvec / GEMM / norm chain.  CPU only."""
 import numpy as np
 import pytest
 
-from llama_cases import CASES, DECODE_TOL, PROMPT_TOL, SEED, tokens
-from oracle import oracle_np
+import oracle.llama_oracle as llama_oracle
+from llama_cases import CASES, DECODE_TOL, PROMPT_TOL, SEED, logit_err, tokens
+from oracle import oracle_c, oracle_np
 from oracle.llama_oracle import MUTATIONS, OracleLlama
 from skainet_amd import llama
 
@@ -33,29 +38,100 @@ def test_every_mutation_moves_the_logits_of_the_conditioned_models(case):
         for m in MUTATIONS:
             if m == "kv_head_mod" and cfg.kv_heads in (1, cfg.n_head):
                 continue  # (i % kv heads == i // group there)
-            errs = [oracle_np.rel_err(a, b) for a, b in zip(_logits(cfg, w, toks, m, bf16=bf16), base)]
-            assert min(errs[2:]) >= 10 * tol, (m, bf16, min(errs[2:]))
+            errs = np.array([logit_err(a, b) for a, b in zip(_logits(cfg, w, toks, m, bf16=bf16), base)])[2:]
+            if bf16:
+                assert errs.min() >= 5 * tol and np.quantile(errs, 0.1) >= 10 * tol, (m, errs.min())
+            else:
+                assert errs.min() >= 10 * tol, (m, errs.min())
+            assert errs.max() >= 50 * tol
 
 
-def test_attention_logits_of_the_conditioned_model_are_of_order_one_to_ten():
+class _Noisy:
+    """oracle_c with relative Gaussian noise of the given size on the result of every decoder operation."""
+
+    def __init__(self, noise, seed):
+        self.noise, self.rng = noise, np.random.default_rng(seed)
+
+    def __getattr__(self, name):
+        f = getattr(oracle_c, name)
+        if name not in ("matvec_q", "attn_decode", "rmsnorm", "rope", "swiglu"):
+            return f
+
+        def noisy(*a, **k):
+            y = f(*a, **k)
+            return (y * (1.0 + self.noise * self.rng.standard_normal(y.shape))).astype(np.float32)
+        return noisy
+
+
+@pytest.mark.parametrize("case", ["q4_k", "q4_k_kv1", "q8_0"])
+def test_fp32_sized_noise_stays_inside_the_tolerance(case, monkeypatch):
+    """2e-7 relative noise on every operation's output (what fp32 accumulation differs from fp64 by) moves the
+    logits by up to 1e-4 of the largest -- not 1e-6: now and then it flips the fp16 rounding of a cached key, and
+    every later attention score of that key moves by 2^-11 of one product.  Still a factor of four inside the bound."""
+    cfg = CASES[case]
+    w = llama.conditioned_weights(cfg, SEED)
+    toks = tokens(44, cfg.vocab)
+    base = _logits(cfg, w, toks)
+    worst = 0.0
+    for seed in range(3):
+        monkeypatch.setattr(llama_oracle, "oracle_c", _Noisy(2e-7, seed))
+        worst = max(worst, max(logit_err(a, b) for a, b in zip(_logits(cfg, w, toks), base)))
+        monkeypatch.setattr(llama_oracle, "oracle_c", oracle_c)
+    assert 1e-6 < worst < DECODE_TOL / 4, worst
+
+
+def test_fp32_sized_noise_on_the_prompt_path_stays_inside_its_tolerance(monkeypatch):
+    """With every projection's input rounded to bf16 the same noise flips bf16 roundings (2^-9 of one activation
+    each): 1.5e-3 to 2.5e-3 of the largest logit after a 41-token prompt -- the prompt tolerance is 5e-3 for that
+    reason, and the mutations are held to five of those at every step above."""
+    cfg = CASES["q4_k_kv2"]
+    w = llama.conditioned_weights(cfg, SEED)
+    prompt = tokens(41, cfg.vocab, seed=2)
+    o = OracleLlama(cfg, w)
+    o.prefill(prompt, bf16_gemm=True)
+    base = o.logits.copy()
+    for seed in range(3):
+        monkeypatch.setattr(llama_oracle, "oracle_c", _Noisy(2e-7, seed))
+        o = OracleLlama(cfg, w)
+        o.prefill(prompt, bf16_gemm=True)
+        monkeypatch.setattr(llama_oracle, "oracle_c", oracle_c)
+        assert 1e-4 < logit_err(o.logits, base) < PROMPT_TOL
+
+
+def test_attention_scores_of_the_conditioned_model_are_of_order_one_to_ten():
     cfg = CASES["q4_k"]
     w = llama.conditioned_weights(cfg, SEED)
     o = OracleLlama(cfg, w)
-    for t in tokens(20, cfg.vocab):
+    for t in tokens(30, cfg.vocab):
         o.step(t)
-    from oracle import oracle_c
-
     # keys and queries are drawn alike (same gain), so key-key products have the spread of the attention's scores
-    k = oracle_c.h2f(o.k[0, :20])                      # [tokens, heads, dim]
-    s = np.einsum("thd,shd->hts", k, k) / np.sqrt(cfg.head_dim)
-    off = s[:, ~np.eye(20, dtype=bool)]
-    assert 1.0 < off.std() < 10.0, off.std()
+    for layer in range(cfg.n_layer):
+        k = oracle_c.h2f(o.k[layer, :30])                      # [tokens, heads, dim]
+        s = np.einsum("thd,shd->hts", k, k) / np.sqrt(cfg.head_dim)
+        off = s[:, ~np.eye(30, dtype=bool)]
+        assert 1.0 < off.std() < 10.0, off.std()
+
+
+def test_conditioned_weights_are_centred_and_scaled():
+    """synth.conditioned_weight: mean within a tenth of the spread, and rows map a unit-rms vector to about `gain`
+    (d is scaled by a power of two, so to within a factor of sqrt 2)."""
+    from skainet_amd import synth
+
+    for t in (8, 14, 12, 13, 2, 6):
+        for gain in (1.0, 3.0):
+            wts = oracle_c.dequant(t, synth.conditioned_weight(t, 128, 1024, 5, gain=gain)).astype(np.float64)
+            assert abs(wts.mean()) < 0.1 * wts.std(), t
+            assert gain / 1.5 < np.sqrt((wts ** 2).mean() * 1024) < gain * 1.5, t
+    blocks = synth.conditioned_weight(12, 4, 512, 1).reshape(-1, 144)
+    assert blocks[:, 16:].min() == 0 and blocks[:, 16:].max() == 255      # all sixteen nibble values in use
+    assert (blocks[:, 2:4].view(np.float16) > 0).all()                    # dmin in use: the minima are not zero
 
 
 def test_benchmark_draws_hide_the_same_mutations():
     """The reason for the conditioned models: with synth.weight's Q4_K blocks the feed-forward output buries the
     attention branch: with the rotary embedding dropped, more than half of the steps stay below the bar of ten
-    tolerances that the conditioned models clear at every step (there the smallest change is a thousand tolerances)."""
+    tolerances that the conditioned models clear at every step -- in the benchmark models' own metric, which is
+    relative to each logit (theirs are all of one sign and size)."""
     cfg = CASES["q4_k"]
     w = llama.random_weights(cfg, seed=3)
     toks = tokens(12, cfg.vocab)
