@@ -135,3 +135,45 @@ def test_several_steps_per_call_equal_one_step_per_call(hip):
         tok = want
     a.free()
     b.free()
+
+
+def test_hidden_4096_at_the_benchmark_length_matches_the_oracle_golden(hip, golden_dir):
+    """Four distinct layers of the 7B model's width (hidden 4096, FFN 11008, 32 heads x 128, vocabulary 32000) on
+    conditioned weights, 512-token prompt and 128 decode steps, against tests/golden/conditioned_4layer_512_128.npz
+    (tests/golden/make_conditioned_golden.py: ten minutes of the CPU oracle).  Here the prompt GEMMs (M = 512), the
+    prompt attention, the 2 -> 3 page boundary at 512 and the decode attention at contexts 513 to 640 all shape
+    logits that the golden's own mutation record says move by at least 0.07 of the largest logit when the rotary
+    embedding or the attention window is wrong.  Decode steps are fed the oracle's tokens.
+
+    Tolerance: 5e-3 for two layers with bf16 prompt activations, times sqrt(4 / 2) for four: 7e-3 of the largest
+    logit, for the prompt's last row and for every stored step (whose cache was written by the prompt path)."""
+    import os
+
+    gold = np.load(os.path.join(golden_dir, "conditioned_4layer_512_128.npz"))
+    tol = PROMPT_TOL * np.sqrt(int(gold["n_layer"]) / 2)
+    for m in ("no_rope", "pos_plus_one", "ctx_minus_one", "last_only"):
+        assert float(gold[f"mutation_{m}_min"]) >= 9 * tol, m  # (recorded by the script that wrote the golden)
+    stride = int(gold["stride"])
+    cfg = llama.Config(n_layer=int(gold["n_layer"]), max_tokens=1024)
+    model = llama.LlamaModel(hip, cfg, weights=llama.conditioned_weights(cfg, int(gold["seed"])))
+
+    def check(tag, got_token):
+        want, absmax = gold[f"{tag}_sample"].astype(np.float64), float(gold[f"{tag}_absmax"])
+        err = float(np.max(np.abs(model.logits()[::stride].astype(np.float64) - want)) / absmax)
+        assert err <= tol, (tag, err)
+        if float(gold[f"{tag}_margin"]) > 2 * tol * absmax:
+            assert got_token == int(gold[f"{tag}_argmax"]), tag
+        return err
+
+    errs = {"prefill": check("prefill", model.prefill(gold["prompt"].tolist()))}
+    fed = [int(gold["first"])] + gold["tokens"].tolist()
+    assert len(set(fed)) > 40  # (a golden whose greedy tokens repeat one token would say little)
+    same = 0
+    for i in range(128):
+        tok = model.decode(fed[i], 1)[0]
+        same += tok == fed[i + 1]
+        if f"step{i}_sample" in gold.files:
+            errs[f"step{i}"] = check(f"step{i}", tok)
+    print("logit errors:", {k: f"{v:.2e}" for k, v in errs.items()}, "greedy tokens equal:", same, "of 128")
+    assert same >= 120  # (steps whose top two logits are closer than the tolerance may differ)
+    model.free()
