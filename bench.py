@@ -195,37 +195,6 @@ def bench_gemm(ctx, qtype, m, n, k, reps=20, expanded=False):
             "frac_mfma_f16_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)}
 
 
-def machine_figures(ctx):
-    """Figures of the machine that the GEMM's design argument uses: time per matrix instruction with independent
-    vector instructions behind it, the rate at which operand fragments arrive in a compute unit's registers, and the
-    cost of each part of the Q4_K GEMM's loop next to its matrix instructions."""
-    scratch = ctx.alloc(512 * 1024)
-    flag = ctx.alloc(16)
-    overlap = {f"{w}_wavefronts_per_simd": {str(nv): round(ctx.test_mfma_valu_overlap(w, nv, scratch), 2) for nv in (0, 2, 4, 6, 7, 8, 12)}
-               for w in (1, 2)}
-    delivery = {}
-    for mib in (8, 64):
-        data = ctx.alloc(mib << 20)
-        ctx.memset(data, 1, mib << 20)
-        delivery[f"{mib}_mib_of_distinct_data"] = {str(sh): round(ctx.test_fragment_delivery(sh, data, mib, flag), 1) for sh in (1, 2, 4, 8)}
-        data.free()
-    # the Q4_K GEMM's loop with parts left out (two passes: the clock of a box moves under such a load)
-    data = ctx.alloc(64 << 20)
-    ctx.memset(data, 0x3c, 64 << 20)
-    parts = (("matrix instructions only", 0), ("+ nibble decode from LDS", 3), ("+ activation fragments from memory", 7),
-             ("+ header unpack per superblock", 15), ("+ accumulator rescale", 31), ("+ min term (the whole loop)", 63),
-             ("whole loop without the fragments from memory", 59), ("whole loop without the rescale", 47),
-             ("whole loop without the header unpack", 55), ("matrix instructions and fragments only", 4))
-    loop = {name: [round(ctx.test_q4k_gemm_loop(p, data, scratch), 1) for _ in range(2)] for name, p in parts}
-    data.free()
-    scratch.free()
-    flag.free()
-    return {"mode": "machine",
-            "ns_per_mfma_32x32x16_f16_and_simd_by_vector_instructions_behind_it": overlap,
-            "fragment_gbs_per_compute_unit_by_wavefronts_sharing_a_stream": delivery,
-            "q4k_gemm_loop_ns_per_k_step_and_simd": loop}
-
-
 def matvec_timeline(ctx, n, k, reps=20, queued=12):
     """In-kernel timeline of the headline kernel (its measuring build, skn_test_matvec_q4k_stamps): `queued` launches back
     to back over rotating weight copies, the stamps of the last one; percentiles over its wavefronts, averaged over
@@ -376,7 +345,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline", "machine"], default="bench",
+    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline"], default="bench",
                     help="decode / attention / gemm: only that leg (for kernel traces).  timeline: the headline kernel's in-kernel time stamps.  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
     ap.add_argument("--no-graph", action="store_true",
@@ -391,10 +360,6 @@ def main():
     if args.no_graph:
         ctx.set_option("llama.graph", 0)
     n, k = 4096, 11008
-    if args.mode == "machine":
-        print(json.dumps(machine_figures(ctx)))
-        ctx.close()
-        return
     if args.mode == "timeline":
         print(json.dumps(matvec_timeline(ctx, n, k)))
         ctx.close()

@@ -14,7 +14,7 @@ import java.lang.foreign.ValueLayout.JAVA_LONG
 import java.lang.invoke.MethodHandle
 
 object SknLib {
-    const val ABI_VERSION = 2
+    const val ABI_VERSION = 3
     const val OK = 0
     const val ERR_ARG = -1
     const val ERR_TYPE = -2
@@ -84,11 +84,13 @@ object SknLib {
     val llamaPrefill: MethodHandle = h("skn_llama_prefill", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS, JAVA_INT, ADDRESS))
     val llamaDecode: MethodHandle = h("skn_llama_decode", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS))
     val llamaLogits: MethodHandle = h("skn_llama_logits", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
+    val synthWeight: MethodHandle = h("skn_synth_weight", FunctionDescriptor.of(JAVA_INT, JAVA_INT, JAVA_LONG, JAVA_LONG, JAVA_LONG, ADDRESS, JAVA_LONG))
+    val synthActivationF32: MethodHandle = h("skn_synth_activation_f32", FunctionDescriptor.of(JAVA_INT, JAVA_LONG, JAVA_LONG, ADDRESS))
+    val synthActivationBf16: MethodHandle = h("skn_synth_activation_bf16", FunctionDescriptor.of(JAVA_INT, JAVA_LONG, JAVA_LONG, ADDRESS))
+    val synthKvF16: MethodHandle = h("skn_synth_kv_f16", FunctionDescriptor.of(JAVA_INT, JAVA_LONG, JAVA_LONG, ADDRESS))
+    val synthChecksum: MethodHandle = h("skn_synth_checksum", FunctionDescriptor.of(JAVA_LONG, ADDRESS, JAVA_LONG))
     val testFusedMatvec: MethodHandle = h("skn_test_fused_matvec", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, JAVA_FLOAT, ADDRESS, ADDRESS, ADDRESS, JAVA_FLOAT))
     val testMatvecQ4kStamps: MethodHandle = h("skn_test_matvec_q4k_stamps", FunctionDescriptor.of(JAVA_INT, ADDRESS, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
-    val testMfmaValuOverlap: MethodHandle = h("skn_test_mfma_valu_overlap", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, JAVA_INT, ADDRESS, ADDRESS))
-    val testFragmentDelivery: MethodHandle = h("skn_test_fragment_delivery", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, ADDRESS))
-    val testQ4kGemmLoop: MethodHandle = h("skn_test_q4k_gemm_loop", FunctionDescriptor.of(JAVA_INT, ADDRESS, JAVA_INT, ADDRESS, ADDRESS, ADDRESS))
 
     init {
         val v = abiVersion.invokeExact() as Int

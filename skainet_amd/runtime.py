@@ -56,6 +56,11 @@ class LlamaWeights(C.Structure):
 
 _SIGNATURES = {
     # name: (restype, argtypes)
+    "skn_synth_weight": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_uint64, C.c_void_p, C.c_size_t]),
+    "skn_synth_activation_f32": (C.c_int, [C.c_int64, C.c_uint64, C.c_void_p]),
+    "skn_synth_activation_bf16": (C.c_int, [C.c_int64, C.c_uint64, C.c_void_p]),
+    "skn_synth_kv_f16": (C.c_int, [C.c_int64, C.c_uint64, C.c_void_p]),
+    "skn_synth_checksum": (C.c_uint64, [C.c_void_p, C.c_size_t]),
     "skn_abi_version": (C.c_int, []),
     "skn_init": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
     "skn_shutdown": (None, [C.c_void_p]),
@@ -87,9 +92,6 @@ _SIGNATURES = {
     "skn_gemm_expand": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
     "skn_gemm_expanded": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p]),
     "skn_test_matvec_q4k_stamps": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]),
-    "skn_test_mfma_valu_overlap": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
-    "skn_test_fragment_delivery": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.POINTER(C.c_double)]),
-    "skn_test_q4k_gemm_loop": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]),
     "skn_kv_create": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_void_p)]),
     "skn_kv_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "skn_kv_reset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
@@ -156,6 +158,42 @@ def row_bytes(ggml_type, k):
     if rc < 0:
         raise SknError(int(rc), lib.skn_last_error(None).decode())
     return int(rc)
+
+
+def synth_weight(ggml_type, n_rows, k, seed):
+    """skn_synth_weight: the library's seeded blocks of an [n_rows, k] weight (host array; needs no device)."""
+    lib = load_library()
+    out = np.empty(n_rows * row_bytes(ggml_type, k), dtype=np.uint8)
+    rc = lib.skn_synth_weight(ggml_type, n_rows, k, seed, out.ctypes.data, out.nbytes)
+    if rc != OK:
+        raise SknError(rc, lib.skn_last_error(None).decode())
+    return out
+
+
+def _synth_vector(name, dtype, n, seed):
+    lib = load_library()
+    out = np.empty(n, dtype=dtype)
+    rc = getattr(lib, name)(n, seed, out.ctypes.data)
+    if rc != OK:
+        raise SknError(rc, lib.skn_last_error(None).decode())
+    return out
+
+
+def synth_activation_f32(n, seed):
+    return _synth_vector("skn_synth_activation_f32", np.float32, n, seed)
+
+
+def synth_activation_bf16(n, seed):
+    return _synth_vector("skn_synth_activation_bf16", np.uint16, n, seed)
+
+
+def synth_kv_f16(n, seed):
+    return _synth_vector("skn_synth_kv_f16", np.uint16, n, seed)
+
+
+def synth_checksum(arr):
+    a = np.ascontiguousarray(arr)
+    return int(load_library().skn_synth_checksum(a.ctypes.data, a.nbytes))
 
 
 class DeviceBuffer:
@@ -375,21 +413,6 @@ class Context:
     def test_matvec_q4k_stamps(self, w_dev, n, k, x_dev, y_dev, stamps_dev):
         """The Q4_K matvec with the kernel's measuring build: eight 64-bit stamps per row in stamps_dev."""
         self._check(self.lib.skn_test_matvec_q4k_stamps(self.handle, _ptr(w_dev), n, k, _ptr(x_dev), _ptr(y_dev), _ptr(stamps_dev)))
-
-    def test_mfma_valu_overlap(self, waves_per_simd, valu_per_mfma, scratch_dev):
-        out = C.c_double()
-        self._check(self.lib.skn_test_mfma_valu_overlap(self.handle, waves_per_simd, valu_per_mfma, _ptr(scratch_dev), C.byref(out)))
-        return out.value
-
-    def test_fragment_delivery(self, share, data_dev, data_mib, flag_dev):
-        out = C.c_double()
-        self._check(self.lib.skn_test_fragment_delivery(self.handle, share, _ptr(data_dev), data_mib, _ptr(flag_dev), C.byref(out)))
-        return out.value
-
-    def test_q4k_gemm_loop(self, parts, data_dev, scratch_dev):
-        out = C.c_double()
-        self._check(self.lib.skn_test_q4k_gemm_loop(self.handle, parts, _ptr(data_dev), _ptr(scratch_dev), C.byref(out)))
-        return out.value
 
     def rmsnorm(self, x_dev, w_dev, rows, n, eps, y_dev):
         self._check(self.lib.skn_rmsnorm(self.handle, _ptr(x_dev), _ptr(w_dev), rows, n, eps, _ptr(y_dev)))

@@ -205,3 +205,91 @@ def conditioned_weight(qtype, n_rows, k, seed, gain=1.0):
         sc[:, 4:8] = (packed[:, 8:12] & 0x0F) | ((packed[:, 0:4] >> 6) << 4)
         b[:, 4:16] = pack_q4k_scales(sc, sc)
     return b.reshape(-1)
+
+
+# ---- the library's generator, restated ------------------------------------------------------------------------
+# skn_synth_* (csrc/synth.hip) produce the benchmark inputs inside the library so that C, ctypes and Kotlin harnesses
+# draw identical bytes.  The functions below are the same algorithm in NumPy -- counter-based SplitMix64 words, integer
+# arithmetic up to the final conversion -- and tests/test_synth_abi.py holds the two equal byte for byte.
+
+_G = np.uint64(0x9E3779B97F4A7C15)
+
+
+def _mix(z):
+    z = np.asarray(z, dtype=np.uint64)
+    z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return z ^ (z >> np.uint64(31))
+
+
+def _words(seed, stream, first, count):
+    """Words first .. first + count - 1 of a stream."""
+    with np.errstate(over="ignore"):
+        base = _mix(np.array([seed], dtype=np.uint64) + _G * np.uint64(stream + 1))[0]
+        idx = np.arange(first + 1, first + count + 1, dtype=np.uint64)
+        return _mix(base + _G * idx)
+
+
+def _stream_bytes(seed, stream, n):
+    return _words(seed, stream, 0, (n + 7) // 8).astype("<u8").view(np.uint8)[:n]
+
+
+def _stream_normal(seed, stream, n):
+    w = _words(seed, stream, 0, 6 * n).reshape(n, 6)
+    total = ((w & np.uint64(0xFFFFFFFF)) + (w >> np.uint64(32))).sum(axis=1, dtype=np.uint64)
+    return (total.astype(np.int64) - np.int64(6 << 32)).astype(np.float64) * (1.0 / 4294967296.0)
+
+
+def _f16_via_f32(values):
+    return np.ascontiguousarray(values.astype(np.float32).astype(np.float16)).view(np.uint8).reshape(-1, 2)
+
+
+def lib_weight(qtype, n_rows, k, seed):
+    """What skn_synth_weight writes: raw blocks of an [n_rows, k] Q8_0 / Q4_K / Q6_K weight."""
+    if qtype not in (Q8_0, Q4_K, Q6_K):
+        raise ValueError(f"ggml type {qtype} has no generator (Q8_0, Q4_K, Q6_K)")
+    elems, nbytes = BLOCK[qtype]
+    if k % elems:
+        raise ValueError(f"row size {k} is not a multiple of the block size {elems}")
+    nb = n_rows * (k // elems)
+    b = np.empty((nb, nbytes), dtype=np.uint8)
+    if nb == 0:
+        return b.reshape(-1)
+    if qtype == Q8_0:
+        b[:, 0:2] = _f16_via_f32(np.abs(_stream_normal(seed, 1, nb)) * 0.02)
+        u = _stream_bytes(seed, 0, 64 * nb).reshape(nb, 32, 2).astype(np.uint32)
+        u16 = u[:, :, 0] | (u[:, :, 1] << 8)
+        b[:, 2:34] = (((u16 * 255) >> 16).astype(np.int32) - 127).astype(np.int8).view(np.uint8)
+    elif qtype == Q4_K:
+        b[:, 0:2] = _f16_via_f32(np.abs(_stream_normal(seed, 1, nb)) * 0.01)
+        b[:, 2:4] = _f16_via_f32(np.abs(_stream_normal(seed, 2, nb)) * 0.005)
+        v = _stream_bytes(seed, 3, 16 * nb).reshape(nb, 16) & 63
+        b[:, 4:16] = pack_q4k_scales(v[:, 0:8], v[:, 8:16])
+        b[:, 16:144] = _stream_bytes(seed, 0, 128 * nb).reshape(nb, 128)
+    else:
+        b[:, 0:192] = _stream_bytes(seed, 0, 192 * nb).reshape(nb, 192)
+        v = _stream_bytes(seed, 3, 16 * nb).reshape(nb, 16) & 63
+        b[:, 192:208] = (v.astype(np.int16) - 32).astype(np.int8).view(np.uint8)
+        b[:, 208:210] = _f16_via_f32(np.abs(_stream_normal(seed, 1, nb)) * 0.01)
+    return b.reshape(-1)
+
+
+def lib_activation_f32(n, seed):
+    return _stream_normal(seed, 0, n).astype(np.float32)
+
+
+def lib_activation_bf16(n, seed):
+    return f32_to_bf16_bits(lib_activation_f32(n, seed))
+
+
+def lib_kv_f16(n, seed):
+    return lib_activation_f32(n, seed).astype(np.float16).view(np.uint16)
+
+
+def lib_checksum(arr):
+    """FNV-1a 64 over every byte (skn_synth_checksum); vectorised: h_n = (h_(n-1) ^ b_n) * P has no closed form, so
+    this walks the bytes in Python and is meant for small buffers."""
+    h = 0xCBF29CE484222325
+    for byte in np.ascontiguousarray(arr).view(np.uint8).reshape(-1).tolist():
+        h = ((h ^ byte) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+    return h

@@ -18,7 +18,7 @@
 
 static int host_leg(void) {
     int elems = 0, bytes = 0;
-    CHECK(skn_abi_version() == 2);
+    CHECK(skn_abi_version() == 3);
     CHECK(skn_type_block(SKN_TYPE_Q4_K, &elems, &bytes) == SKN_OK && elems == 256 && bytes == 144);
     CHECK(skn_type_block(SKN_TYPE_Q8_0, &elems, &bytes) == SKN_OK && elems == 32 && bytes == 34);
     CHECK(skn_type_block(SKN_TYPE_Q6_K, &elems, &bytes) == SKN_OK && elems == 256 && bytes == 210);
@@ -26,6 +26,17 @@ static int host_leg(void) {
     CHECK(skn_row_bytes(SKN_TYPE_Q4_K, 100) == SKN_ERR_SHAPE);
     CHECK(strstr(skn_last_error(NULL), "is not a multiple of block size (256)") != NULL);
     CHECK(strcmp(skn_status_string(SKN_ERR_POOL), skn_status_string(SKN_OK)) != 0);
+    /* the library's seeded generators: the checksums tests/test_synth_abi.py holds for the same calls */
+    {
+        static uint8_t w[2 * 2 * 144];
+        static float x[512];
+        CHECK(skn_row_bytes(SKN_TYPE_Q4_K, 512) * 2 == (long long)sizeof w);
+        CHECK(skn_synth_weight(SKN_TYPE_Q4_K, 2, 512, 42u, w, sizeof w) == SKN_OK);
+        CHECK(skn_synth_checksum(w, sizeof w) == 0xB1D64B923C1648B4ull);
+        CHECK(skn_synth_activation_f32(512, 42u, x) == SKN_OK);
+        CHECK(skn_synth_checksum(x, sizeof x) == 0x9A9CFB33CCC7FEA4ull);
+        CHECK(skn_synth_weight(SKN_TYPE_Q4_0, 2, 512, 42u, w, sizeof w) == SKN_ERR_TYPE);
+    }
     return 0;
 }
 

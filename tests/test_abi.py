@@ -85,7 +85,7 @@ def test_format_table_matches_reference_constants():
 
 def test_status_strings_and_version():
     lib = runtime.load_library()
-    assert lib.skn_abi_version() == 2
+    assert lib.skn_abi_version() == 3
     assert lib.skn_status_string(0) == b"ok"
     assert lib.skn_status_string(-3) == b"shape mismatch"
     assert lib.skn_status_string(-99) == b"unknown status"

@@ -271,44 +271,3 @@ def test_gemm_expanded_errors(hip):
     assert hip.gemm_expanded_bytes(Q6_K, 0, 256) == 0
     hip.gemm_expanded(buf, 0, 256, buf, 2, buf)  # nothing to do
     buf.free()
-
-
-def test_machine_measurements_run(hip):
-    """The two machine figures of `bench.py --mode machine`: they run, and come out in the range the design argues from
-    (a matrix instruction of 32 clocks, vector instructions that hide only up to a point, fragment rates of a compute
-    unit between L2 and vector-cache speed)."""
-    scratch, flag, data = hip.alloc(512 * 1024), hip.alloc(16), hip.alloc(8 << 20)
-    hip.memset(data, 1, 8 << 20)
-    alone = hip.test_mfma_valu_overlap(2, 0, scratch)
-    loaded = hip.test_mfma_valu_overlap(2, 12, scratch)
-    assert 5.0 < alone < 60.0 and alone < loaded < 6 * alone
-    distinct = hip.test_fragment_delivery(1, data, 8, flag)
-    shared = hip.test_fragment_delivery(8, data, 8, flag)
-    assert 20.0 < distinct < 1000.0 and shared > 0.7 * distinct
-    big = hip.alloc(64 << 20)
-    hip.memset(big, 0x3c, 64 << 20)
-    bare, whole = hip.test_q4k_gemm_loop(0, big, scratch), hip.test_q4k_gemm_loop(63, big, scratch)
-    assert 40.0 < bare < 600.0 and bare < whole < 8 * bare
-    with pytest.raises(runtime.SknError, match="not built"):
-        hip.test_q4k_gemm_loop(5, big, scratch)
-    big.free()
-    with pytest.raises(runtime.SknError, match="not built"):
-        hip.test_mfma_valu_overlap(1, 5, scratch)
-    with pytest.raises(runtime.SknError, match="share must be"):
-        hip.test_fragment_delivery(3, data, 8, flag)
-    for b in (scratch, flag, data):
-        b.free()
-
-
-def test_gemm_errors(hip):
-    buf = hip.alloc(1 << 16)
-    with pytest.raises(runtime.SknError) as e:
-        hip.gemm_q(Q4_K, buf, 4, 200, buf, 2, buf)
-    assert e.value.code == runtime.ERR_SHAPE
-    with pytest.raises(runtime.SknError) as e:
-        hip.gemm_q(16, buf, 4, 256, buf, 2, buf)
-    assert e.value.code == runtime.ERR_TYPE
-    with pytest.raises(runtime.SknError) as e:
-        hip.gemm_q(Q4_K, None, 4, 256, buf, 2, buf)
-    assert e.value.code == runtime.ERR_ARG
-    hip.gemm_q(Q4_K, buf, 4, 256, buf, 0, buf)  # no activation rows: nothing to do
