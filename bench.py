@@ -313,7 +313,23 @@ def cpu_baseline(qtype, n, k, budget_s=10.0):
     t1 = time.perf_counter()
     oracle_c.matvec_q(qtype, raw, n, k, x, reference_algorithm=True)
     ref_alg = time.perf_counter() - t1
+    # the same oracle on one thread
+    oracle_c.set_num_threads(1)
+    try:
+        t2 = time.perf_counter()
+        for _ in range(3):
+            oracle_c.matvec_q(qtype, raw, n, k, x)
+        single = (time.perf_counter() - t2) / 3
+    finally:
+        oracle_c.set_num_threads(cores)
     nbytes = matvec_bytes(qtype, n, k)
+    # The reference is Kotlin: were a JVM and a Kotlin compiler on this box, its CPU restatement
+    # (bindings/kotlin/common/CpuQuantReference.kt) could be timed beside the oracle.  Probed, never required.
+    import shutil
+
+    jvm = {tool: shutil.which(tool) for tool in ("java", "kotlinc")}
+    kotlin = ("absent (no " + " / ".join(t for t, path in jvm.items() if not path) + " on this box)" if not all(jvm.values())
+              else "java and kotlinc present; the Kotlin restatement is not compiled or run by this script")
     return {
         "value": nbytes / per / 1e9,
         "unit": "GB/s",
@@ -321,7 +337,10 @@ def cpu_baseline(qtype, n, k, budget_s=10.0):
         "kind": "port",
         "sample": f"{reps} repetitions of the full Q4_K {n}x{k} matvec ({dt:.1f} s), fp64 accumulation, OpenMP over rows",
         "ms_per_matvec": per * 1e3,
+        "single_thread_ms": single * 1e3,
+        "single_thread_gbs": nbytes / single / 1e9,
         "reference_algorithm_1thread_ms": ref_alg * 1e3,
+        "kotlin_cpu_reference": kotlin,
     }
 
 
@@ -398,6 +417,10 @@ def main():
         ctx.close()
         return
     head = bench_matvec(ctx, Q4_K, n, k, args.steps, args.warmup)
+    # What this machine streams at the headline's byte count with next to no arithmetic: the dense F16 matvec of the
+    # library over a weight of the same bytes (4096 x 3096 x 2 = the 25 362 432 bytes of the Q4_K blocks), cold like the
+    # headline (24 rotating copies).  The headline's fraction of the published peak stands beside its fraction of this.
+    rd = bench_matvec(ctx, 1, 4096, 3096, min(args.steps, 600), min(args.warmup, 50), copies=N_COPIES, seed=8100)
 
     extra = {"device": info["name"], "compute_units": info["compute_units"]}
     if not args.no_extra:
@@ -471,6 +494,14 @@ def main():
             "kernel": "matvec_q4k_kernel",
             "kernel_us": round(head["kernel_us"], 3),
             "cache_hot_gbs": round(head["hot_kernel_gbs"], 2),
+            "read_rate_same_bytes": {
+                "kernel": "dense F16 matvec 4096 x 3096 (skn_matvec_q), the same weight bytes, cold",
+                "bytes_per_launch": rd["bytes_per_launch"],
+                "kernel_us": round(rd["kernel_us"], 3),
+                "gbs": round(rd["kernel_gbs"], 2),
+                "frac": round(rd["kernel_gbs"] / HBM_PEAK_GBS, 4),
+            },
+            "frac_of_read_rate": round(head["kernel_gbs"] / rd["kernel_gbs"], 4),
         },
         "extra": extra,
     }

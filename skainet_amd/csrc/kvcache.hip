@@ -38,7 +38,9 @@ __global__ void kv_append_kernel(uint16_t* __restrict__ k_pool, uint16_t* __rest
     // in and returns the ticket counter to zero for the next launch.
     if (threadIdx.x == 0) {
         const int total = gridDim.x * gridDim.y;
-        if (__hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == total - 1) {
+        // (acquire-release at device scope: the other workgroups' reads of len are ordered before their tickets, the
+        // last holder's update after all of them, in the language's memory model and not only on this hardware)
+        if (__hip_atomic_fetch_add(ticket, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == total - 1) {
             for (int e = 0; e < (int)gridDim.x; e++) len[a.seq[e]] += 1;
             __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }

@@ -25,9 +25,10 @@ namespace {
 //   * a nibble masked in place (q & 0x000F000F, q & 0x00F000F0) is read as a pair of fp16 subnormals
 //     n * 2^-24 (or 16n * 2^-24), which v_fma_mix_f32 multiplies with the fp32 activation directly: no
 //     integer-to-float conversion, one mask per two weights, one fused multiply-add per weight;
-//   * the powers of two are folded into the staged data: the activations that meet high nibbles are stored
-//     divided by 16, the per-sub-block sums of x (for the "- dmin * m" term) multiplied by 2^-24, and the row
-//     total is multiplied by 2^24 once.
+//   * the powers of two are folded in where they cost least: a high nibble is read sixteen-fold, so the scale of
+//     its sub-block is divided by 16 (once per lane and step; x itself is staged as it is), the per-sub-block
+//     sums of x (for the "- dmin * m" term) are multiplied by 2^-24 in the staging, and the row total is
+//     multiplied by 2^24 once.
 //
 //   y = 2^24 * sum_blocks [ d * (sc_lo * A_lo + sc_hi * A_hi) - dmin * (m_lo * S_lo + m_hi * S_hi) ]
 
@@ -115,16 +116,15 @@ __device__ __forceinline__ void q4k_stage_load(const float* __restrict__ x, int 
     for (int j = 0; j < J; j++) st.v[j] = x4[min(tid + j * nthreads, n4 - 1)];
 }
 
-// Q4K: the scalings of the Q4_K kernel.  Otherwise (Q8_0): x is stored as is and the half-column sums are
-// multiplied by 128, the offset that turns the signed quants into unsigned bytes.
-// HI: the bit of the float4's position among the lane's sixteen that tells a high-nibble one (8: the second 32 of
-// the 64 activations, as in Q4_K / Q5_K; 4: elements 16..31 of each block of 32, as in Q4_0 / Q4_1).
+// Q4K: the half-column sums carry the 2^-24 of the Q4_K kernel's nibble units.  Otherwise (Q8_0): they are
+// multiplied by 128, the offset that turns the signed quants into unsigned bytes.  x is stored as it is.
+// HI: kept for the callers' sake (the bit of a float4's position that tells a high-nibble one); unused since the
+// sixteen-fold reading of high nibbles is undone in the scales instead of in the staged x.
 template <bool Q4K = true, int HI = 8>
 __device__ __forceinline__ void q4k_stage_store_one(const float4& v, int f, float4* xs, float* ss) {
     const int cc = f >> 4, i16 = f & 15;
     const int step = cc >> 6, ln = cc & 63;
-    const float mul = (Q4K && (i16 & HI)) ? 0.0625f : 1.0f;  // activations that meet high nibbles are stored divided by 16
-    xs[(step * 16 + i16) * kXPitch + ln] = make_float4(v.x * mul, v.y * mul, v.z * mul, v.w * mul);
+    xs[(step * 16 + i16) * kXPitch + ln] = v;
     float sum = (v.x + v.y) + (v.z + v.w);
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0xB1, 0xF, 0xF, true));   // lane ^ 1
     sum += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(sum), 0x4E, 0xF, 0xF, true));   // lane ^ 2
@@ -297,7 +297,8 @@ __device__ __forceinline__ void q4x_step(const Q4xLoads (&L)[R], const float4* _
                     q4k_dot_dword(q[i], xl[i], xh[i], alo, ahi);
                 }
             }
-            v[r] = fmaf(d, fmaf(kZero, sxb, alo + ahi), fmaf(m, sxb, v[r]));
+            const float both = kTable ? alo + ahi : fmaf(ahi, 0.0625f, alo);  // (high nibbles read sixteen-fold)
+            v[r] = fmaf(d, fmaf(kZero, sxb, both), fmaf(m, sxb, v[r]));
         }
     }
 #pragma unroll
@@ -349,7 +350,7 @@ __device__ __forceinline__ void q4k_step(const LT (&L)[R], const float4* __restr
         q4k_pair_scales(L[r].h, pair, sc0, sc1, m0, m1);
         const uint32_t dword0 = L[r].h.x;  // by value: a bit cast of a vector element reads the whole vector's start
         const half2_t dd = __builtin_bit_cast(half2_t, dword0);
-        const float t1 = fmaf(sc1, ahi[r], sc0 * alo[r]);
+        const float t1 = fmaf(sc1 * 0.0625f, ahi[r], sc0 * alo[r]);  // (the high nibbles were read sixteen-fold)
         const float t2 = fmaf(m1, sx.y, m0 * sx.x);
         const float v = fmaf((float)dd.x, t1, -((float)dd.y * t2));
         acc[r] += L[r].ok ? v : 0.f;
@@ -1889,7 +1890,25 @@ extern "C" int skn_test_fused_matvec(skn_ctx* ctx, int ggml_type, int epi, const
     rope.head_dim = kv->head_dim;
     rope.page_tokens = kv->page_tokens;
     rope.log2_base = log2((double)rope_base);
+    // option test.rope_table: the pair frequencies come from a device table of doubles, formed on the host as the
+    // decoder forms its own (the branch every decoder launch takes); otherwise the kernel forms them with exp2
+    double* table = nullptr;
+    if (ctx->opt_test_rope_table) {
+        std::vector<double> f(kv->head_dim / 2);
+        for (int i = 0; i < kv->head_dim / 2; i++) f[i] = pow((double)rope_base, -2.0 * i / kv->head_dim);
+        SKN_HIP(ctx, hipMalloc((void**)&table, f.size() * sizeof(double)));
+        if (hipMemcpy(table, f.data(), f.size() * sizeof(double), hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipFree(table);
+            return skn_fail(ctx, SKN_ERR_HIP, "skn_test_fused_matvec: uploading the rotary frequencies failed");
+        }
+        rope.inv_freq = table;
+    }
     rc = skn_matvec_q4k_fused(ctx, seg, n_out, k, x_dev, norm_w_dev, eps, y_dev, SKN_EPI_ROPE, &rope, ggml_type);
+    if (table) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(table);
+    }
     if (rc != SKN_OK) return rc;
     return skn_kv_advance_len(ctx, kv, 0, 1);
 }
@@ -1901,6 +1920,9 @@ extern "C" int skn_test_matvec_q4k_stamps(skn_ctx* ctx, const void* w_dev, int n
     SKN_REQUIRE(ctx, w_dev && x_dev && y_dev && stamps_dev, SKN_ERR_ARG, "skn_test_matvec_q4k_stamps: null pointer");
     SKN_REQUIRE(ctx, n > 0 && k % 256 == 0 && k > 8192 && k <= 12288, SKN_ERR_SHAPE,
                 "skn_test_matvec_q4k_stamps: k (%d) must be a multiple of 256 in (8192, 12288]", k);
+    // (every wavefront of the last workgroup writes its eight words: the stamp buffer is 8 words per row only when
+    // the rows fill whole workgroups of eight)
+    SKN_REQUIRE(ctx, n % 8 == 0, SKN_ERR_SHAPE, "skn_test_matvec_q4k_stamps: n (%d) must be a multiple of 8", n);
     SKN_REQUIRE(ctx, (((uintptr_t)w_dev | (uintptr_t)x_dev) & 15) == 0 && ((uintptr_t)stamps_dev & 7) == 0, SKN_ERR_ARG,
                 "skn_test_matvec_q4k_stamps: misaligned pointer");
     auto kern = matvec_q4k_kernel<3, 1, kFmtQ4K, true>;

@@ -195,5 +195,7 @@ def test_measuring_build_of_the_q4k_matvec(hip):
     assert np.all((t[:, 7] >> np.uint64(32)) < 8)  # XCC_ID
     with pytest.raises(runtime.SknError, match="multiple of 256 in"):
         hip.test_matvec_q4k_stamps(w, n, 4096, xd, y, stamps)
+    with pytest.raises(runtime.SknError, match="multiple of 8"):  # (stamps are written per wavefront of whole workgroups)
+        hip.test_matvec_q4k_stamps(w, n - 3, k, xd, y, stamps)
     for b in (w, xd, y, stamps):
         b.free()

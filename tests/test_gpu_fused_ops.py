@@ -120,3 +120,39 @@ def test_q4k_fused_forms_at_the_7b_shapes(hip):
     assert oracle_np.rel_err(ko.download(np.uint16, hdim).view(np.float16).astype(np.float32).reshape(heads, dim), kk) <= TOL
     assert oracle_np.rel_err(vo.download(np.uint16, hdim).view(np.float16).astype(np.float32).reshape(heads, dim), vv) <= TOL
     kv.free()
+
+
+@pytest.mark.parametrize("pos", [21, 256, 8189])
+@pytest.mark.parametrize("table", [0, 1])
+@pytest.mark.parametrize("kv_heads", [4, 2])
+def test_rotary_epilogue_with_and_without_the_frequency_table(hip, pos, table, kv_heads):
+    """The rotary epilogue takes a pair's frequency either from a device table of doubles (what every decoder launch
+    passes: base^(-2i/d) formed on the host) or from exp2 inside the kernel.  Both branches, at a position on the
+    second page, on a page boundary and near 8192, with as many K / V heads as query heads and with fewer (the k
+    and v segments then have fewer rows than q, which moves the table index), against the oracle's rotation."""
+    heads, dim, k, page = 4, 128, 1024, 256
+    hq, hkv = heads * dim, kv_heads * dim
+    wq = synth.weight(synth.Q4_K, hq, k, seed=140)
+    wk, wv = synth.weight(synth.Q4_K, hkv, k, seed=141), synth.weight(synth.Q4_K, hkv, k, seed=142)
+    x = synth.activation_f32(k, seed=150) * 3.0
+    g = (1.0 + 0.1 * np.random.default_rng(151).standard_normal(k)).astype(np.float32)
+    kv = hip.kv_cache(1, kv_heads, dim, page, 8192)
+    fill_k = hip.to_device(synth.kv_f16((pos, kv_heads, dim), seed=152))
+    kv.append_run(0, fill_k, fill_k, pos)
+    y = hip.alloc(4 * hq)
+    hip.set_option("test.rope_table", table)
+    try:
+        hip.test_fused_matvec(synth.Q4_K, ROPE, [(hip.to_device(wq), hq), (hip.to_device(wk), hkv), (hip.to_device(wv), hkv)], k,
+                              hip.to_device(x), hip.to_device(g), 1e-5, y, kv=kv, pos_dev=hip.alloc(16))
+    finally:
+        hip.set_option("test.rope_table", 0)
+    xn = _norm(x, g, 1e-5)
+    q = oracle_c.rope(oracle_c.matvec_q(synth.Q4_K, wq, hq, k, xn).reshape(heads, dim), pos, 10000.0)
+    kk = oracle_c.rope(oracle_c.matvec_q(synth.Q4_K, wk, hkv, k, xn).reshape(kv_heads, dim), pos, 10000.0)
+    vv = oracle_c.matvec_q(synth.Q4_K, wv, hkv, k, xn).reshape(kv_heads, dim)
+    assert oracle_np.rel_err(y.download(np.float32, hq).reshape(heads, dim), q) <= TOL
+    ko, vo = hip.alloc(2 * hkv), hip.alloc(2 * hkv)
+    kv.gather(0, pos, pos + 1, ko, vo)
+    assert oracle_np.rel_err(ko.download(np.uint16, hkv).view(np.float16).astype(np.float32).reshape(kv_heads, dim), kk) <= TOL
+    assert oracle_np.rel_err(vo.download(np.uint16, hkv).view(np.float16).astype(np.float32).reshape(kv_heads, dim), vv) <= TOL
+    kv.free()
