@@ -231,6 +231,148 @@ __global__ __launch_bounds__(kAttnThreads) void attn_decode_kernel(
     if (tid == 0) __hip_atomic_store(&counters[pair], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
 }
 
+
+// The same streams on sixteen wavefronts, for the decoder's step: a workgroup's token range (up to 256 tokens at
+// head_dim 128) is requested in one go, the streams of a wavefront merge through lane exchanges and the sixteen
+// wavefronts through LDS -- and that is all: with more than one split the workgroup leaves its unnormalised output and
+// its (max, sum) in memory with ordinary stores and ends.  Whoever reads them next merges them (the output
+// projection's staging, csrc/matvec.hip), so the launch has no device-wide counter, no waiting for stores and no
+// second round of loads behind one.
+constexpr int kWideThreads = 1024;
+
+template <int D, bool POW2>
+__global__ __launch_bounds__(kWideThreads) void attn_decode_wide_kernel(
+    const uint16_t* __restrict__ k_pool, const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ table,
+    const int32_t* __restrict__ nctx, const float* __restrict__ q, float* __restrict__ opart, float* __restrict__ ml,
+    float* __restrict__ out, int n_head, int kv_heads, int page_tokens, int page_shift, int pages_per_seq, int n_splits,
+    float scale, int seq_fixed) {
+    constexpr int LPT = D / 8, G = 64 / LPT, W = kWideThreads / 64, NS = W * G, U = kUnroll;
+    __shared__ float so[W][D];
+    __shared__ float sm[W], sl[W];
+    const int split = blockIdx.x, h = blockIdx.y, s = blockIdx.z;
+    const int kvh = kv_heads == n_head ? h : h / (n_head / kv_heads);
+    const int kv_seq = seq_fixed >= 0 ? seq_fixed : s;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane % LPT, g = lane / LPT;
+    const int stream = wave * G + g;
+    const int n = nctx[s];
+    const int per = ((n + n_splits - 1) / n_splits + NS - 1) / NS * NS;
+    const int t_begin = split * per;
+    const int t_end = min(n, t_begin + per);
+
+    float qf[8];
+    {
+        const float4* qp = reinterpret_cast<const float4*>(q + ((size_t)s * n_head + h) * D + c * 8);
+        const float4 a = qp[0], b = qp[1];
+        qf[0] = a.x * scale, qf[1] = a.y * scale, qf[2] = a.z * scale, qf[3] = a.w * scale;
+        qf[4] = b.x * scale, qf[5] = b.y * scale, qf[6] = b.z * scale, qf[7] = b.w * scale;
+    }
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) o[j] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const int32_t* trow = table + (size_t)kv_seq * pages_per_seq;
+    const int my_page = trow[min(lane, pages_per_seq - 1)];
+
+    for (int base = t_begin; base < t_end; base += NS * U) {
+        u32x4 kk[U], vv[U];
+        bool ok[U];
+        int page[U], slot[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int t = base + u * NS + stream;
+            ok[u] = t < t_end;
+            const int tc = min(t, t_end - 1);
+            const int pi = POW2 ? tc >> page_shift : tc / page_tokens;
+            slot[u] = tc - pi * page_tokens;
+            page[u] = __shfl(my_page, pi & 63, 64);
+            if (pi >= 64) page[u] = trow[pi];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t off = (((size_t)page[u] * kv_heads + kvh) * page_tokens + slot[u]) * D + c * 8;
+            kk[u] = *reinterpret_cast<const u32x4*>(k_pool + off);
+            vv[u] = *reinterpret_cast<const u32x4*>(v_pool + off);
+        }
+        float sc[U];
+        float m_new = m_run;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float d = group_sum<LPT>(dot8(kk[u], qf));
+            sc[u] = ok[u] ? d : -INFINITY;
+            m_new = fmaxf(m_new, sc[u]);
+        }
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __expf(m_run - m_safe);
+        float p[U], psum = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            p[u] = __expf(sc[u] - m_safe);
+            psum += p[u];
+        }
+        l_run = fmaf(l_run, alpha, psum);
+        m_run = m_new;
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] *= alpha;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t w = vv[u][j];
+                const half2_t hv = __builtin_bit_cast(half2_t, w);
+                o[2 * j] = fmaf(p[u], (float)hv.x, o[2 * j]);
+                o[2 * j + 1] = fmaf(p[u], (float)hv.y, o[2 * j + 1]);
+            }
+        }
+    }
+    // the G streams of the wavefront: lanes with the same c hold the same dimensions
+    float mw = m_run;
+#pragma unroll
+    for (int off = LPT; off < 64; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
+    const float mw_safe = mw == -INFINITY ? 0.f : mw;
+    const float wg = __expf(m_run - mw_safe);  // (an empty stream: exp(-inf) = 0)
+    float lw = l_run * wg;
+#pragma unroll
+    for (int j = 0; j < 8; j++) o[j] *= wg;
+#pragma unroll
+    for (int off = LPT; off < 64; off <<= 1) {
+        lw += __shfl_xor(lw, off, 64);
+#pragma unroll
+        for (int j = 0; j < 8; j++) o[j] += __shfl_xor(o[j], off, 64);
+    }
+    if (g == 0) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) so[wave][c * 8 + j] = o[j];
+        if (c == 0) {
+            sm[wave] = mw;
+            sl[wave] = lw;
+        }
+    }
+    __syncthreads();
+    if (tid < D) {
+        float M = -INFINITY, acc = 0.f, L = 0.f;
+#pragma unroll
+        for (int i = 0; i < W; i++) M = fmaxf(M, sm[i]);
+        const float m_safe = M == -INFINITY ? 0.f : M;
+#pragma unroll
+        for (int i = 0; i < W; i++) {
+            const float wgt = __expf(sm[i] - m_safe);
+            acc = fmaf(wgt, so[i][tid], acc);
+            L = fmaf(wgt, sl[i], L);
+        }
+        const int pair = s * n_head + h, n_pairs = gridDim.z * n_head;
+        if (n_splits == 1) {
+            out[(size_t)pair * D + tid] = L > 0.f ? acc / L : 0.f;
+        } else {
+            opart[((size_t)split * n_pairs + pair) * D + tid] = acc;
+            if (tid == 0) {
+                ml[2 * ((size_t)split * n_pairs + pair)] = M;
+                ml[2 * ((size_t)split * n_pairs + pair) + 1] = L;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 // Shared with the decoder.  n_queries query rows; row z attends to nctx_dev[z] tokens of sequence z
@@ -268,6 +410,38 @@ int skn_attn_launch_ex(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32
     else if (D == 128) SKN_ATTN_LAUNCH(128);
     else SKN_ATTN_LAUNCH(256);
 #undef SKN_ATTN_LAUNCH
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+int skn_attn_launch_unmerged(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
+                             int seq_fixed, int n_splits, float* opart, float* ml, float scale, float* out_dev, int n_q_head) {
+    const int D = kv->head_dim;
+    if (n_q_head <= 0) n_q_head = kv->n_head;
+    SKN_REQUIRE(ctx, n_q_head % kv->n_head == 0, SKN_ERR_SHAPE,
+                "attention: %d query heads are not a multiple of the %d cached heads", n_q_head, kv->n_head);
+    SKN_REQUIRE(ctx, D == 64 || D == 128 || D == 256, SKN_ERR_SHAPE, "attention: head_dim %d is not supported (64, 128 or 256)", D);
+    SKN_REQUIRE(ctx, n_splits >= 1 && (n_splits == 1 ? out_dev != nullptr : (opart != nullptr && ml != nullptr)), SKN_ERR_ARG,
+                "attention: %d splits without their buffers", n_splits);
+    int page_shift = -1;
+    if ((kv->page_tokens & (kv->page_tokens - 1)) == 0)
+        for (page_shift = 0; (1 << page_shift) < kv->page_tokens; page_shift++) {}
+    dim3 grid(n_splits, n_q_head, n_queries), block(kWideThreads);
+#define SKN_ATTN_WIDE(DD)                                                                                              \
+    do {                                                                                                               \
+        if (page_shift >= 0)                                                                                           \
+            skn_launch(ctx, attn_decode_wide_kernel<DD, true>, grid, block, 0, kv->k_pool, kv->v_pool, kv->page_table_dev, \
+                       nctx_dev, q_dev, opart, ml, out_dev, n_q_head, kv->n_head, kv->page_tokens, page_shift,         \
+                       kv->pages_per_seq, n_splits, scale, seq_fixed);                                                 \
+        else                                                                                                           \
+            skn_launch(ctx, attn_decode_wide_kernel<DD, false>, grid, block, 0, kv->k_pool, kv->v_pool, kv->page_table_dev, \
+                       nctx_dev, q_dev, opart, ml, out_dev, n_q_head, kv->n_head, kv->page_tokens, page_shift,         \
+                       kv->pages_per_seq, n_splits, scale, seq_fixed);                                                 \
+    } while (0)
+    if (D == 64) SKN_ATTN_WIDE(64);
+    else if (D == 128) SKN_ATTN_WIDE(128);
+    else SKN_ATTN_WIDE(256);
+#undef SKN_ATTN_WIDE
     SKN_LAUNCH_CHECK(ctx);
     return SKN_OK;
 }

@@ -28,7 +28,7 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1;
     int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
     bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
     long long stat_launches = 0, stat_captures = 0;  // kernel launches issued (or recorded) / decode-step graphs captured
@@ -61,6 +61,7 @@ struct skn_q4k_segments {
 // one rotary pair: q pairs are rotated and stored to y (fp32), k pairs are rotated and stored as fp16 into the
 // cache page of the token's position, v pairs are stored as fp16 beside them.
 enum { SKN_EPI_STORE = 0, SKN_EPI_ADD = 1, SKN_EPI_SWIGLU = 2, SKN_EPI_ROPE = 3 };
+struct skn_kv;
 struct skn_rope_epilogue {
     const int32_t* pos_dev = nullptr;     // position of the token (device scalar)
     const int32_t* page_table = nullptr;  // page table row of the token's sequence
@@ -69,7 +70,17 @@ struct skn_rope_epilogue {
     int n_head = 0, head_dim = 0, page_tokens = 0;
     double log2_base = 0.0;  // log2 of the rotary base, in double: the angle pos * base^(-2i/d) is formed in double
     const double* inv_freq = nullptr;  // optional device table base^(-2i/d), i < head_dim / 2 (saves the exp2 per wavefront)
+    // SKN_EPI_ADD without a norm (the output projection of an attention block): x is not a finished vector but the
+    // unmerged split partials of the decode attention -- x[split][pair][head_dim] unnormalised outputs, merge_ml
+    // [split][pair] (max, sum) -- and the staging merges them (skn_attn_launch_unmerged wrote them).  0 splits: plain x.
+    const float* merge_ml = nullptr;
+    int merge_splits = 0, merge_pairs = 0, merge_head_f4 = 0;  // pairs = query rows x heads, head_f4 = head_dim / 4
 };
+// Decode attention whose split partials are left unmerged for the consumer above (n_splits >= 2), or merged into out
+// (n_splits == 1).  One workgroup of sixteen wavefronts per (split, head, query row); no device counters, no atomics.
+// opart: n_splits * n_queries * n_q_head * head_dim floats, ml: two floats per (split, query row, head).
+int skn_attn_launch_unmerged(skn_ctx* ctx, skn_kv* kv, const float* q_dev, const int32_t* nctx_dev, int n_queries,
+                             int seq_fixed, int n_splits, float* opart, float* ml, float scale, float* out_dev, int n_q_head);
 int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, int k, const float* x, const float* norm_w,
                          float eps, float* y, int epi, const skn_rope_epilogue* rope = nullptr, int ggml_type = SKN_TYPE_Q4_K);
 // the formats the fused kernels take (every matrix of a launch in the same one; k a multiple of 256)

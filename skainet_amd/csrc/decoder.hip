@@ -350,11 +350,30 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
                        kv->page_tokens, log2((double)c.rope_base));
             SKN_LAUNCH_CHECK(ctx);
         }
-        SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
-        if (f_o) {
+        if (f_o && ctx->opt_llama_attn_wide && n_splits * 128 > 32768 / D) {
+            // The attention leaves the partials of its splits unmerged and the output projection's staging merges them:
+            // no device-wide counter, no store-then-reload chain inside the attention launch.  A workgroup of sixteen
+            // wavefronts takes 32768 / head_dim tokens per round of requests, so the splits are counted in those units.
+            const int per_round = 32768 / D;
+            int wide = 2;  // 2, 4 or 8 (what the merge in the projection's staging is built for)
+            while (wide < 8 && wide * per_round < n_splits * 128) wide *= 2;
+            if (ctx->opt_llama_attn_wide > 1) wide = std::min(wide, ctx->opt_llama_attn_wide);  // (tuning: 2, 4 or 8 caps the count)
+            float* opart = m->attn_partial;
+            float* ml = m->attn_partial + (size_t)wide * NH * D;
+            SKN_TRY(skn_attn_launch_unmerged(ctx, kv, m->q, m->state + 2, 1, 0, wide, opart, ml, scale, m->att, NH));
+            skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
+            skn_rope_epilogue mg;
+            mg.merge_ml = ml;
+            mg.merge_splits = wide;
+            mg.merge_pairs = NH;
+            mg.merge_head_f4 = D / 4;
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, wide > 1 ? opart : m->att, nullptr, 0.f, m->x, SKN_EPI_ADD, wide > 1 ? &mg : nullptr, L.type_o));
+        } else if (f_o) {
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD, nullptr, L.type_o));
         } else {
+            SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
             SKN_TRY(skn_matvec_q(ctx, L.type_o, L.wo, H, H, m->att, m->proj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
             SKN_LAUNCH_CHECK(ctx);
@@ -380,6 +399,8 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             SKN_LAUNCH_CHECK(ctx);
         }
     }
+    // (the final norm folded into the head's matvec was measured: the fused kernel's two rows per wavefront cost the
+    // 32000-row head more than the norm's launch saves, 30 us against 22 + 4)
     skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, m->w.out_norm, m->xn, H, c.rms_eps);
     SKN_LAUNCH_CHECK(ctx);
     SKN_TRY(skn_matvec_q(ctx, m->w.type_head, m->w.out_head, c.vocab, H, m->xn, m->logits));

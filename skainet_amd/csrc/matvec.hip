@@ -1351,6 +1351,33 @@ __device__ __forceinline__ void q4k_epilogue(const skn_rope_epilogue& rope, cons
     }
 }
 
+// One float4 of the attention output out of the unmerged partials of S splits: sum_s w_s part_s / sum_s w_s l_s with
+// w_s = exp(max_s - max over the splits); (max, sum) of split s and head h at ml[s * pairs + h].
+template <int S>
+__device__ __forceinline__ float4 q4k_merge_splits(const float4* __restrict__ part, const float2* __restrict__ ml, int n4, int f,
+                                                   int head, int pairs) {
+    float2 e[S];
+    float4 v[S];
+#pragma unroll
+    for (int sp = 0; sp < S; sp++) e[sp] = ml[sp * pairs + head];
+#pragma unroll
+    for (int sp = 0; sp < S; sp++) v[sp] = part[(size_t)sp * n4 + f];
+    float mx = e[0].x;
+#pragma unroll
+    for (int sp = 1; sp < S; sp++) mx = fmaxf(mx, e[sp].x);
+    const float m_safe = mx == -INFINITY ? 0.f : mx;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    float den = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < S; sp++) {
+        const float wgt = __expf(e[sp].x - m_safe);
+        a.x = fmaf(wgt, v[sp].x, a.x), a.y = fmaf(wgt, v[sp].y, a.y), a.z = fmaf(wgt, v[sp].z, a.z), a.w = fmaf(wgt, v[sp].w, a.w);
+        den = fmaf(wgt, e[sp].y, den);
+    }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    return make_float4(a.x * inv, a.y * inv, a.z * inv, a.w * inv);
+}
+
 // ---- fused forms used by the decoder ---------------------------------------------------------------------
 // Up to three weight matrices with the same k stacked along the output axis (q, k, v projections in one launch;
 // gate and up paired row by row), optional RMSNorm of x folded into the staging (every workgroup needs all of
@@ -1393,7 +1420,28 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
             rope_freq = rope.inv_freq[q4k_rope_elem(seg, rope, min((int)(blockIdx.x * 8 + (threadIdx.x >> 6)), (n_out + 1) / 2 - 1)) >> 1];
     }
     Q4kStage<J> st, nw;
-    q4k_stage_load<J>(x, n4, tid, 512, st);
+    bool merged = false;
+    if constexpr (EPI == SKN_EPI_ADD && !NORM) {
+        // x as the unmerged split partials of the decode attention: float4 f of x belongs to head f / head_f4; its value
+        // is sum_s w_s * part_s / sum_s w_s * l_s with w_s = exp(max_s - max over the splits), the merge the attention
+        // kernel otherwise does behind a device-wide counter
+        if (rope.merge_splits > 1) {
+            merged = true;
+            const float4* part = reinterpret_cast<const float4*>(x);
+            const float2* ml = reinterpret_cast<const float2*>(rope.merge_ml);
+#pragma unroll
+            for (int j = 0; j < J; j++) {
+                const int f = min(tid + j * 512, n4 - 1), head = f / rope.merge_head_f4;
+                // (the split count as a constant: every load of a float4's merge is requested before any is used)
+                switch (rope.merge_splits) {
+                    case 2: st.v[j] = q4k_merge_splits<2>(part, ml, n4, f, head, rope.merge_pairs); break;
+                    case 4: st.v[j] = q4k_merge_splits<4>(part, ml, n4, f, head, rope.merge_pairs); break;
+                    default: st.v[j] = q4k_merge_splits<8>(part, ml, n4, f, head, rope.merge_pairs); break;
+                }
+            }
+        }
+    }
+    if (!merged) q4k_stage_load<J>(x, n4, tid, 512, st);
     if (NORM) q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
 
     // the two rows of this wavefront: consecutive rows of the stacked matrices, or row i of gate and of up
@@ -1821,6 +1869,17 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
     }
     SKN_REQUIRE(ctx, k > 0 && k % 256 == 0 && k <= 16384, SKN_ERR_SHAPE, "fused Q4_K matvec: unsupported k %d", k);
     skn_rope_epilogue rope;
+    if (epi == SKN_EPI_ADD && rope_in && rope_in->merge_splits > 1) {
+        SKN_REQUIRE(ctx, rope_in->merge_splits == 2 || rope_in->merge_splits == 4 || rope_in->merge_splits == 8, SKN_ERR_ARG,
+                    "fused matvec: %d split partials (2, 4 or 8 are merged)", rope_in->merge_splits);
+        SKN_REQUIRE(ctx, !norm_w && rope_in->merge_ml && rope_in->merge_head_f4 > 0 && rope_in->merge_pairs * rope_in->merge_head_f4 * 4 == k &&
+                             ((uintptr_t)x & 15) == 0,
+                    SKN_ERR_ARG, "fused matvec: the split partials do not cover k = %d", k);
+        rope.merge_ml = rope_in->merge_ml;
+        rope.merge_splits = rope_in->merge_splits;
+        rope.merge_pairs = rope_in->merge_pairs;
+        rope.merge_head_f4 = rope_in->merge_head_f4;
+    }
     if (epi == SKN_EPI_ROPE) {
         SKN_REQUIRE(ctx, rope_in && rope_in->pos_dev && rope_in->page_table && rope_in->k_pool && rope_in->v_pool,
                     SKN_ERR_ARG, "fused Q4_K matvec: the rotary epilogue needs its cache arguments");

@@ -177,3 +177,48 @@ def test_hidden_4096_at_the_benchmark_length_matches_the_oracle_golden(hip, gold
     print("logit errors:", {k: f"{v:.2e}" for k, v in errs.items()}, "greedy tokens equal:", same, "of 128")
     assert same >= 120  # (steps whose top two logits are closer than the tolerance may differ)
     model.free()
+
+
+@pytest.mark.parametrize("wide", [1, 2, 0])
+@pytest.mark.parametrize("case,prompt_len", [("q4_k_kv2", 250), ("q4_k", 500), ("mixed", 500)])
+def test_decode_across_the_split_boundaries_of_the_attention(hip, case, prompt_len, wide):
+    """Contexts of 251 to 280 and 501 to 530 tokens: the decode attention goes from one workgroup per head to two and
+    from two to four while the steps run (llama.attn_wide = 1: the splits' partials are merged by the output projection's
+    staging; 0: by the attention kernel's last workgroup).  Prompt through the prompt path, thirty steps fed random
+    tokens, every step's logits against the oracle.  Tolerance: the prompt bound times 1.6 -- a prompt of 500 tokens has
+    ten times the bf16 roundings of the 41-token prompts above to flip (measured here: up to 4.7e-3, the same to three
+    digits on both paths); every mutation of the sensitivity test stays five times above it."""
+    import dataclasses
+
+    tol = 1.6 * PROMPT_TOL
+
+    cfg = dataclasses.replace(CASES[case], max_tokens=640)
+    w = llama.conditioned_weights(cfg, SEED)
+    key = (case, "long", prompt_len)
+    if key not in _ORACLE:
+        ora = OracleLlama(cfg, w)
+        prompt = tokens(prompt_len, cfg.vocab, seed=6)
+        ora.prefill(prompt, bf16_gemm=True)
+        first = ora.logits.copy()
+        toks = tokens(30, cfg.vocab, seed=8)
+        out = []
+        for t in toks:
+            ora.step(t)
+            out.append(ora.logits.copy())
+        _ORACLE[key] = (prompt, first, toks, out)
+    prompt, first, toks, want = _ORACLE[key]
+    hip.set_option("llama.attn_wide", wide)
+    try:
+        model = llama.LlamaModel(hip, cfg, weights=w)
+        model.prefill(prompt)
+        worst = logit_err(model.logits(), first)
+        assert worst <= tol, (case, "prompt", worst)
+        for i, t in enumerate(toks):
+            model.decode(t, 1)
+            err = logit_err(model.logits(), want[i])
+            worst = max(worst, err)
+            assert err <= tol, (case, wide, i, err)
+        print(f"{case} prompt {prompt_len} wide={wide}: worst logit error {worst:.2e}")
+        model.free()
+    finally:
+        hip.set_option("llama.attn_wide", 1)
