@@ -236,6 +236,27 @@ def matvec_timeline(ctx, n, k, reps=20, queued=12):
     return out
 
 
+def matvec_split_figures(ctx, n, k, steps=600, warmup=50):
+    """The headline matvec with k split across workgroups (option q4k.split) beside the default kernel, and beside the
+    dense F16 matvec over the same weight bytes: kernel durations from per-launch events, cold weights."""
+    out = {"mode": "ksplit", "workload": f"Q4_K matvec N={n} K={k}"}
+    r = bench_matvec(ctx, Q4_K, n, k, steps, warmup)
+    out["default_whole_rows_per_wavefront"] = {"kernel_us": round(r["kernel_us"], 3), "wall_us": round(r["ms_per_step"] * 1e3, 3)}
+    for split, rows, name in ((1, 1, "ticket_merge_1_row"), (1, 2, "ticket_merge_2_rows"), (2, 1, "atomic_add_1_row"), (2, 2, "atomic_add_2_rows")):
+        ctx.set_option("q4k.split", split)
+        ctx.set_option("q4k.rows", rows)
+        try:
+            r = bench_matvec(ctx, Q4_K, n, k, steps, warmup)
+        finally:
+            ctx.set_option("q4k.split", 0)
+            ctx.set_option("q4k.rows", 0)
+        # (with atomic adds every step is a fill of y and the kernel: the per-launch figure averages both)
+        out[name] = {"mean_us_per_launch": round(r["kernel_us"], 3), "wall_us_per_step": round(r["ms_per_step"] * 1e3, 3)}
+    rd = bench_matvec(ctx, 1, n, (n * (k // 256) * 144) // (2 * n), steps, warmup, seed=8100)
+    out["f16_matvec_same_weight_bytes"] = {"kernel_us": round(rd["kernel_us"], 3)}
+    return out
+
+
 def gemm_expanded_rows(ctx):
     """The Q6_K shapes of the GEMM leg with their expanded weights kept between calls."""
     return {f"q6_k_expanded_{mm}x{nn}x{kk}": bench_gemm(ctx, Q6_K, mm, nn, kk, expanded=True)
@@ -364,8 +385,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
-    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline"], default="bench",
-                    help="decode / attention / gemm: only that leg (for kernel traces).  timeline: the headline kernel's in-kernel time stamps.  copy: run --steps plain device copies of the headline weight size instead (the known-size "
+    ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline", "ksplit"], default="bench",
+                    help="decode / attention / gemm: only that leg (for kernel traces).  timeline: the headline kernel's in-kernel time stamps.  ksplit: the headline matvec with k split across workgroups beside the default.  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode without the captured step graph (kernel tracers that cannot follow graph launches)")
@@ -381,6 +402,10 @@ def main():
     n, k = 4096, 11008
     if args.mode == "timeline":
         print(json.dumps(matvec_timeline(ctx, n, k)))
+        ctx.close()
+        return
+    if args.mode == "ksplit":
+        print(json.dumps(matvec_split_figures(ctx, n, k, min(args.steps, 600), min(args.warmup, 50))))
         ctx.close()
         return
     if args.mode == "copy":

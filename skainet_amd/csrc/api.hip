@@ -89,6 +89,7 @@ void skn_shutdown(skn_ctx* ctx) {
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     if (ctx->attn_counters) (void)hipFree(ctx->attn_counters);
     if (ctx->gemm_ws) (void)hipFree(ctx->gemm_ws);
+    if (ctx->split_scratch) (void)hipFree(ctx->split_scratch);
     if (ctx->prefill_ws) (void)hipFree(ctx->prefill_ws);
     for (hipEvent_t e : ctx->prof_events) (void)hipEventDestroy(e);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
@@ -272,6 +273,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     SKN_REQUIRE(ctx, key != nullptr, SKN_ERR_ARG, "skn_set_option: key is null");
     if (!strcmp(key, "q4k.waves")) ctx->opt_q4k_waves = value;
     else if (!strcmp(key, "q4k.rows")) ctx->opt_q4k_rows = value;
+    else if (!strcmp(key, "q4k.split")) ctx->opt_q4k_split = value;
     else if (!strcmp(key, "attn.splits")) ctx->opt_attn_splits = value;
     else if (!strcmp(key, "llama.graph")) {
         SKN_REQUIRE(ctx, !(value && ctx->profiler_attached), SKN_ERR_STATE,

@@ -28,6 +28,7 @@ struct skn_ctx {
     size_t prof_used = 0;
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
+    int opt_q4k_split = 0;  // Q4_K matvec with k split across workgroups (measured alternative): 1 ticket merge, 2 atomic adds
     int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1, opt_llama_norm_handoff = 1;
     int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
     bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
@@ -38,6 +39,10 @@ struct skn_ctx {
     size_t attn_scratch_bytes = 0;
     int* attn_counters = nullptr;  // one per (sequence, head): workgroups of a split attention count themselves in
     int attn_counters_cap = 0;
+    // partials and tickets of the split Q4_K matvec (option q4k.split), grown on demand
+    void* split_scratch = nullptr;
+    size_t split_scratch_bytes = 0;
+    int split_scratch_n = 0, split_scratch_slices = 0;
     // prompt attention workspace (K and V of a sequence in matrix-core operand order), grown on demand
     void* prefill_ws = nullptr;
     size_t prefill_ws_bytes = 0;

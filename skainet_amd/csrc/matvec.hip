@@ -500,6 +500,92 @@ __global__ __launch_bounds__(512) void matvec_q4k_kernel(const uint8_t* __restri
     }
 }
 
+// The same arithmetic with k split across workgroups: workgroup (g, s) takes rows R * 8 g .. and the s-th step of
+// sixteen superblocks, stages only that 4096-slice of x (17 KB of LDS instead of the whole vector, so four workgroups
+// and 32 wavefronts fit a compute unit) and leaves one partial per row.  MERGE 1: the partials go to a scratch array
+// and the workgroup that takes a row group's last ticket adds them in slice order (deterministic; the counters return
+// to zero).  MERGE 2: they are added into y with floating-point atomics (y zeroed by the caller; the order of the
+// additions, and with it the last bit, varies).  Measured slower than whole rows per wavefront at every shape tried --
+// a launch of 1.5 rounds of workgroups pays the latency to first data twice, and the ticket costs two more round
+// trips -- and therefore not the default (option q4k.split; profiles/matvec_q4k_4096x11008.md has the figures).
+template <int R, int MERGE>
+__global__ __launch_bounds__(512) void matvec_q4k_split_kernel(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                               float* __restrict__ y, int n_rows, int nb, int n_slices,
+                                                               float* part, int* tickets) {
+    __shared__ float4 xs[16 * kXPitch];
+    __shared__ float ss[128];
+    __shared__ int last_flag;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = blockIdx.x / n_slices, s = blockIdx.x - g * n_slices;
+    const int sub = lane >> 2, p = lane & 3;
+    const int n4 = nb * 64;
+    Q4kStage<2> st;
+    {
+        const float4* x4 = reinterpret_cast<const float4*>(x);
+#pragma unroll
+        for (int j = 0; j < 2; j++) st.v[j] = x4[min(s * 1024 + tid + j * 512, n4 - 1)];
+    }
+    const int row0 = (g * 8 + wave) * R;
+    const int blk = s * 16 + sub;
+    Q4kLoads L[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const u32x4* bp = reinterpret_cast<const u32x4*>(w + (size_t)min(row0 + r, n_rows - 1) * nb * 144) + min(blk, nb - 1) * 9;
+        L[r].qa = bp[1 + 2 * p];
+        L[r].qb = bp[2 + 2 * p];
+        L[r].h = bp[0];
+        L[r].ok = row0 + r < n_rows && blk < nb;
+    }
+    // local float4 f of the slice goes where float4 f of a whole vector's first step goes (a float4 past the end of x
+    // repeats the last one; its superblock is masked)
+    q4k_stage_store<2>(st, 1024, tid, 512, xs, ss);
+    __syncthreads();
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    q4k_step<R>(L, xs, ss, 0, lane, p, acc);
+    float tot[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) tot[r] = wave_sum(acc[r]) * 16777216.0f;
+    if (n_slices == 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (row0 + r < n_rows) y[row0 + r] = tot[r];
+        }
+        return;
+    }
+    if (MERGE == 2) {
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (row0 + r < n_rows) atomicAdd(&y[row0 + r], tot[r]);
+        }
+        return;
+    }
+    // partials and tickets as device-scope atomics, the stores waited for before the ticket is taken (the hand-off of
+    // the decode attention's split merge)
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (row0 + r < n_rows) __hip_atomic_store(&part[(size_t)s * n_rows + row0 + r], tot[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) last_flag = __hip_atomic_fetch_add(&tickets[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_slices - 1;
+    __syncthreads();
+    if (!last_flag) return;
+    if (tid < 8 * R) {
+        const int row = g * 8 * R + tid;
+        if (row < n_rows) {
+            float sum = 0.f;
+            for (int i = 0; i < n_slices; i++) sum += __hip_atomic_load(&part[(size_t)i * n_rows + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            y[row] = sum;
+        }
+    }
+    if (tid == 0) __hip_atomic_store(&tickets[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // ------------------------------------------------------------------------------------------ Q8_0
 //
 // 34-byte blocks (f16 d, 32 x int8), only 2-byte aligned.  Two consecutive blocks are 68 bytes = 17 dwords:
@@ -2116,6 +2202,39 @@ extern "C" int skn_matvec_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int 
         }
     }
     if (!skn_is_core_quant(ggml_type)) return skn_matvec_other(ctx, ggml_type, w, n, k, x_dev, y_dev);
+    if (ggml_type == SKN_TYPE_Q4_K && ctx->opt_q4k_split > 0 && nb <= 64) {
+        // k split across workgroups (a measured alternative, not the default): 1 = partials merged behind a ticket,
+        // 2 = floating-point atomic adds into a zeroed y
+        const int slices = (nb + 15) / 16, rows = ctx->opt_q4k_rows >= 2 ? 2 : 1;
+        const int groups = (n + 8 * rows - 1) / (8 * rows);
+        const size_t need = (size_t)slices * n * sizeof(float) + (size_t)groups * sizeof(int);
+        if (need > ctx->split_scratch_bytes) {
+            SKN_HIP(ctx, hipStreamSynchronize(ctx->stream));
+            if (ctx->split_scratch) SKN_HIP(ctx, hipFree(ctx->split_scratch));
+            ctx->split_scratch = nullptr, ctx->split_scratch_bytes = 0;
+            SKN_HIP(ctx, hipMalloc(&ctx->split_scratch, need));
+            ctx->split_scratch_bytes = need;
+            SKN_HIP(ctx, hipMemsetAsync(ctx->split_scratch, 0, need, ctx->stream));  // (tickets start at zero and return to it)
+        }
+        float* part = (float*)ctx->split_scratch;
+        int* tickets = (int*)((uint8_t*)ctx->split_scratch + (size_t)slices * n * sizeof(float));
+        // (the scratch is laid out for this n: another n re-zeroes the tickets' new place)
+        if (ctx->split_scratch_n != n || ctx->split_scratch_slices != slices) {
+            SKN_HIP(ctx, hipMemsetAsync(ctx->split_scratch, 0, ctx->split_scratch_bytes, ctx->stream));
+            ctx->split_scratch_n = n, ctx->split_scratch_slices = slices;
+        }
+        dim3 grid((unsigned)(groups * slices)), block(512);
+        if (ctx->opt_q4k_split >= 2) {
+            if (slices > 1) SKN_HIP(ctx, hipMemsetAsync(y_dev, 0, (size_t)n * sizeof(float), ctx->stream));
+            if (rows == 2) skn_launch(ctx, matvec_q4k_split_kernel<2, 2>, grid, block, 0, w, x_dev, y_dev, n, nb, slices, part, tickets);
+            else skn_launch(ctx, matvec_q4k_split_kernel<1, 2>, grid, block, 0, w, x_dev, y_dev, n, nb, slices, part, tickets);
+        } else {
+            if (rows == 2) skn_launch(ctx, matvec_q4k_split_kernel<2, 1>, grid, block, 0, w, x_dev, y_dev, n, nb, slices, part, tickets);
+            else skn_launch(ctx, matvec_q4k_split_kernel<1, 1>, grid, block, 0, w, x_dev, y_dev, n, nb, slices, part, tickets);
+        }
+        SKN_LAUNCH_CHECK(ctx);
+        return SKN_OK;
+    }
     if (ggml_type == SKN_TYPE_Q4_K) {
         int waves = ctx->opt_q4k_waves, rows = ctx->opt_q4k_rows;
         if (waves <= 0) waves = 8;

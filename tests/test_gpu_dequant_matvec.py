@@ -199,3 +199,35 @@ def test_measuring_build_of_the_q4k_matvec(hip):
         hip.test_matvec_q4k_stamps(w, n - 3, k, xd, y, stamps)
     for b in (w, xd, y, stamps):
         b.free()
+
+
+@pytest.mark.parametrize("n,k", [(4096, 11008), (70, 4096), (64, 8192), (33, 256)])
+@pytest.mark.parametrize("split,rows", [(1, 1), (1, 2), (2, 1), (2, 2)])
+def test_q4k_matvec_with_k_split_across_workgroups(hip, n, k, split, rows):
+    """Option q4k.split: a workgroup takes one step of sixteen superblocks of its rows; partials merged behind a ticket
+    (1: the sum runs in slice order, so two calls give the same bits) or by atomic adds into a zeroed y (2).  Same
+    answer as the oracle at the operation's bound, at the headline shape, with a ragged last row group, with two and
+    one slices; the ticket counters are back at zero after every call (a second call on another weight is right too)."""
+    raw = synth.weight(synth.Q4_K, n, k, seed=300 + n)
+    raw2 = synth.weight(synth.Q4_K, n, k, seed=301 + n)
+    x = synth.activation_f32(k, seed=302)
+    w, w2, xd, y = hip.to_device(raw), hip.to_device(raw2), hip.to_device(x), hip.alloc(4 * n)
+    hip.set_option("q4k.split", split)
+    hip.set_option("q4k.rows", rows)
+    try:
+        hip.matvec_q(synth.Q4_K, w, n, k, xd, y)
+        first = y.download(np.float32, n)
+        assert oracle_np.rel_err(first, oracle_c.matvec_q(synth.Q4_K, raw, n, k, x)) <= 1e-3
+        hip.matvec_q(synth.Q4_K, w2, n, k, xd, y)
+        assert oracle_np.rel_err(y.download(np.float32, n), oracle_c.matvec_q(synth.Q4_K, raw2, n, k, x)) <= 1e-3
+        hip.matvec_q(synth.Q4_K, w, n, k, xd, y)
+        again = y.download(np.float32, n)
+        if split == 1:
+            assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+        else:
+            assert oracle_np.rel_err(again, first) <= 1e-4  # (the order of the atomic additions moves the last bit)
+    finally:
+        hip.set_option("q4k.split", 0)
+        hip.set_option("q4k.rows", 0)
+    for b in (w, w2, xd, y):
+        b.free()
