@@ -388,6 +388,8 @@ def main():
     ap.add_argument("--mode", choices=["bench", "copy", "decode", "attention", "gemm", "formats", "timeline", "ksplit"], default="bench",
                     help="decode / attention / gemm: only that leg (for kernel traces).  timeline: the headline kernel's in-kernel time stamps.  ksplit: the headline matvec with k split across workgroups beside the default.  copy: run --steps plain device copies of the headline weight size instead (the known-size "
                          "workload that hardware traffic counters are calibrated against)")
+    ap.add_argument("--set", action="append", default=[], metavar="KEY=VALUE",
+                    help="a tuning option of the library (skn_set_option) for this run, e.g. --set attn.splits=2 or --set llama.attn_wide=0; repeatable")
     ap.add_argument("--no-graph", action="store_true",
                     help="decode without the captured step graph (kernel tracers that cannot follow graph launches)")
     args = ap.parse_args()
@@ -399,6 +401,9 @@ def main():
     info = ctx.device_info()
     if args.no_graph:
         ctx.set_option("llama.graph", 0)
+    for kv in args.set:
+        key, _, val = kv.partition("=")
+        ctx.set_option(key, int(val))
     n, k = 4096, 11008
     if args.mode == "timeline":
         print(json.dumps(matvec_timeline(ctx, n, k)))
@@ -457,6 +462,12 @@ def main():
             extra[name] = {key: (round(r[key], 3) if isinstance(r[key], float) else r[key])
                            for key in ("kernel_us", "kernel_gbs", "hot_kernel_us", "hot_kernel_gbs", "wall_gbs")}
             extra[name]["frac_hbm_peak"] = round(r["kernel_gbs"] / HBM_PEAK_GBS, 4)
+        # the smallest shape beside the dense F16 matvec over its weight bytes (4096 x 1152 x 2 = 9 437 184), as the
+        # headline stands beside its own: at 9.4 MB a launch is mostly its fixed cost, for any kernel
+        rs = bench_matvec(ctx, 1, 4096, 1152, es, ew, copies=64, seed=8200)
+        extra["q4_k_4096x4096"]["read_rate_same_bytes"] = {"kernel": "dense F16 matvec 4096 x 1152", "kernel_us": round(rs["kernel_us"], 3),
+                                                          "frac": round(rs["kernel_gbs"] / HBM_PEAK_GBS, 4)}
+        extra["q4_k_4096x4096"]["frac_of_read_rate"] = round(extra["q4_k_4096x4096"]["kernel_gbs"] / rs["kernel_gbs"], 4)
         other = bench_other_formats(ctx)["4096x4096"]
         extra["other_formats_4096x4096"] = other
         extra["dequant_4096x4096"] = {name: bench_dequant(ctx, qt, 4096, 4096)

@@ -286,7 +286,6 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     else if (!strcmp(key, "matvec.stage")) ctx->opt_matvec_stage = value;
     else if (!strcmp(key, "test.rope_table")) ctx->opt_test_rope_table = value;
     else if (!strcmp(key, "llama.attn_wide")) ctx->opt_llama_attn_wide = value;
-    else if (!strcmp(key, "llama.norm_handoff")) ctx->opt_llama_norm_handoff = value;
     else return skn_fail(ctx, SKN_ERR_ARG, "skn_set_option: unknown option '%s'", key);
     ctx->opt_generation++;  // whatever was captured with the old settings is stale
     return SKN_OK;

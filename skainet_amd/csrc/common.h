@@ -29,7 +29,7 @@ struct skn_ctx {
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
     int opt_q4k_split = 0;  // Q4_K matvec with k split across workgroups (measured alternative): 1 ticket merge, 2 atomic adds
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1, opt_llama_norm_handoff = 1;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1;
     int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
     bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
     long long stat_launches = 0, stat_captures = 0;  // kernel launches issued (or recorded) / decode-step graphs captured
@@ -80,15 +80,6 @@ struct skn_rope_epilogue {
     // [split][pair] (max, sum) -- and the staging merges them (skn_attn_launch_unmerged wrote them).  0 splits: plain x.
     const float* merge_ml = nullptr;
     int merge_splits = 0, merge_pairs = 0, merge_head_f4 = 0;  // pairs = query rows x heads, head_f4 = head_dim / 4
-    // The RMSNorm between two fused launches, split between them.  Producer (SKN_EPI_ADD): besides y += W x it stores
-    // next_xg = y * next_g (the consumer's norm weights) and one partial sum of y^2 per workgroup into next_sq.
-    // Consumer (a launch with norm_w): with pre_sq set, x is that next_xg and the sum of squares is the sum of the
-    // pre_sq_n partials, in index order -- it loads no norm weights and squares nothing.
-    const float* next_g = nullptr;
-    float* next_xg = nullptr;
-    float* next_sq = nullptr;
-    const float* pre_sq = nullptr;
-    int pre_sq_n = 0;
 };
 // Decode attention whose split partials are left unmerged for the consumer above (n_splits >= 2), or merged into out
 // (n_splits == 1).  One workgroup of sixteen wavefronts per (split, head, query row); no device counters, no atomics.

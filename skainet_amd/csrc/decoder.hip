@@ -18,7 +18,6 @@ struct skn_llama {
     // decode-step buffers
     float *x = nullptr, *xn = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *att = nullptr, *proj = nullptr;
     float *gate = nullptr, *up = nullptr, *mid = nullptr, *logits = nullptr, *attn_partial = nullptr;
-    float *xg = nullptr, *sq = nullptr;  // residual stream times the next norm's weights, partial sums of its squares (norm hand-off between fused launches)
     int *attn_counters = nullptr, *pcounters = nullptr;  // split counters of the attention launches (zero between launches)
     int32_t* state = nullptr;       // [0] token, [1] position, [2] context length, [3] step index
     int32_t* tokens_out = nullptr;  // device array of produced tokens
@@ -305,15 +304,6 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
     skn_launch(ctx, embed_rows_kernel, dim3(1), dim3(1024), 0, (const uint8_t*)m->w.tok_embd, m->w.type_embd, H,
                (const int32_t*)m->state, m->x);
     SKN_LAUNCH_CHECK(ctx);
-    // The RMSNorm between two fused launches is split between them: the launch that writes the residual stream also
-    // writes it times the next norm's weights and its workgroups' sums of squares; the launch that follows reads those.
-    const bool handoff = ctx->opt_llama_fused && ctx->opt_llama_norm_handoff && c.hidden % 256 == 0 && c.hidden <= 16384;
-    const int sq_n = (c.hidden / 2 + 7) / 8;  // workgroups of a producer launch: eight wavefronts of two rows
-    auto qkv_fused = [&](int l) {
-        const skn_llama_layer& L = m->layers[l];
-        return ctx->opt_llama_fused && skn_matvec_fusable(L.type_q) && skn_matvec_fusable(L.type_k) && skn_matvec_fusable(L.type_v);
-    };
-    bool pre_valid = false;  // m->xg / m->sq hold the input of the next norm
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];
@@ -338,7 +328,6 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             rope.page_tokens = kv->page_tokens;
             rope.log2_base = log2((double)c.rope_base);
             rope.inv_freq = m->inv_freq;
-            if (pre_valid) rope.pre_sq = m->sq, rope.pre_sq_n = sq_n;
             const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
             const uint8_t* mats[3] = {(const uint8_t*)L.wq, (const uint8_t*)L.wk, (const uint8_t*)L.wv};
             bool done[3] = {false, false, false};
@@ -348,7 +337,7 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
                 int n_out = 0;
                 for (int j = i; j < 3; j++)
                     if (types[j] == types[i]) part.w[j] = mats[j], part.rows[j] = rows[j], n_out += rows[j], done[j] = true;
-                SKN_TRY(skn_matvec_q4k_fused(ctx, part, n_out, H, pre_valid ? m->xg : m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope, types[i]));
+                SKN_TRY(skn_matvec_q4k_fused(ctx, part, n_out, H, m->x, L.attn_norm, c.rms_eps, m->q, SKN_EPI_ROPE, &rope, types[i]));
             }
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.attn_norm, m->xn, H, c.rms_eps);
@@ -378,26 +367,20 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
             mg.merge_splits = wide;
             mg.merge_pairs = NH;
             mg.merge_head_f4 = D / 4;
-            if (handoff && f_gu) mg.next_g = L.ffn_norm, mg.next_xg = m->xg, mg.next_sq = m->sq;
             SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, opart, nullptr, 0.f, m->x, SKN_EPI_ADD, &mg, L.type_o));
         } else if (f_o) {
             SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
             skn_q4k_segments wo = {{(const uint8_t*)L.wo, nullptr, nullptr}, {H, 0, 0}};
-            skn_rope_epilogue ex;
-            if (handoff && f_gu) ex.next_g = L.ffn_norm, ex.next_xg = m->xg, ex.next_sq = m->sq;
-            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD, &ex, L.type_o));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wo, H, H, m->att, nullptr, 0.f, m->x, SKN_EPI_ADD, nullptr, L.type_o));
         } else {
             SKN_TRY(skn_attn_launch_ex(ctx, kv, m->q, m->state + 2, 1, 0, n_splits, m->attn_partial, m->attn_counters, scale, m->att, NH));
             SKN_TRY(skn_matvec_q(ctx, L.type_o, L.wo, H, H, m->att, m->proj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
             SKN_LAUNCH_CHECK(ctx);
         }
-        pre_valid = handoff && f_o && f_gu;
         if (f_gu) {
             skn_q4k_segments gu = {{(const uint8_t*)L.w_gate, (const uint8_t*)L.w_up, nullptr}, {F, F, 0}};
-            skn_rope_epilogue ex;
-            if (pre_valid) ex.pre_sq = m->sq, ex.pre_sq_n = sq_n;
-            SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, pre_valid ? m->xg : m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU, &ex, L.type_gate));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, gu, F, H, m->x, L.ffn_norm, c.rms_eps, m->mid, SKN_EPI_SWIGLU, nullptr, L.type_gate));
         } else {
             skn_launch(ctx, rmsnorm_rows_kernel, dim3(1), dim3(256), 0, (const float*)m->x, L.ffn_norm, m->xn, H, c.rms_eps);
             SKN_LAUNCH_CHECK(ctx);
@@ -407,12 +390,9 @@ int decode_step(skn_ctx* ctx, skn_llama* m, int n_splits) {
                        m->mid, (int64_t)F);
             SKN_LAUNCH_CHECK(ctx);
         }
-        pre_valid = handoff && f_down && l + 1 < c.n_layer && fuse && qkv_fused(l + 1);
         if (f_down) {
             skn_q4k_segments wd = {{(const uint8_t*)L.w_down, nullptr, nullptr}, {H, 0, 0}};
-            skn_rope_epilogue ex;
-            if (pre_valid) ex.next_g = m->layers[l + 1].attn_norm, ex.next_xg = m->xg, ex.next_sq = m->sq;
-            SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD, &ex, L.type_down));
+            SKN_TRY(skn_matvec_q4k_fused(ctx, wd, H, F, m->mid, nullptr, 0.f, m->x, SKN_EPI_ADD, nullptr, L.type_down));
         } else {
             SKN_TRY(skn_matvec_q(ctx, L.type_down, L.w_down, H, F, m->mid, m->proj));
             skn_launch(ctx, add_rows_kernel, dim3(nblk(H)), dim3(256), 0, m->x, (const float*)m->proj, (int64_t)H);
@@ -559,8 +539,6 @@ int skn_llama_create(skn_ctx* ctx, const skn_llama_config* cfg, const skn_llama_
         (void)hipGetLastError();
         rc = skn_fail(ctx, SKN_ERR_HIP, "skn_llama_create: clearing the attention counters failed");
     }
-    A(&m->xg, (size_t)cfg->hidden);
-    A(&m->sq, (size_t)(cfg->hidden / 16 + 1));
     A(&m->state, (size_t)4);
     A(&m->inv_freq, (size_t)cfg->head_dim / 2);
     if (rc == SKN_OK) {

@@ -1528,16 +1528,7 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
         }
     }
     if (!merged) q4k_stage_load<J>(x, n4, tid, 512, st);
-    // (norm weights and squares only when the producer of x has not already multiplied and summed)
-    const bool prenormed = NORM && rope.pre_sq != nullptr;
-    float pre = 0.f;
-    if (NORM) {
-        if (prenormed) {
-            for (int i = tid; i < rope.pre_sq_n; i += 512) pre += rope.pre_sq[i];
-        } else {
-            q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
-        }
-    }
+    if (NORM) q4k_stage_load<J>(norm_w, n4, tid, 512, nw);
 
     // the two rows of this wavefront: consecutive rows of the stacked matrices, or row i of gate and of up
     const int unit = blockIdx.x * 8 + wave;
@@ -1641,19 +1632,17 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     // totals are multiplied by r = 1 / sqrt(mean(x^2) + eps) at the end, so the sum of squares needs no
     // barrier of its own (its eight partials are read after the staging barrier)
     if (NORM) {
-        float sq = pre;
-        if (!prenormed) {
+        float sq = 0.f;
 #pragma unroll
-            for (int j = 0; j < J; j++) {
-                if (tid + j * 512 < n4) {
-                    const float4 v = st.v[j];
-                    sq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
-                }
-                st.v[j].x *= nw.v[j].x;
-                st.v[j].y *= nw.v[j].y;
-                st.v[j].z *= nw.v[j].z;
-                st.v[j].w *= nw.v[j].w;
+        for (int j = 0; j < J; j++) {
+            if (tid + j * 512 < n4) {
+                const float4 v = st.v[j];
+                sq += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
             }
+            st.v[j].x *= nw.v[j].x;
+            st.v[j].y *= nw.v[j].y;
+            st.v[j].z *= nw.v[j].z;
+            st.v[j].w *= nw.v[j].w;
         }
         sq = wave_sum(sq);
         if (lane == 0) red[wave] = sq;
@@ -1700,33 +1689,6 @@ __global__ __launch_bounds__(512) void matvec_q4k_fused_kernel(skn_q4k_segments 
     const float back = (Q8 || Q8K || T1 || kPlainX) ? rinv : 16777216.0f * rinv;  // (the nibble formats work in units of 2^-24)
     const float t0 = wave_sum(acc[0]) * back;
     const float t1 = wave_sum(acc[1]) * back;
-    if constexpr (EPI == SKN_EPI_ADD) {
-        if (rope.next_g) {
-            // the residual stream's new rows, the same rows times the next norm's weights, and this workgroup's share
-            // of the sum of squares (its eight wavefronts' shares added in wavefront order)
-            if (lane == 0) {
-                float sq = 0.f;
-                const int r0 = unit * 2, r1 = unit * 2 + 1;
-                if (r0 < n_out) {
-                    const float v = y[r0] + t0;
-                    y[r0] = v;
-                    rope.next_xg[r0] = v * rope.next_g[r0];
-                    sq = v * v;
-                }
-                if (r1 < n_out) {
-                    const float v = y[r1] + t1;
-                    y[r1] = v;
-                    rope.next_xg[r1] = v * rope.next_g[r1];
-                    sq = fmaf(v, v, sq);
-                }
-                red[wave] = sq;
-            }
-            __syncthreads();
-            if (tid == 0)
-                rope.next_sq[blockIdx.x] = ((red[0] + red[1]) + (red[2] + red[3])) + ((red[4] + red[5]) + (red[6] + red[7]));
-            return;
-        }
-    }
     if (lane == 0) q4k_epilogue<EPI>(rope, rc, y, n_out, unit, t0, t1);
 }
 
@@ -2003,17 +1965,6 @@ int skn_matvec_q4k_fused(skn_ctx* ctx, const skn_q4k_segments& seg, int n_out, i
         rope.merge_splits = rope_in->merge_splits;
         rope.merge_pairs = rope_in->merge_pairs;
         rope.merge_head_f4 = rope_in->merge_head_f4;
-    }
-    if (rope_in && epi == SKN_EPI_ADD && rope_in->next_g) {
-        SKN_REQUIRE(ctx, rope_in->next_xg && rope_in->next_sq, SKN_ERR_ARG, "fused matvec: the norm hand-off lacks a buffer");
-        rope.next_g = rope_in->next_g;
-        rope.next_xg = rope_in->next_xg;
-        rope.next_sq = rope_in->next_sq;
-    }
-    if (rope_in && norm_w && rope_in->pre_sq) {
-        SKN_REQUIRE(ctx, rope_in->pre_sq_n > 0, SKN_ERR_ARG, "fused matvec: no partial sums of squares");
-        rope.pre_sq = rope_in->pre_sq;
-        rope.pre_sq_n = rope_in->pre_sq_n;
     }
     if (epi == SKN_EPI_ROPE) {
         SKN_REQUIRE(ctx, rope_in && rope_in->pos_dev && rope_in->page_table && rope_in->k_pool && rope_in->v_pool,
