@@ -125,7 +125,26 @@ def bench_attention(ctx, steps, warmup):
     nbytes = n_seq * n_head * n_ctx * dim * 2 * 2 + 2 * 4 * n_seq * n_head * dim
     kv.free()
     per_step_us = kernel_ms / steps * 1e3
+    # what the memory system gives a plain stream of the same size: the dense F16 matvec over 32768 x 8192 (536 870 912
+    # weight bytes, twice the last-level cache, so every launch reads memory)
+    rn, rk = 32768, 8192
+    wbig = ctx.alloc(2 * rn * rk)
+    ctx.memset(wbig, 0x3c, 2 * rn * rk)
+    xb, yb = ctx.to_device(synth.activation_f32(rk, seed=5)), ctx.alloc(4 * rn)
+    for _ in range(3):
+        ctx.matvec_q(1, wbig, rn, rk, xb, yb)
+    ctx.prof_start(20)
+    for _ in range(20):
+        ctx.matvec_q(1, wbig, rn, rk, xb, yb)
+    rms, rl = ctx.prof_stop()
+    for b in (wbig, xb, yb):
+        b.free()
+    read_us = rms / rl * 1e3
+    read_gbs = (2 * rn * rk + 4 * rk + 4 * rn) / (read_us * 1e-6) / 1e9
     return {
+        "read_rate_same_bytes_us": read_us,
+        "read_rate_same_bytes_frac": read_gbs / HBM_PEAK_GBS,
+        "frac_of_read_rate": nbytes / (per_step_us * 1e-6) / 1e9 / read_gbs,
         "bytes_per_step": nbytes,
         "kernel_us_per_step": per_step_us,
         "kernel_gbs": nbytes / (per_step_us * 1e-6) / 1e9,
