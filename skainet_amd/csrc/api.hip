@@ -283,6 +283,7 @@ int skn_set_option(skn_ctx* ctx, const char* key, int value) {
     else if (!strcmp(key, "llama.fused")) ctx->opt_llama_fused = value;
     else if (!strcmp(key, "llama.expand_weights")) ctx->opt_llama_expand = value;
     else if (!strcmp(key, "gemm.tile")) ctx->opt_gemm_tile = value;
+    else if (!strcmp(key, "gemm.q6k_fused")) ctx->opt_gemm_q6k_fused = value;
     else if (!strcmp(key, "matvec.stage")) ctx->opt_matvec_stage = value;
     else if (!strcmp(key, "test.rope_table")) ctx->opt_test_rope_table = value;
     else if (!strcmp(key, "llama.attn_wide")) ctx->opt_llama_attn_wide = value;

@@ -29,7 +29,7 @@ struct skn_ctx {
     std::vector<hipEvent_t> prof_events;
     // tuning options (skn_set_option); 0 = library default
     int opt_q4k_split = 0;  // Q4_K matvec with k split across workgroups (measured alternative): 1 ticket merge, 2 atomic adds
-    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1;
+    int opt_q4k_waves = 0, opt_q4k_rows = 0, opt_attn_splits = 0, opt_llama_graph = 1, opt_llama_fused = 1, opt_gemm_tile = 0, opt_matvec_stage = 1, opt_llama_expand = 0, opt_test_rope_table = 0, opt_llama_attn_wide = 1, opt_gemm_q6k_fused = 1;
     int opt_generation = 0;          // bumped by every skn_set_option / skn_set_stream: captured work is stamped with it
     bool profiler_attached = false;  // a rocprofiler tool library is loaded into this process: graphs are not replayed
     long long stat_launches = 0, stat_captures = 0;  // kernel launches issued (or recorded) / decode-step graphs captured

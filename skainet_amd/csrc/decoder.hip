@@ -458,7 +458,7 @@ int ensure_prompt_buffers(skn_ctx* ctx, skn_llama* m, int T) {
     SKN_TRY(dev_alloc(ctx, m, &m->pb16, T * (F > H ? F : H)));
     SKN_TRY(dev_alloc(ctx, m, &m->ptok, (size_t)T));
     SKN_TRY(dev_alloc(ctx, m, &m->pnctx, (size_t)T));
-    // splits = ceil(4 * CUs / pairs) bounds pairs * splits by pairs + 4 * CUs
+    // splits <= ceil(CUs / pairs) keeps pairs * splits below pairs + CUs; the rest is head room
     SKN_TRY(dev_alloc(ctx, m, &m->ppartial, ((size_t)T * c.n_head + 4 * (size_t)ctx->compute_units) * (c.head_dim + 2)));
     SKN_TRY(dev_alloc(ctx, m, &m->pcounters, (size_t)T * c.n_head));
     SKN_HIP(ctx, hipMemsetAsync(m->pcounters, 0, (size_t)T * c.n_head * sizeof(int), ctx->stream));
@@ -622,8 +622,9 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
                (const int32_t*)m->ptok, m->px);
     SKN_LAUNCH_CHECK(ctx);
     const float scale = 1.0f / sqrtf((float)D);
-    int n_splits = (4 * ctx->compute_units + T * NH - 1) / (T * NH);
-    if (n_splits > (pos0 + T + 63) / 64) n_splits = (pos0 + T + 63) / 64;
+    int n_splits = skn_attn_splits(ctx, T * NH, pos0 + T);
+    // (the option attn.splits may ask for more than the partials buffer of ensure_prompt_buffers holds)
+    n_splits = std::min(n_splits, 1 + 4 * ctx->compute_units / (T * NH));
     for (int l = 0; l < c.n_layer; l++) {
         const skn_llama_layer& L = m->layers[l];
         skn_kv* kv = m->kv[l];

@@ -823,6 +823,252 @@ int launch_hilo_gemm_mt(skn_ctx* ctx, int mt, const u32x4* afrag, const u32x4* b
     return launch_hilo_gemm<4, 4>(ctx, afrag, bfrag, isc, c, m, n, k, accumulate);
 }
 
+// ---- Q6_K path: weights unpacked in the kernel, two matrix instructions per k-step -----------------------
+// w[n, 256 b + e] = d * sc_g * (q - 32) with q in 0..63, sc_g an int8 (one per sixteen elements), d fp16.  The integer
+// sc_g (q - 32) needs thirteen bits, two more than an fp16 operand holds, so the scale is split, sc = 16 s1 + s0 with
+// s0 in 0..15 and s1 in -8..7: (q - 32) s1 and (q - 32) s0 / 16 are exact fp16 numbers, each goes through the matrix
+// core into the same accumulator, which then holds sum a sc (q - 32) / 16 of the superblock; at its end 16 d times
+// that is added to the tile's running total and the accumulator starts again from zero (the first matrix instruction
+// of a superblock takes no addend).  A quant is put together in place as the fp16 number 1024 + q (0x6400 | q: the
+// low four bits masked out of ql, the two high bits out of qh shifted beside them), a pair per register, and one
+// packed fused multiply-add per part, (1024 + q) s - 1056 s, makes the operand: the product is exact inside the
+// instruction and 1056 s = 33 s 2^5 is an fp16 number, so nothing is rounded before the fp32 accumulation.
+// Workgroup of four wavefronts, one per SIMD, tile (32 MT) x 64 as in the general path below: wavefront kq takes
+// superblocks kq, kq + 4, ... of all the tile and the four partial tiles are added through LDS at the end.  The
+// activations come in the fragment order of the Q4_K path; the element order inside a k-step -- 4 dw + {0, 2},
+// 32 + 4 dw + {0, 2}, 4 dw + {1, 3}, 32 + 4 dw + {1, 3} with dw = 4 h + s in a chunk of 64 -- is the one Q6_K's own
+// layout hands out: inside a half of 128 elements, element 32 Q + l has its low bits in nibble Q / 2 of byte
+// 32 (Q % 2) + l of ql and its high bits at 2 Q of byte l of qh, so chunk c of the superblock (quarters 2 (c % 2) and
+// 2 (c % 2) + 1 of half c / 2) takes dword s of three sixteen-byte pieces per lane -- ql + 64 (c / 2) + 16 h, the same
+// + 32, qh + 32 (c / 2) + 16 h -- shifted right by 4 (c % 2).  Each lane reads the pieces of its own weight row (32
+// rows per request, 210 bytes per superblock, no alignment beyond two bytes) straight into registers, half a
+// superblock ahead; nothing but the final exchange passes through LDS and the loop has no barrier.
+struct Q6kHalf {
+    u32x4 qa[2], qb[2], qh[2];  // per 32-column block: ql + 16 h, ql + 32 + 16 h, qh + 16 h of the half
+};
+
+template <int MT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void gemm_q6k_frag_kernel(const u32x4* __restrict__ afrag, const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
+                          float* __restrict__ c, int m, int n, int k, int m_tiles, int n_tiles, int accumulate,
+                          uint32_t a_bytes, uint32_t w_bytes, int xcd_rows) {
+    extern __shared__ __align__(16) float red[];  // 2 MT tiles x 3 copies x 1024 floats
+    const int lane = threadIdx.x & 63;
+    const int kq = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int h = lane >> 5, r = lane & 31;
+    // Workgroup -> tile.  The packed weights of a tile are small (53 KiB per 64 columns at k = 4096) beside the
+    // activations of its rows (1 MiB per 128 rows), so with up to eight row tiles an XCD (blockIdx % 8) keeps to one
+    // row tile, whose activations then stay in its L2 while the column tiles stream through.
+    int mt, tn;
+    if (xcd_rows) {
+        const int xcd = blockIdx.x & 7, per = 8 / m_tiles;
+        mt = xcd % m_tiles;
+        tn = (blockIdx.x >> 3) * per + xcd / m_tiles;
+    } else {
+        const int slot_in_xcd = blockIdx.x >> 3;
+        mt = slot_in_xcd % m_tiles;
+        tn = (slot_in_xcd / m_tiles) * 8 + (blockIdx.x & 7);
+    }
+    if (tn >= n_tiles) return;
+    const int nb = k >> 8, nch = k >> 6;
+    // The weights are read with buffer loads too: the lane's byte offset (its weight row, its sixteen-byte half) plus
+    // a scalar one (superblock, piece).  A piece of an odd superblock starts at an address that is only a multiple
+    // of two.
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
+    int wrow[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) wrow[j] = min(tn * kBN + 32 * j + r, n - 1) * nb * 210 + 16 * h;
+
+    const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void*)afrag, 0, (int)a_bytes, 0x00020000);
+    uint32_t abase[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) abase[i] = (uint32_t)(mt * MT + i) * (uint32_t)nch * 4096u;
+    constexpr int RING = 4;  // ring of k-steps, RING - 1 ahead (eight deep: the same time)
+    u32x4 a[RING][MT];
+    auto afetch = [&](int step, int slot) __attribute__((always_inline)) {  // step: 16 per superblock, absolute
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+            a[slot][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, lane * 16, (int)(abase[i] + (uint32_t)step * 1024u), 0));
+    };
+    auto wload = [&](int j, int off) __attribute__((always_inline)) {
+        return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow[j], off, 0));
+    };
+    auto load_half = [&](int sb, int hf, Q6kHalf& H) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            H.qa[j] = wload(j, sb * 210 + 64 * hf);
+            H.qb[j] = wload(j, sb * 210 + 64 * hf + 32);
+            H.qh[j] = wload(j, sb * 210 + 128 + 32 * hf);
+        }
+    };
+    // the sixteen scales of the superblock (both halves of the lanes read all of them: the lane's own sixteen-byte
+    // offset is taken back out) and its d, per column block
+    u32x4 scl[2], scl_n[2];
+    uint32_t dh[2], dh_n[2];
+    auto load_head = [&](int sb, u32x4 (&sc_out)[2], uint32_t (&d_out)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            sc_out[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow[j] - 16 * h, sb * 210 + 192, 0));
+            d_out[j] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(wrsrc, wrow[j] - 16 * h, sb * 210 + 208, 0);
+        }
+    };
+
+    float16_t acc[MT][2], total[MT][2];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) total[i][j][x] = 0.f;
+
+    Q6kHalf H0, H1;
+    if (kq < nb) {
+        load_head(kq, scl_n, dh_n);
+        load_half(kq, 0, H0);
+#pragma unroll
+        for (int s = 0; s < RING - 1; s++) afetch(16 * kq + s, s);
+    }
+    for (int sb = kq; sb < nb; sb += 4) {
+        const int sb_next = min(sb + 4, nb - 1);  // (past the end: a repeat of the last superblock, unused)
+        float dsc[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            scl[j] = scl_n[j];
+            dh[j] = dh_n[j];
+            dsc[j] = (float)__builtin_bit_cast(_Float16, (uint16_t)dh[j]) * 16.0f;
+        }
+        // one chunk of 64 elements = four k-steps; cc = 0..3, its half is cc / 2
+        auto chunk = [&](auto cc_const, const Q6kHalf& H) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            constexpr int par = cc & 1;
+            half2_t s0v[2][2], c0v[2][2], s1v[2][2], c1v[2][2];  // [column block][low 32 / high 32 of the chunk]
+            u32x4 qa[2], qb[2], qh[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                qa[j] = par ? H.qa[j] >> 4u : H.qa[j];
+                qb[j] = par ? H.qb[j] >> 4u : H.qb[j];
+                qh[j] = par ? H.qh[j] >> 4u : H.qh[j];
+                const uint32_t dw = scl[j][cc];  // scales 4 cc .. 4 cc + 3: the lane's groups are bytes h and 2 + h
+#pragma unroll
+                for (int g = 0; g < 2; g++) {
+                    const int sc = __builtin_amdgcn_sbfe((int)dw, (unsigned)(8 * h + 16 * g), 8u);
+                    const float f0 = (float)(sc & 15) * 0.0625f, f1 = (float)(sc >> 4);
+                    s0v[j][g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(f0, f0));  // (four bits and a power of two: exact)
+                    s1v[j][g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(f1, f1));
+                    c0v[j][g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(-1056.0f * f0, -1056.0f * f0));
+                    c1v[j][g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(-1056.0f * f1, -1056.0f * f1));
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                half8_t f0[2], f1[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const uint32_t x = qa[j][s], y = qb[j][s], z = qh[j][s];
+                    const uint32_t x8 = x >> 8, y8 = y >> 8, z8 = z >> 8;
+                    const half2_t t[4] = {
+                        __builtin_bit_cast(half2_t, ((z & 0x00030003u) << 4) | ((x & 0x000F000Fu) | 0x64006400u)),
+                        __builtin_bit_cast(half2_t, ((z & 0x000C000Cu) << 2) | ((y & 0x000F000Fu) | 0x64006400u)),
+                        __builtin_bit_cast(half2_t, ((z8 & 0x00030003u) << 4) | ((x8 & 0x000F000Fu) | 0x64006400u)),
+                        __builtin_bit_cast(half2_t, ((z8 & 0x000C000Cu) << 2) | ((y8 & 0x000F000Fu) | 0x64006400u))};
+                    u32x4 o0, o1;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        o0[e] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(t[e], s0v[j][e & 1], c0v[j][e & 1]));
+                        o1[e] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(t[e], s1v[j][e & 1], c1v[j][e & 1]));
+                    }
+                    f0[j] = __builtin_bit_cast(half8_t, o0);
+                    f1[j] = __builtin_bit_cast(half8_t, o1);
+                }
+                const int step = 4 * cc + s, slot = step & (RING - 1);
+                // (the two matrix instructions of a tile are kept eight apart; the first of a superblock takes no addend)
+                const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, f1[j], step == 0 ? zero : acc[i][j], 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, f0[j], acc[i][j], 0, 0, 0);
+                }
+                // the slot of step - 1 is free: refill it RING - 1 steps ahead
+                const int ahead = step + RING - 1;
+                afetch(ahead < 16 ? 16 * sb + ahead : 16 * sb_next + ahead - 16, ahead & (RING - 1));
+            }
+        };
+        load_half(sb, 1, H1);
+        chunk(std::integral_constant<int, 0>{}, H0);
+        chunk(std::integral_constant<int, 1>{}, H0);
+        load_head(sb_next, scl_n, dh_n);
+        load_half(sb_next, 0, H0);
+        chunk(std::integral_constant<int, 2>{}, H1);
+        chunk(std::integral_constant<int, 3>{}, H1);
+        // the superblock's sum, in units of 16 d, joins the total
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int x = 0; x < 16; x++) total[i][j][x] = fmaf(dsc[j], acc[i][j][x], total[i][j][x]);
+    }
+
+    // the four partial tiles: tile t = 2 i + j belongs to wavefront t % 4, the other three hand theirs over
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = 2 * i + j, owner = t & 3;
+            if (kq != owner) {
+                float* dst = red + (t * 3 + ((kq - owner + 4) & 3) - 1) * 1024 + lane;
+#pragma unroll
+                for (int x = 0; x < 16; x++) dst[64 * x] = total[i][j][x];
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = 2 * i + j;
+            if (kq == (t & 3)) {
+                float16_t sum = total[i][j];
+#pragma unroll
+                for (int o = 0; o < 3; o++)
+#pragma unroll
+                    for (int x = 0; x < 16; x++) sum[x] += red[(t * 3 + o) * 1024 + 64 * x + lane];
+                store_tile(sum, c, n, (mt * MT + i) * 32, tn * kBN + 32 * j, m, n, inv_scale, lane, accumulate != 0);
+            }
+        }
+}
+
+template <int MT>
+int launch_q6k_gemm(skn_ctx* ctx, const u32x4* afrag, const uint8_t* w, const float* isc, float* c, int m, int n, int k,
+                    int accumulate) {
+    constexpr int kLds = 2 * MT * 3 * 4096;
+    const int m_tiles = (m + 32 * MT - 1) / (32 * MT), n_tiles = (n + kBN - 1) / kBN;
+    const int xcd_rows = 8 % m_tiles == 0 ? 1 : 0;
+    const unsigned grid = xcd_rows ? (unsigned)(8 * ((n_tiles + 8 / m_tiles - 1) / (8 / m_tiles))) : (unsigned)(((n_tiles + 7) / 8) * 8 * m_tiles);
+    const uint32_t a_bytes = (uint32_t)((size_t)m_tiles * 32 * MT * k * 2);  // (checked by the caller to fit)
+    const uint32_t w_bytes = (uint32_t)((size_t)n * (k / 256) * 210);  // (checked by the caller to fit)
+    skn_launch(ctx, gemm_q6k_frag_kernel<MT>, dim3(grid), dim3(256), kLds, afrag, w, isc, c, m, n, k, m_tiles, n_tiles, accumulate,
+               a_bytes, w_bytes, xcd_rows);
+    SKN_LAUNCH_CHECK(ctx);
+    return SKN_OK;
+}
+
+int launch_q6k_gemm_mt(skn_ctx* ctx, int mt, const u32x4* afrag, const uint8_t* w, const float* isc, float* c, int m, int n,
+                       int k, int accumulate) {
+    if (mt == 1) return launch_q6k_gemm<1>(ctx, afrag, w, isc, c, m, n, k, accumulate);
+    if (mt == 2) return launch_q6k_gemm<2>(ctx, afrag, w, isc, c, m, n, k, accumulate);
+    return launch_q6k_gemm<4>(ctx, afrag, w, isc, c, m, n, k, accumulate);
+}
+
 // grows the context's GEMM workspace; the pointer stays valid until the next growth
 int gemm_workspace(skn_ctx* ctx, size_t bytes, uint8_t** out) {
     if (bytes > ctx->gemm_ws_bytes) {
@@ -853,6 +1099,9 @@ int skn_gemm_init(skn_ctx* ctx) {
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<2, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_frag_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_frag_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_frag_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
     return SKN_OK;
 }
 
@@ -938,8 +1187,11 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     const int mt = hilo_mt(m);
     const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt), n_pad = (n + kBN - 1) / kBN * kBN;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
+    // Q6_K with whole superblocks: the kernel that unpacks the blocks itself (no weight pass, no expanded copy)
+    const bool q6k_fused = ggml_type == SKN_TYPE_Q6_K && k % 256 == 0 && ctx->opt_gemm_q6k_fused != 0 && af_bytes < ((size_t)1 << 31) &&
+                           (size_t)n * (k / 256) * 210 < ((size_t)1 << 31);
     uint8_t* ws;
-    int rc = gemm_workspace(ctx, af_bytes + is_bytes + (size_t)n_pad * k * 4, &ws);
+    int rc = gemm_workspace(ctx, af_bytes + is_bytes + (q6k_fused ? 0 : (size_t)n_pad * k * 4), &ws);
     if (rc != SKN_OK) return rc;
     _Float16* afrag = (_Float16*)ws;
     float* isc = (float*)(ws + af_bytes);
@@ -948,6 +1200,7 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     _Float16* no_sums = nullptr;
     launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k);
     SKN_LAUNCH_CHECK(ctx);
+    if (q6k_fused) return launch_q6k_gemm_mt(ctx, mt, (const u32x4*)afrag, (const uint8_t*)w_dev, isc, c_dev, m, n, k, 0);
     rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;
     return launch_hilo_gemm_mt(ctx, mt, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k, 0);

@@ -171,6 +171,33 @@ def test_gemm_general_path_weight_magnitudes(hip):
         assert oracle_np.rel_err(got[:, col], want[:, col]) <= TOL, col
 
 
+@pytest.mark.parametrize("m,n,k", [(160, 100, 1280), (40, 64, 256), (512, 64, 2048)])
+def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
+    """Q6_K blocks as real files hold them: int8 scales over all of -128..127 (the benchmark's generator stops at
+    +-32), d of either sign, zero and subnormal d, superblock counts that do not divide by the four wavefronts that
+    share a tile's k; with and without the kernel that unpacks the blocks itself."""
+    rng = np.random.default_rng(1000 + k)
+    raw = synth.weight(Q6_K, n, k, seed=31).reshape(-1, 210).copy()
+    nblk = raw.shape[0]
+    raw[:, 192:208] = rng.integers(-128, 128, size=(nblk, 16), dtype=np.int8).view(np.uint8)
+    raw[::7, 192:208] = np.array([-128, 127, -1, 0, 15, 16, -16, -17] * 2, dtype=np.int8).view(np.uint8)
+    d = (rng.standard_normal(nblk) * 0.01).astype(np.float16)
+    d[::5] = 0.0
+    d[3::11] = np.float16(6e-8)  # the smallest subnormal
+    raw[:, 208:210] = d.view(np.uint8).reshape(-1, 2)
+    raw = raw.reshape(-1)
+    a = synth.activation_bf16((m, k), seed=m + 5)
+    want = oracle_c.gemm_q(Q6_K, raw, n, k, a, m)
+    for fused in (1, 0):
+        hip.set_option("gemm.q6k_fused", fused)
+        try:
+            got = hip.gemm_q_host(Q6_K, raw, n, k, a, m)
+        finally:
+            hip.set_option("gemm.q6k_fused", 1)
+        err = oracle_np.rel_err(got, want)
+        assert err <= TOL, f"fused={fused}: rel err {err}"
+
+
 @pytest.mark.parametrize("n", [4096, 14336])
 def test_gemm_benchmark_shapes_q6k(hip, n):
     """M=512, K=4096 with Q6_K weights (the mixed-precision prefill case), sampled columns."""
@@ -220,7 +247,8 @@ def test_gemm_full_width_slice(hip):
 def test_gemm_with_expanded_weights_equals_the_per_call_path(hip, qtype, m, n, k):
     """skn_gemm_expand + skn_gemm_expanded: the weight pass of the general path done once; same kernels, so the
     product equals skn_gemm_q's bit for bit for every other format, and the oracle's to the tolerance (also for Q4_K,
-    which skn_gemm_q multiplies on its own path).  The copy serves any number of products."""
+    which skn_gemm_q multiplies on its own path, as it does Q6_K unless the option gemm.q6k_fused is off: another order
+    of additions, so its bits are compared with the option off).  The copy serves any number of products."""
     raw = synth.weight(qtype, n, k, seed=21)
     w = hip.to_device(raw)
     assert hip.gemm_expanded_bytes(qtype, n, k) == (n + 63) // 64 * 64 * k * 4
@@ -234,7 +262,12 @@ def test_gemm_with_expanded_weights_equals_the_per_call_path(hip, qtype, m, n, k
         got = c.download(np.float32, m * n).reshape(m, n)
         assert oracle_np.rel_err(got, oracle_c.gemm_q(qtype, raw, n, k, a, m)) <= TOL
         if qtype != Q4_K:
-            assert np.array_equal(got.view(np.uint32), hip.gemm_q_host(qtype, raw, n, k, a, m).view(np.uint32))
+            hip.set_option("gemm.q6k_fused", 0)
+            try:
+                per_call = hip.gemm_q_host(qtype, raw, n, k, a, m)
+            finally:
+                hip.set_option("gemm.q6k_fused", 1)
+            assert np.array_equal(got.view(np.uint32), per_call.view(np.uint32))
         a_dev.free(), c.free()
     exp.free(), w.free()
 
