@@ -171,11 +171,11 @@ def test_gemm_general_path_weight_magnitudes(hip):
         assert oracle_np.rel_err(got[:, col], want[:, col]) <= TOL, col
 
 
-@pytest.mark.parametrize("m,n,k", [(160, 100, 1280), (40, 64, 256), (512, 64, 2048)])
+@pytest.mark.parametrize("m,n,k", [(160, 100, 1280), (40, 64, 256), (512, 64, 2048), (300, 200, 768)])
 def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     """Q6_K blocks as real files hold them: int8 scales over all of -128..127 (the benchmark's generator stops at
     +-32), d of either sign, zero and subnormal d, superblock counts that do not divide by the four wavefronts that
-    share a tile's k; with and without the kernel that unpacks the blocks itself."""
+    share a tile's k; with both forms of the kernel that unpacks the blocks itself and without it."""
     rng = np.random.default_rng(1000 + k)
     raw = synth.weight(Q6_K, n, k, seed=31).reshape(-1, 210).copy()
     nblk = raw.shape[0]
@@ -188,7 +188,7 @@ def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     raw = raw.reshape(-1)
     a = synth.activation_bf16((m, k), seed=m + 5)
     want = oracle_c.gemm_q(Q6_K, raw, n, k, a, m)
-    for fused in (1, 0):
+    for fused in (1, 2, 0):
         hip.set_option("gemm.q6k_fused", fused)
         try:
             got = hip.gemm_q_host(Q6_K, raw, n, k, a, m)
