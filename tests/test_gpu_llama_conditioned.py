@@ -222,3 +222,43 @@ def test_decode_across_the_split_boundaries_of_the_attention(hip, case, prompt_l
         model.free()
     finally:
         hip.set_option("llama.attn_wide", 1)
+
+
+_HEAD_DIMS = {
+    # eight heads of 64 (prompt attention and rotary pairs at the smaller head), four cached
+    "hd64": llama.Config(n_layer=2, hidden=512, ffn=768, n_head=8, n_kv_head=4, head_dim=64, vocab=512, max_tokens=96, page_tokens=16),
+    # two heads of 256: the prompt has no matrix-core attention at this size and takes the decode kernel, one query
+    # row per prompt token
+    "hd256": llama.Config(n_layer=2, hidden=512, ffn=768, n_head=2, n_kv_head=1, head_dim=256, vocab=512, max_tokens=96, page_tokens=16),
+}
+
+
+@pytest.mark.parametrize("splits", [0, 1])
+@pytest.mark.parametrize("name", list(_HEAD_DIMS))
+def test_other_head_sizes_prompt_then_decode(hip, name, splits):
+    """head_dim 64 and 256 through the prompt path and the decode path (the cases above are all 128): a prompt of 70
+    tokens -- two splits of the attention where the prompt takes the decode kernel -- and 24 steps, with the split count
+    the library chooses and with one."""
+    cfg = _HEAD_DIMS[name]
+    weights = llama.conditioned_weights(cfg, SEED)
+    ora = OracleLlama(cfg, weights)
+    prompt = tokens(70, cfg.vocab, seed=2)
+    ora.prefill(prompt, bf16_gemm=True)
+    first = ora.logits.copy()
+    toks = tokens(24, cfg.vocab, seed=4)
+    hip.set_option("attn.splits", splits)
+    try:
+        model = llama.LlamaModel(hip, cfg, weights=weights)
+        model.prefill(prompt)
+        worst = logit_err(model.logits(), first)
+        assert worst <= PROMPT_TOL, (name, "prompt", worst)
+        for i, t in enumerate(toks):
+            ora.step(t)
+            model.decode(t, 1)
+            err = logit_err(model.logits(), ora.logits)
+            worst = max(worst, err)
+            assert err <= PROMPT_TOL, (name, splits, i, err)
+        print(f"{name} splits={splits}: worst logit error {worst:.2e}")
+        model.free()
+    finally:
+        hip.set_option("attn.splits", 0)
