@@ -1332,7 +1332,8 @@ int launch_q6k_gemm(skn_ctx* ctx, const u32x4* afrag, const uint8_t* w, const fl
     const uint32_t a_bytes = (uint32_t)((size_t)m_tiles * 32 * MT * k * 2);  // (checked by the caller to fit)
     const uint32_t w_bytes = (uint32_t)((size_t)n * (k / 256) * 210);  // (checked by the caller to fit)
     // 128-row tiles: the kernel with specialised wavefronts (measured 6 - 11 % faster); option value 2 keeps to the other
-    if (MT == 4 && xcd_rows && ctx->opt_gemm_q6k_fused != 2) {
+    // (up to 16384 elements per row: a rescale per superblock rounds the accumulators once more, the other form does not)
+    if (MT == 4 && xcd_rows && k <= 16384 && ctx->opt_gemm_q6k_fused != 2) {
         skn_launch(ctx, gemm_q6k_pc_kernel, dim3(grid), dim3(512), kQ6PcLds, afrag, w, isc, c, m, n, k, m_tiles, n_tiles, accumulate,
                    a_bytes, w_bytes);
         SKN_LAUNCH_CHECK(ctx);
