@@ -692,6 +692,264 @@ int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfra
     return SKN_OK;
 }
 
+// ---- Q4_K path for wide weight matrices: a 256 x 128 tile, weights unpacked once for all its rows -------------
+// The arithmetic of gemm_q4k_frag_kernel with its two costs divided differently.  A workgroup of eight wavefronts
+// holds a 256 x 128 tile and walks k superblock by superblock.  Four consumers, one per SIMD, own 64 rows each --
+// a 64 x 128 tile per wavefront: an activation fragment feeds four matrix instructions instead of two, so the
+// activations a compute unit takes in per matrix instruction halve -- and four producers, their SIMD neighbours, own
+// 32 columns each: a producer unpacks the fragments of its columns once for all 256 rows (a quarter of the vector
+// instructions per matrix instruction of the other kernel) into LDS, one phase (a chunk of 64 elements, four k-steps)
+// ahead, two buffers, one bare barrier per phase; entering a superblock it leaves the min operands and the ratio by
+// which the accumulators change their unit beside them.  The consumers load their activation fragments themselves
+// (ring of eight k-steps), read the weight fragments one k-step ahead and issue the matrix instructions.  No split of
+// k, so no exchange at the end.
+constexpr int kTlStage = 4 * 4 * 1024;           // a phase: four k-steps x four column blocks x 1 KiB
+constexpr int kTlAux = 128 * 32 + 128 * 4;       // a superblock's min operands (128 columns x (hi, lo) x 16 B) and ratios
+constexpr int kTlLds = 2 * kTlStage + 2 * kTlAux + 128 * 4 + 256 * 4;
+
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const uint8_t* __restrict__ w,
+                          float* __restrict__ c, const float* __restrict__ inv_scale, int m, int n, int k, int m_tiles,
+                          int accumulate, uint32_t a_bytes, uint32_t w_bytes) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const int me = wave & 3;  // consumer: its 64 rows; producer: its 32 columns
+    const bool producer = wave >= 4;
+    const int h = lane >> 5, r = lane & 31;
+    const int nb = k >> 8, nch = k >> 6;
+    const int mt = blockIdx.x % m_tiles, tn = blockIdx.x / m_tiles;  // (the row tiles of a column tile run side by side)
+    const int n0 = tn * 128;
+    uint8_t* stage = lds;
+    uint8_t* aux = lds + 2 * kTlStage;
+    uint8_t* fin = aux + 2 * kTlAux;
+    float* isc_lds = reinterpret_cast<float*>(fin + 128 * 4);  // the scales of the tile's 256 rows, for the store at the end
+    if (tid < 256) isc_lds[tid] = inv_scale[mt * 256 + tid];
+    auto barrier = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+
+    if (producer) {
+        const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
+        const int col = 32 * me + r;  // column of the tile
+        const int wrow = min(n0 + col, n - 1) * nb * 144;
+        // One set of registers for the header and the four nibble pieces: piece x of superblock s is requested in
+        // phase (s - 1, x), unpacked in phase (s, x - 1) -- three phases later -- and replaced in phase (s, x).
+        u32x4 hd, q[4];
+        auto load_piece = [&](int sb, int cc) __attribute__((always_inline)) {
+            q[cc] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 144 + 16 + 32 * cc, 0));
+        };
+        auto load_header = [&](int sb) __attribute__((always_inline)) {
+            hd = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow, sb * 144, 0));
+        };
+        uint32_t sc4[2], mn4[2];
+        float sc_unit = 1.f, cs = 1.f;
+        auto byte_f = [](uint32_t word, int b) { return (float)((word >> (8 * b)) & 0xFFu); };
+        // header of the superblock in hd -> scales, mins, units; its ratio and min operands into aux[sb & 1]
+        auto enter = [&](int sb) __attribute__((always_inline)) {
+            uint8_t* ax = aux + (sb & 1) * kTlAux;
+            // (the header is taken up here and no earlier: without this the compiler computes on it, and waits for
+            // it, phases before)
+            asm volatile("" : "+v"(hd));
+            const uint32_t dw0 = hd[0], s0 = hd[1], s1 = hd[2], s2 = hd[3];
+            const half2_t dd = __builtin_bit_cast(half2_t, dw0);
+            const float d = (float)dd.x, dmin = (float)dd.y;
+            const bool live = d != 0.f;  // (a zero d: the products are zeroed)
+            sc4[0] = live ? s0 & 0x3F3F3F3Fu : 0u;
+            sc4[1] = live ? (s2 & 0x0F0F0F0Fu) | ((s0 >> 2) & 0x30303030u) : 0u;
+            mn4[0] = s1 & 0x3F3F3F3Fu;
+            mn4[1] = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
+            // (units, power pw and saturation as in gemm_q4k_frag_kernel)
+            const int e_d = (int)((__float_as_uint(d) >> 23) & 0xFFu), e_m = (int)((__float_as_uint(dmin) >> 23) & 0xFFu);
+            const int pw = live ? min(max(e_m - e_d - 10, 0), 10) : 0;
+            sc_unit = __uint_as_float((uint32_t)(127 + 10 - pw) << 23);
+            const float cs_new = live ? d * __uint_as_float((uint32_t)(127 + 14 + pw) << 23)
+                                      : (dmin != 0.f ? fabsf(dmin) * 512.0f : cs);
+            const float inv = 1.0f / cs_new, ratio = cs * inv;
+            const float min_unit = fminf(fmaxf(-dmin * inv * 4096.0f, -1023.f), 1023.f);
+            cs = cs_new;
+            if (h == 0) {
+                half8_t vh, vl;
+#pragma unroll
+                for (int x = 0; x < 8; x++) {
+                    _Float16 a, b;
+                    skn_split_hilo(min_unit * byte_f(mn4[x >> 2], x & 3), a, b);
+                    vh[x] = a, vl[x] = b;
+                }
+                *reinterpret_cast<half8_t*>(ax + col * 32) = vh;
+                *reinterpret_cast<half8_t*>(ax + col * 32 + 16) = vl;
+                *reinterpret_cast<float*>(ax + 128 * 32 + col * 4) = ratio;
+            }
+        };
+        // chunk cc of the superblock in q -> four k-steps of this producer's column block into buffer `buf`
+        auto unpack = [&](auto cc_const, int buf) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            uint8_t* dst = stage + buf * kTlStage + me * 1024 + lane * 16;
+            asm volatile("" : "+v"(q[cc]));  // (as for the header)
+            const float fl = byte_f(sc4[cc >> 1], 2 * (cc & 1)) * sc_unit;
+            const float fh = byte_f(sc4[cc >> 1], 2 * (cc & 1) + 1) * (sc_unit * 0.0625f);
+            const half2_t mul_lo = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(fl, fl));  // (six bits times a power of two: exact)
+            const half2_t mul_hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(fh, fh));
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+                const uint32_t qq = q[cc][s4], q8 = qq >> 8;
+                const uint32_t l02 = qq & 0x000F000Fu, h02 = qq & 0x00F000F0u;
+                const uint32_t l13 = q8 & 0x000F000Fu, h13 = q8 & 0x00F000F0u;
+                u32x4 o;
+                o.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l02) * mul_lo);
+                o.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h02) * mul_hi);
+                o.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, l13) * mul_lo);
+                o.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, h13) * mul_hi);
+                *reinterpret_cast<u32x4*>(dst + s4 * 4096) = o;
+            }
+        };
+        // while the consumers multiply phase (sb, cc): the request of the next superblock's piece cc (its header
+        // with piece 0), then the weights of the phase after this one
+        auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            const int sbn = min(sb + 1, nb - 1);  // (past the end: a repeat, unused)
+            if (cc == 0) load_header(sbn);
+            load_piece(sbn, cc);
+            if (cc < 3) {
+                unpack(std::integral_constant<int, (cc + 1) & 3>{}, (cc + 1) & 1);
+            } else {
+                // (after the last superblock this unpacks its repeat into buffers that nobody reads any more -- done
+                // without a branch so that the requests above are not moved down into one -- and the unit is kept)
+                const float keep = cs;
+                enter(sb + 1);
+                unpack(C0{}, 0);
+                if (sb + 1 >= nb) cs = keep;
+            }
+            barrier();
+        };
+        load_header(0);
+#pragma unroll
+        for (int x = 0; x < 4; x++) load_piece(0, x);
+        enter(0);
+        unpack(C0{}, 0);
+        barrier();
+        for (int sb = 0; sb < nb; sb++) {
+            phase(sb, C0{});
+            phase(sb, C1{});
+            phase(sb, C2{});
+            phase(sb, C3{});
+        }
+        // the unit the accumulators ended in
+        if (h == 0) *reinterpret_cast<float*>(fin + col * 4) = cs;
+        barrier();
+    } else {
+        constexpr int MT = 2;
+        const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void*)afrag, 0, (int)a_bytes, 0x00020000);
+        const int mb0 = mt * 8 + me * MT;  // first row block of this consumer
+        uint32_t abase[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) abase[i] = (uint32_t)(mb0 + i) * (uint32_t)nch * 4096u;
+        u32x4 a[8][MT];  // ring of eight k-steps, seven ahead
+        auto afetch = [&](int step, int slot) __attribute__((always_inline)) {  // step: absolute, 16 per superblock
+            step = min(step, 16 * nb - 1);  // (past the end: the last step again, unused)
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+                a[slot][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, lane * 16, (int)(abase[i] + (uint32_t)step * 1024u), 0));
+        };
+        float16_t acc[MT][4];
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
+        u32x4 sf[MT];
+        auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            const uint8_t* ax = aux + (sb & 1) * kTlAux;
+            float ratio[4];
+            if (cc == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) ratio[j] = *reinterpret_cast<const float*>(ax + 128 * 32 + (j * 32 + r) * 4);
+            }
+            if (cc == 0) {  // (the sub-block sums of the rows: needed three phases on)
+#pragma unroll
+                for (int i = 0; i < MT; i++) sf[i] = sfrag[((size_t)(mb0 + i) * nb + sb) * 64 + lane];
+            }
+            const uint8_t* src = stage + (cc & 1) * kTlStage + lane * 16;
+            // (the weight fragments of step s + 1 are read from LDS before the matrix instructions of step s are issued)
+            half8_t fb[2][4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(src + j * 1024);
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+                const int step = 4 * cc + s4, slot = step & 7;
+                if (s4 + 1 < 4) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) fb[(s4 + 1) & 1][j] = *reinterpret_cast<const half8_t*>(src + (s4 + 1) * 4096 + j * 1024);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (cc == 0 && s4 == 0) {
+                            // entering a superblock: the accumulators change their unit, tile by tile between the
+                            // matrix instructions of the first k-step
+#pragma unroll
+                            for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio[j];
+                        }
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[s4 & 1][j], acc[i][j], 0, 0, 0);
+                    }
+                }
+                afetch(16 * sb + step + 7, (step + 7) & 7);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (cc == 3) {  // the "- dmin * m" term of the superblock
+                half8_t vh[4], vl[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    vh[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32);
+                    vl[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32 + 16);
+                }
+                // (the two products of a tile eight instructions apart)
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sf[i]), vh[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sf[i]), vl[j], acc[i][j], 0, 0, 0);
+            }
+            barrier();
+        };
+#pragma unroll
+        for (int s = 0; s < 7; s++) afetch(s, s);
+        barrier();
+        for (int sb = 0; sb < nb; sb++) {
+            phase(sb, C0{});
+            phase(sb, C1{});
+            phase(sb, C2{});
+            phase(sb, C3{});
+        }
+        barrier();
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float sc[16];
+#pragma unroll
+            for (int x = 0; x < 16; x++) sc[x] = isc_lds[(me * MT + i) * 32 + 8 * (x >> 2) + 4 * h + (x & 3)];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float unit = *reinterpret_cast<const float*>(fin + (j * 32 + r) * 4);
+#pragma unroll
+                for (int x = 0; x < 16; x++) acc[i][j][x] *= unit;
+                store_tile_scaled(acc[i][j], c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, sc, lane, accumulate != 0);
+            }
+        }
+    }
+}
+
 // ---- general path: activations x (hi + lo * 2^-11) weights, both operands loaded in fragment order ---------
 // Workgroup of four wavefronts, one per SIMD, tile (32 MT) x 64.  The tile is not divided spatially: wavefront
 // kq computes all of it over a quarter of k (k is a multiple of 64, so the k-steps divide evenly) and the four
@@ -1379,6 +1637,7 @@ inline size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 int skn_gemm_init(skn_ctx* ctx) {
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 2>() + 32 * 2 * 2 * 4));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_frag_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, frag_lds_bytes<2, 1>() + 32 * 2 * 1 * 4));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q4k_tall_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kTlLds));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<2, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
@@ -1417,9 +1676,14 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     // staging per product, but the two wavefronts of a SIMD no longer meet at the same barriers (measured 4-11 %
     // faster on grids of several rounds, 3 % slower on single-round grids).
     const int n_tiles_all = fs.n_tiles;
-    const bool small_tiles = ctx->opt_gemm_tile == 1 ||
-                             (ctx->opt_gemm_tile == 0 && (m <= 128 || ((m + 127) / 128) * n_tiles_all > ctx->compute_units));
-    const int mt_rows = small_tiles ? 64 : 128;
+    // one matrix, wide enough that 256 x 128 tiles fill the machine: the kernel that unpacks the weights once per tile
+    const int tall_tiles = ((m + 255) / 256) * ((segs[0].n + 127) / 128);
+    const bool tall = nseg == 1 && !swiglu_pair && (size_t)segs[0].n * (k / 256) * 144 < ((size_t)1 << 31) &&
+                      (ctx->opt_gemm_tile == 3 || (ctx->opt_gemm_tile == 0 && m > 128 && 4 * tall_tiles >= 3 * ctx->compute_units &&
+                                                   tall_tiles <= ctx->compute_units));
+    const bool small_tiles = !tall && (ctx->opt_gemm_tile == 1 ||
+                             (ctx->opt_gemm_tile == 0 && (m <= 128 || ((m + 127) / 128) * n_tiles_all > ctx->compute_units)));
+    const int mt_rows = tall ? 256 : small_tiles ? 64 : 128;
     const int m_tiles = (m + mt_rows - 1) / mt_rows, m_pad = m_tiles * mt_rows;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), sf_bytes = align_up((size_t)m_pad * (k / 256) * 16 * 2);
     SKN_REQUIRE(ctx, af_bytes < ((size_t)1 << 31), SKN_ERR_SHAPE,
@@ -1438,6 +1702,14 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
         default: return skn_fail(ctx, SKN_ERR_ARG, "Q4_K GEMM: unknown activation source %d", src.kind);
     }
     SKN_LAUNCH_CHECK(ctx);
+    if (tall) {
+        const int n_tiles = (fs.n[0] + 127) / 128;
+        skn_launch(ctx, gemm_q4k_tall_kernel, dim3(m_tiles * n_tiles), dim3(512), kTlLds, (const u32x4*)afrag, (const u32x4*)sfrag, fs.w[0],
+                   fs.c[0], isc, m, fs.n[0], k, m_tiles, fs.accumulate[0], (uint32_t)((size_t)m_pad * k * 2),
+                   (uint32_t)((size_t)fs.n[0] * (k / 256) * 144));
+        SKN_LAUNCH_CHECK(ctx);
+        return SKN_OK;
+    }
     if (mt_rows == 128) return launch_frag<2, 2>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
     return launch_frag<2, 1>(ctx, m_tiles, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m, k);
 }

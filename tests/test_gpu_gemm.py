@@ -171,6 +171,23 @@ def test_gemm_general_path_weight_magnitudes(hip):
         assert oracle_np.rel_err(got[:, col], want[:, col]) <= TOL, col
 
 
+@pytest.mark.parametrize("m,n,k", [(512, 256, 4096), (200, 192, 11008), (130, 100, 768), (65, 64, 256), (300, 129, 1024), (1, 1, 256)])
+def test_gemm_q4k_wide_tile_kernel_on_small_and_ragged_shapes(hip, m, n, k):
+    """The Q4_K kernel with 256 x 128 tiles, which the library picks by itself only where such tiles fill the machine
+    (N = 14336 at M = 512: test_gemm_benchmark_shape_q4k_n14336), forced on shapes with partial tiles in both
+    directions and with 1, 3, 4, 16 and 43 superblocks per row."""
+    raw = synth.weight(Q4_K, n, k, seed=3 * n + k)
+    a = synth.activation_bf16((m, k), seed=m + 17)
+    want = oracle_c.gemm_q(Q4_K, raw, n, k, a, m)
+    hip.set_option("gemm.tile", 3)
+    try:
+        got = hip.gemm_q_host(Q4_K, raw, n, k, a, m)
+    finally:
+        hip.set_option("gemm.tile", 0)
+    err = oracle_np.rel_err(got, want)
+    assert err <= TOL, f"rel err {err}"
+
+
 @pytest.mark.parametrize("m,n,k", [(160, 100, 1280), (40, 64, 256), (512, 64, 2048), (300, 200, 768)])
 def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     """Q6_K blocks as real files hold them: int8 scales over all of -128..127 (the benchmark's generator stops at
