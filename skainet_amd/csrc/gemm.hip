@@ -1580,6 +1580,231 @@ void gemm_q6k_pc_kernel(const u32x4* __restrict__ afrag, const uint8_t* __restri
     }
 }
 
+// The same for wide weight matrices in the form of gemm_q4k_tall_kernel: a 256 x 128 tile, k walked superblock by
+// superblock by all eight wavefronts; four consumers own 64 rows each (a 64 x 128 tile per wavefront), four producers
+// 32 columns each, whose blocks they unpack once for all 256 rows into LDS (per k-step and column block the two
+// parts of the split scale as two fragments), a chunk of 64 elements ahead, two buffers, one bare barrier per chunk.
+// The consumers take the two parts one after the other (the same activation fragment, eight matrix instructions
+// each) and read the next half-step's four fragments from LDS while the current eight instructions run.
+// Accumulators in units of 16 d as in gemm_q6k_pc_kernel.
+constexpr int kQ6TlStage = 4 * 8 * 1024;          // a phase: four k-steps x (four column blocks x two parts) x 1 KiB
+constexpr int kQ6TlLds = 2 * kQ6TlStage + 2 * 128 * 4 + 128 * 4 + 256 * 4;
+
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
+                          float* __restrict__ c, int m, int n, int k, int m_tiles, int accumulate, uint32_t a_bytes,
+                          uint32_t w_bytes) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const int me = wave & 3;  // consumer: its 64 rows; producer: its 32 columns
+    const bool producer = wave >= 4;
+    const int h = lane >> 5, r = lane & 31;
+    const int nb = k >> 8, nch = k >> 6;
+    const int mt = blockIdx.x % m_tiles, tn = blockIdx.x / m_tiles;  // (the row tiles of a column tile run side by side)
+    const int n0 = tn * 128;
+    uint8_t* stage = lds;
+    float* ratios = reinterpret_cast<float*>(lds + 2 * kQ6TlStage);  // [superblock parity][128 columns]
+    float* fin = ratios + 2 * 128;                                   // the last unit of the 128 columns
+    float* isc_lds = fin + 128;                                      // the scales of the tile's 256 rows
+    if (tid < 256) isc_lds[tid] = inv_scale[mt * 256 + tid];
+    auto barrier = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+
+    if (producer) {
+        const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
+        const int col = 32 * me + r;
+        const int wrow = min(n0 + col, n - 1) * nb * 210;
+        u32x4 qa[2], qb[2], qh[2];  // [half of the superblock]: ql + 16 h, ql + 32 + 16 h, qh + 16 h
+        u32x4 scl, scl_n;
+        uint32_t dh_n = 0;
+        auto load_half = [&](int sb, int hf) __attribute__((always_inline)) {
+            qa[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 64 * hf, 0));
+            qb[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 64 * hf + 32, 0));
+            qh[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 128 + 32 * hf, 0));
+        };
+        auto load_head = [&](int sb) __attribute__((always_inline)) {
+            scl_n = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow, sb * 210 + 192, 0));
+            dh_n = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(wrsrc, wrow, sb * 210 + 208, 0);
+        };
+        float cs = 1.f;
+        bool live = true;
+        // entering superblock sb: its head becomes current, its ratio goes to ratios[sb & 1]
+        auto enter = [&](int sb) __attribute__((always_inline)) {
+            asm volatile("" : "+v"(scl_n), "+v"(dh_n));  // (taken up here and no earlier)
+            scl = scl_n;
+            const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)dh_n);
+            live = d != 0.f;  // (a zero d: the products are zeroed and the unit stays)
+            const float cs_new = live ? d * 16.0f : cs;
+            const float ratio = cs / cs_new;
+            cs = cs_new;
+            if (h == 0) ratios[(sb & 1) * 128 + col] = ratio;
+        };
+        // chunk cc of the current superblock -> four k-steps x two parts of this producer's column block into `buf`
+        auto unpack = [&](auto cc_const, int buf) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            constexpr int par = cc & 1, hf = cc >> 1;
+            uint8_t* dst = stage + buf * kQ6TlStage + me * 2048 + lane * 16;
+            asm volatile("" : "+v"(qa[hf]), "+v"(qb[hf]), "+v"(qh[hf]));  // (as for the head)
+            const u32x4 xa = par ? qa[hf] >> 4u : qa[hf], xb = par ? qb[hf] >> 4u : qb[hf], xh = par ? qh[hf] >> 4u : qh[hf];
+            half2_t s0v[2], c0v[2], s1v[2], c1v[2];  // [low 32 / high 32 of the chunk]
+            const uint32_t dw = scl[cc];  // scales 4 cc .. 4 cc + 3: the lane's groups are bytes h and 2 + h
+#pragma unroll
+            for (int g = 0; g < 2; g++) {
+                const int sc = live ? __builtin_amdgcn_sbfe((int)dw, (unsigned)(8 * h + 16 * g), 8u) : 0;
+                const float f0 = (float)(sc & 15) * 0.0625f, f1 = (float)(sc >> 4);
+                s0v[g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(f0, f0));  // (four bits and a power of two: exact)
+                s1v[g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(f1, f1));
+                c0v[g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(-1056.0f * f0, -1056.0f * f0));
+                c1v[g] = __builtin_bit_cast(half2_t, __builtin_amdgcn_cvt_pkrtz(-1056.0f * f1, -1056.0f * f1));
+            }
+#pragma unroll
+            for (int s4 = 0; s4 < 4; s4++) {
+                const uint32_t x = xa[s4], y = xb[s4], z = xh[s4];
+                const uint32_t x8 = x >> 8, y8 = y >> 8, z8 = z >> 8;
+                const half2_t t[4] = {
+                    __builtin_bit_cast(half2_t, ((z & 0x00030003u) << 4) | ((x & 0x000F000Fu) | 0x64006400u)),
+                    __builtin_bit_cast(half2_t, ((z & 0x000C000Cu) << 2) | ((y & 0x000F000Fu) | 0x64006400u)),
+                    __builtin_bit_cast(half2_t, ((z8 & 0x00030003u) << 4) | ((x8 & 0x000F000Fu) | 0x64006400u)),
+                    __builtin_bit_cast(half2_t, ((z8 & 0x000C000Cu) << 2) | ((y8 & 0x000F000Fu) | 0x64006400u))};
+                u32x4 o0, o1;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    o0[e] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(t[e], s0v[e & 1], c0v[e & 1]));
+                    o1[e] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(t[e], s1v[e & 1], c1v[e & 1]));
+                }
+                *reinterpret_cast<u32x4*>(dst + s4 * 8192) = o1;          // part 1: (q - 32) s1
+                *reinterpret_cast<u32x4*>(dst + s4 * 8192 + 1024) = o0;   // part 0: (q - 32) s0 / 16
+            }
+        };
+        // While the consumers multiply phase (sb, cc) the producer unpacks the phase after it.  Requests, two phases
+        // before their use: head and first half of the next superblock with chunk 2, its second half with its chunk 0.
+        auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            const int sbn = min(sb + 1, nb - 1);  // (past the end: a repeat, unused)
+            if (cc == 0) unpack(C1{}, 1);
+            if (cc == 1) {
+                load_head(sbn);
+                load_half(sbn, 0);
+                unpack(C2{}, 0);
+            }
+            if (cc == 2) unpack(C3{}, 1);
+            if (cc == 3) {
+                // (after the last superblock this unpacks its repeat into a buffer that nobody reads any more -- no
+                // branch, so that the requests above are not moved down into one -- and the unit is kept)
+                const float keep = cs;
+                enter(sb + 1);
+                load_half(sbn, 1);
+                unpack(C0{}, 0);
+                if (sb + 1 >= nb) cs = keep;
+            }
+            barrier();
+        };
+        load_head(0);
+        load_half(0, 0);
+        load_half(0, 1);
+        enter(0);
+        unpack(C0{}, 0);
+        barrier();
+        for (int sb = 0; sb < nb; sb++) {
+            phase(sb, C0{});
+            phase(sb, C1{});
+            phase(sb, C2{});
+            phase(sb, C3{});
+        }
+        if (h == 0) fin[col] = cs;
+        barrier();
+    } else {
+        constexpr int MT = 2;
+        const __amdgpu_buffer_rsrc_t arsrc = __builtin_amdgcn_make_buffer_rsrc((void*)afrag, 0, (int)a_bytes, 0x00020000);
+        const int mb0 = mt * 8 + me * MT;  // first row block of this consumer
+        uint32_t abase[MT];
+#pragma unroll
+        for (int i = 0; i < MT; i++) abase[i] = (uint32_t)(mb0 + i) * (uint32_t)nch * 4096u;
+        u32x4 a[8][MT];  // ring of eight k-steps, seven ahead
+        auto afetch = [&](int step, int slot) __attribute__((always_inline)) {  // step: absolute, 16 per superblock
+            step = min(step, 16 * nb - 1);  // (past the end: the last step again, unused)
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+                a[slot][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(arsrc, lane * 16, (int)(abase[i] + (uint32_t)step * 1024u), 0));
+        };
+        float16_t acc[MT][4];
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
+        auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
+            constexpr int cc = decltype(cc_const)::value;
+            float ratio[4];
+            if (cc == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) ratio[j] = ratios[(sb & 1) * 128 + j * 32 + r];
+            }
+            const uint8_t* src = stage + (cc & 1) * kQ6TlStage + lane * 16;
+            // half-step hs = 2 s4 + (part 1 first, then part 0): fragment (s4, j, pt) at (s4 * 8 + j * 2 + pt') KiB with
+            // pt' = 0 for part 1; the four fragments of half-step hs + 1 are read while those of hs are multiplied
+            half8_t fb[2][4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(src + j * 2048);
+#pragma unroll
+            for (int hs = 0; hs < 8; hs++) {
+                const int s4 = hs >> 1, step = 4 * cc + s4, slot = step & 7;
+                if (hs + 1 < 8) {
+                    const int s4n = (hs + 1) >> 1, ptn = (hs + 1) & 1;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) fb[(hs + 1) & 1][j] = *reinterpret_cast<const half8_t*>(src + s4n * 8192 + j * 2048 + ptn * 1024);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (cc == 0 && hs == 0) {
+                            // entering a superblock: the accumulators change their unit, tile by tile between the
+                            // matrix instructions of the first half-step
+#pragma unroll
+                            for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio[j];
+                        }
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[hs & 1][j], acc[i][j], 0, 0, 0);
+                    }
+                }
+                if (hs & 1) afetch(16 * sb + step + 7, (step + 7) & 7);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            barrier();
+        };
+#pragma unroll
+        for (int s = 0; s < 7; s++) afetch(s, s);
+        barrier();
+        for (int sb = 0; sb < nb; sb++) {
+            phase(sb, C0{});
+            phase(sb, C1{});
+            phase(sb, C2{});
+            phase(sb, C3{});
+        }
+        barrier();
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            float sc[16];
+#pragma unroll
+            for (int x = 0; x < 16; x++) sc[x] = isc_lds[(me * MT + i) * 32 + 8 * (x >> 2) + 4 * h + (x & 3)];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float unit = fin[j * 32 + r];
+#pragma unroll
+                for (int x = 0; x < 16; x++) acc[i][j][x] *= unit;
+                store_tile_scaled(acc[i][j], c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, sc, lane, accumulate != 0);
+            }
+        }
+    }
+}
+
 template <int MT>
 int launch_q6k_gemm(skn_ctx* ctx, const u32x4* afrag, const uint8_t* w, const float* isc, float* c, int m, int n, int k,
                     int accumulate) {
@@ -1641,6 +1866,7 @@ int skn_gemm_init(skn_ctx* ctx) {
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<1, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<2, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_hilo_frag_kernel<4, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 4 * 3 * 4096));
+    SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_tall_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kQ6TlLds));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_pc_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kQ6PcLds));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_frag_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 1 * 3 * 4096));
     SKN_HIP(ctx, hipFuncSetAttribute((const void*)gemm_q6k_frag_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * 2 * 3 * 4096));
@@ -1741,9 +1967,15 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     // the weights as an fp16 pair in fragment order (rows padded to whole 64-column tiles)
     SKN_REQUIRE(ctx, ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG, "skn_gemm_q: activations must be 8-byte aligned");
     const int mt = hilo_mt(m);
-    const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt), n_pad = (n + kBN - 1) / kBN * kBN;
+    // Q6_K with whole superblocks: the kernels that unpack the blocks themselves (no weight pass, no expanded copy);
+    // 256 x 128 tiles where they fill three quarters of the compute units or more in one round (or by option)
+    const int tall_tiles = ((m + 255) / 256) * ((n + 127) / 128);
+    const bool q6k_tall = ggml_type == SKN_TYPE_Q6_K && k % 256 == 0 && k <= 16384 && ctx->opt_gemm_q6k_fused == 1 &&
+                          (ctx->opt_gemm_tile == 3 || (ctx->opt_gemm_tile == 0 && m > 128 && 4 * tall_tiles >= 3 * ctx->compute_units &&
+                                                       tall_tiles <= ctx->compute_units));
+    const int m_rows = q6k_tall ? 256 : 32 * mt;
+    const int m_pad = (m + m_rows - 1) / m_rows * m_rows, n_pad = (n + kBN - 1) / kBN * kBN;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
-    // Q6_K with whole superblocks: the kernel that unpacks the blocks itself (no weight pass, no expanded copy)
     const bool q6k_fused = ggml_type == SKN_TYPE_Q6_K && k % 256 == 0 && ctx->opt_gemm_q6k_fused != 0 && af_bytes < ((size_t)1 << 31) &&
                            (size_t)n * (k / 256) * 210 < ((size_t)1 << 31);
     uint8_t* ws;
@@ -1756,6 +1988,13 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     _Float16* no_sums = nullptr;
     launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k);
     SKN_LAUNCH_CHECK(ctx);
+    if (q6k_fused && q6k_tall) {
+        const int m_tiles = m_pad / 256;
+        skn_launch(ctx, gemm_q6k_tall_kernel, dim3((unsigned)tall_tiles), dim3(512), kQ6TlLds, (const u32x4*)afrag, (const uint8_t*)w_dev,
+                   (const float*)isc, c_dev, m, n, k, m_tiles, 0, (uint32_t)((size_t)m_pad * k * 2), (uint32_t)((size_t)n * (k / 256) * 210));
+        SKN_LAUNCH_CHECK(ctx);
+        return SKN_OK;
+    }
     if (q6k_fused) return launch_q6k_gemm_mt(ctx, mt, (const u32x4*)afrag, (const uint8_t*)w_dev, isc, c_dev, m, n, k, 0);
     rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;

@@ -192,7 +192,7 @@ def test_gemm_q4k_wide_tile_kernel_on_small_and_ragged_shapes(hip, m, n, k):
 def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     """Q6_K blocks as real files hold them: int8 scales over all of -128..127 (the benchmark's generator stops at
     +-32), d of either sign, zero and subnormal d, superblock counts that do not divide by the four wavefronts that
-    share a tile's k; with both forms of the kernel that unpacks the blocks itself and without it."""
+    share a tile's k; with the three forms of the kernel that unpacks the blocks itself and without it."""
     rng = np.random.default_rng(1000 + k)
     raw = synth.weight(Q6_K, n, k, seed=31).reshape(-1, 210).copy()
     nblk = raw.shape[0]
@@ -205,14 +205,16 @@ def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     raw = raw.reshape(-1)
     a = synth.activation_bf16((m, k), seed=m + 5)
     want = oracle_c.gemm_q(Q6_K, raw, n, k, a, m)
-    for fused in (1, 2, 0):
+    for fused, tile in ((1, 0), (1, 3), (2, 0), (0, 0)):  # (tile 3: the 256 x 128 form, otherwise for wide matrices only)
         hip.set_option("gemm.q6k_fused", fused)
+        hip.set_option("gemm.tile", tile)
         try:
             got = hip.gemm_q_host(Q6_K, raw, n, k, a, m)
         finally:
             hip.set_option("gemm.q6k_fused", 1)
+            hip.set_option("gemm.tile", 0)
         err = oracle_np.rel_err(got, want)
-        assert err <= TOL, f"fused={fused}: rel err {err}"
+        assert err <= TOL, f"fused={fused} tile={tile}: rel err {err}"
 
 
 @pytest.mark.parametrize("n", [4096, 14336])
