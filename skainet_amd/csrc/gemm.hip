@@ -698,14 +698,18 @@ int launch_frag(skn_ctx* ctx, int m_tiles, const u32x4* afrag, const u32x4* sfra
 // a 64 x 128 tile per wavefront: an activation fragment feeds four matrix instructions instead of two, so the
 // activations a compute unit takes in per matrix instruction halve -- and four producers, their SIMD neighbours, own
 // 32 columns each: a producer unpacks the fragments of its columns once for all 256 rows (a quarter of the vector
-// instructions per matrix instruction of the other kernel) into LDS, one phase (a chunk of 64 elements, four k-steps)
-// ahead, two buffers, one bare barrier per phase; entering a superblock it leaves the min operands and the ratio by
-// which the accumulators change their unit beside them.  The consumers load their activation fragments themselves
-// (ring of eight k-steps), read the weight fragments one k-step ahead and issue the matrix instructions.  No split of
-// k, so no exchange at the end.
+// instructions per matrix instruction of the other kernel) into LDS, two phases (a phase: a chunk of 64 elements,
+// four k-steps) ahead of the consumers, three buffers, one bare barrier per phase; entering a superblock it leaves
+// the min operands and the ratio by which the accumulators change their unit beside them.  The consumers load their
+// activation fragments themselves (ring of eight k-steps), read the weight fragments one k-step ahead -- across the
+// barrier too: what the next phase starts with was complete a phase ago -- and issue the matrix instructions; the
+// change of unit between two superblocks is spread between the matrix instructions around it.  No split of k, so no
+// exchange at the end.  (Timed in the kernel, the loop of one workgroup alone on the device takes as many core clocks
+// as with all 224 -- nothing shared between compute units holds it -- but the core clock falls from 2.39 GHz to
+// 1.8 - 1.9 GHz with all compute units at this work.)
 constexpr int kTlStage = 4 * 4 * 1024;           // a phase: four k-steps x four column blocks x 1 KiB
 constexpr int kTlAux = 128 * 32 + 128 * 4;       // a superblock's min operands (128 columns x (hi, lo) x 16 B) and ratios
-constexpr int kTlLds = 2 * kTlStage + 2 * kTlAux + 128 * 4 + 256 * 4;
+constexpr int kTlLds = 3 * kTlStage + 2 * kTlAux + 128 * 4 + 256 * 4;
 
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const uint8_t* __restrict__ w,
@@ -721,7 +725,7 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     const int mt = blockIdx.x % m_tiles, tn = blockIdx.x / m_tiles;  // (the row tiles of a column tile run side by side)
     const int n0 = tn * 128;
     uint8_t* stage = lds;
-    uint8_t* aux = lds + 2 * kTlStage;
+    uint8_t* aux = lds + 3 * kTlStage;
     uint8_t* fin = aux + 2 * kTlAux;
     float* isc_lds = reinterpret_cast<float*>(fin + 128 * 4);  // the scales of the tile's 256 rows, for the store at the end
     if (tid < 256) isc_lds[tid] = inv_scale[mt * 256 + tid];
@@ -730,18 +734,27 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     using C1 = std::integral_constant<int, 1>;
     using C2 = std::integral_constant<int, 2>;
     using C3 = std::integral_constant<int, 3>;
+    // the three buffers in turn: phase p is multiplied from b_cur, phase p + 1 lies complete in b_nxt, phase p + 2 is
+    // being written to b_nx2 (byte offsets, uniform)
+    int b_cur = 0, b_nxt = kTlStage, b_nx2 = 2 * kTlStage;
+    auto turn = [&]() __attribute__((always_inline)) {
+        const int t = b_cur;
+        b_cur = b_nxt, b_nxt = b_nx2, b_nx2 = t;
+    };
 
     if (producer) {
         const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
         const int col = 32 * me + r;  // column of the tile
         const int wrow = min(n0 + col, n - 1) * nb * 144;
-        // One set of registers for the header and the four nibble pieces: piece x of superblock s is requested in
-        // phase (s - 1, x), unpacked in phase (s, x - 1) -- three phases later -- and replaced in phase (s, x).
+        // One set of registers for the header and the four nibble pieces; each is requested again, for the next
+        // superblock, right after it is unpacked: four phases before its next use.
         u32x4 hd, q[4];
         auto load_piece = [&](int sb, int cc) __attribute__((always_inline)) {
+            sb = min(sb, nb - 1);  // (past the end: a repeat, unused)
             q[cc] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 144 + 16 + 32 * cc, 0));
         };
         auto load_header = [&](int sb) __attribute__((always_inline)) {
+            sb = min(sb, nb - 1);
             hd = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow, sb * 144, 0));
         };
         uint32_t sc4[2], mn4[2];
@@ -783,10 +796,10 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 *reinterpret_cast<float*>(ax + 128 * 32 + col * 4) = ratio;
             }
         };
-        // chunk cc of the superblock in q -> four k-steps of this producer's column block into buffer `buf`
+        // chunk cc of the superblock in q -> four k-steps of this producer's column block into the buffer at `buf`
         auto unpack = [&](auto cc_const, int buf) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
-            uint8_t* dst = stage + buf * kTlStage + me * 1024 + lane * 16;
+            uint8_t* dst = stage + buf + me * 1024 + lane * 16;
             asm volatile("" : "+v"(q[cc]));  // (as for the header)
             const float fl = byte_f(sc4[cc >> 1], 2 * (cc & 1)) * sc_unit;
             const float fh = byte_f(sc4[cc >> 1], 2 * (cc & 1) + 1) * (sc_unit * 0.0625f);
@@ -805,30 +818,44 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
                 *reinterpret_cast<u32x4*>(dst + s4 * 4096) = o;
             }
         };
-        // while the consumers multiply phase (sb, cc): the request of the next superblock's piece cc (its header
-        // with piece 0), then the weights of the phase after this one
+        // While the consumers multiply phase (sb, cc) the producer unpacks the phase two after it -- chunks 2 and 3 of
+        // the superblock, then chunks 0 and 1 of the next, whose header it takes up with chunk 0 -- and requests the
+        // same piece of the superblock after that.  (After the last superblock it unpacks a repeat into buffers that
+        // nobody reads any more -- no branch, so that the requests are not moved down into one -- and keeps the unit.)
         auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
-            const int sbn = min(sb + 1, nb - 1);  // (past the end: a repeat, unused)
-            if (cc == 0) load_header(sbn);
-            load_piece(sbn, cc);
-            if (cc < 3) {
-                unpack(std::integral_constant<int, (cc + 1) & 3>{}, (cc + 1) & 1);
-            } else {
-                // (after the last superblock this unpacks its repeat into buffers that nobody reads any more -- done
-                // without a branch so that the requests above are not moved down into one -- and the unit is kept)
+            if (cc == 0) {
+                unpack(C2{}, b_nx2);
+                load_piece(sb + 1, 2);
+            }
+            if (cc == 1) {
+                unpack(C3{}, b_nx2);
+                load_piece(sb + 1, 3);
+            }
+            if (cc == 2) {
                 const float keep = cs;
                 enter(sb + 1);
-                unpack(C0{}, 0);
                 if (sb + 1 >= nb) cs = keep;
+                unpack(C0{}, b_nx2);
+                load_header(sb + 2);
+                load_piece(sb + 2, 0);
+            }
+            if (cc == 3) {
+                unpack(C1{}, b_nx2);
+                load_piece(sb + 2, 1);
             }
             barrier();
+            turn();
         };
         load_header(0);
 #pragma unroll
         for (int x = 0; x < 4; x++) load_piece(0, x);
         enter(0);
-        unpack(C0{}, 0);
+        unpack(C0{}, b_cur);
+        unpack(C1{}, b_nxt);
+        load_header(1);
+        load_piece(1, 0);
+        load_piece(1, 1);
         barrier();
         for (int sb = 0; sb < nb; sb++) {
             phase(sb, C0{});
@@ -861,72 +888,101 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
 #pragma unroll
                 for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
         u32x4 sf[MT];
+        half8_t fb[2][4];  // the weight fragments of a k-step, read while the step before it is multiplied; step 0 of a phase in fb[0]
+        float ratio[4] = {1.f, 1.f, 1.f, 1.f};  // of the superblock being entered, by column block
+        // tile t = 4 i + j changes its unit: half `part` of its sixteen registers
+        auto rescale = [&](int t, int part) __attribute__((always_inline)) {
+#pragma unroll
+            for (int x = 0; x < 8; x++) acc[t >> 2][t & 3][8 * part + x] *= ratio[t & 3];
+        };
+        auto fence = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
         auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
             const uint8_t* ax = aux + (sb & 1) * kTlAux;
-            float ratio[4];
-            if (cc == 0) {
-#pragma unroll
-                for (int j = 0; j < 4; j++) ratio[j] = *reinterpret_cast<const float*>(ax + 128 * 32 + (j * 32 + r) * 4);
-            }
+            const uint8_t* axn = aux + ((sb + 1) & 1) * kTlAux;
             if (cc == 0) {  // (the sub-block sums of the rows: needed three phases on)
 #pragma unroll
                 for (int i = 0; i < MT; i++) sf[i] = sfrag[((size_t)(mb0 + i) * nb + sb) * 64 + lane];
             }
-            const uint8_t* src = stage + (cc & 1) * kTlStage + lane * 16;
-            // (the weight fragments of step s + 1 are read from LDS before the matrix instructions of step s are issued)
-            half8_t fb[2][4];
+            const uint8_t* src = stage + b_cur + lane * 16;
+            const uint8_t* srcn = stage + b_nxt + lane * 16;
+            half8_t vh[4], vl[4];
+            float rnext[4];
+            if (cc == 3) {  // (the ratios of the next superblock, left by the producers a phase ago: used at the end of this phase)
 #pragma unroll
-            for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(src + j * 1024);
+                for (int j = 0; j < 4; j++) rnext[j] = *reinterpret_cast<const float*>(axn + 128 * 32 + (j * 32 + r) * 4);
+            }
 #pragma unroll
             for (int s4 = 0; s4 < 4; s4++) {
                 const int step = 4 * cc + s4, slot = step & 7;
-                if (s4 + 1 < 4) {
+                if (s4 < 3) {
 #pragma unroll
                     for (int j = 0; j < 4; j++) fb[(s4 + 1) & 1][j] = *reinterpret_cast<const half8_t*>(src + (s4 + 1) * 4096 + j * 1024);
+                } else if (cc < 3) {  // the next phase's first step: complete since the barrier before this phase
+#pragma unroll
+                    for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(srcn + j * 1024);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) vh[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+                fence();
+                if (cc == 0 && s4 == 0) {
+                    // the superblock's first step: tiles 3 .. 7 change their unit between its matrix instructions
+                    // (tiles 0 .. 2 did before the barrier)
 #pragma unroll
-                for (int i = 0; i < MT; i++) {
-                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+                    for (int t = 0; t < 8; t++) {
+                        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a[slot][t >> 2]), fb[0][t & 3],
+                                                                                    acc[t >> 2][t & 3], 0, 0, 0);
+                        fence();
+                        if (t < 4) rescale(3 + (t >> 1), t & 1);
+                        if (t >= 4 && t < 7) rescale(t + 1, 0), rescale(t + 1, 1);
+                        fence();
+                    }
+                } else {
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (cc == 0 && s4 == 0) {
-                            // entering a superblock: the accumulators change their unit, tile by tile between the
-                            // matrix instructions of the first k-step
+                    for (int i = 0; i < MT; i++) {
+                        const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
 #pragma unroll
-                            for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio[j];
-                        }
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[s4 & 1][j], acc[i][j], 0, 0, 0);
+                        for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[s4 & 1][j], acc[i][j], 0, 0, 0);
                     }
                 }
                 afetch(16 * sb + step + 7, (step + 7) & 7);
-                __builtin_amdgcn_sched_barrier(0);
+                fence();
             }
-            if (cc == 3) {  // the "- dmin * m" term of the superblock
-                half8_t vh[4], vl[4];
+            if (cc == 3) {
+                // The "- dmin * m" term of the superblock (the two products of a tile eight instructions apart), and
+                // under it the reads for what follows: the low parts, then the next phase's first step.
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    vh[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32);
-                    vl[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32 + 16);
-                }
-                // (the two products of a tile eight instructions apart)
+                for (int j = 0; j < 4; j++) vl[j] = *reinterpret_cast<const half8_t*>(ax + (j * 32 + r) * 32 + 16);
+                fence();
 #pragma unroll
                 for (int i = 0; i < MT; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sf[i]), vh[j], acc[i][j], 0, 0, 0);
+                fence();
 #pragma unroll
-                for (int i = 0; i < MT; i++)
+                for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(srcn + j * 1024);
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sf[i]), vl[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 4; j++) ratio[j] = sb + 1 < nb ? rnext[j] : 1.0f;  // (none after the last superblock)
+                fence();
+                // tiles 0 .. 2 change their unit between the last of these instructions
+#pragma unroll
+                for (int t = 0; t < 8; t++) {
+                    acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, sf[t >> 2]), vl[t & 3], acc[t >> 2][t & 3], 0, 0, 0);
+                    fence();
+                    if (t >= 2) rescale((t - 2) >> 1, t & 1);
+                    fence();
+                }
             }
             barrier();
+            turn();
         };
 #pragma unroll
         for (int s = 0; s < 7; s++) afetch(s, s);
         barrier();
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(stage + b_cur + lane * 16 + j * 1024);
         for (int sb = 0; sb < nb; sb++) {
             phase(sb, C0{});
             phase(sb, C1{});
@@ -1583,12 +1639,13 @@ void gemm_q6k_pc_kernel(const u32x4* __restrict__ afrag, const uint8_t* __restri
 // The same for wide weight matrices in the form of gemm_q4k_tall_kernel: a 256 x 128 tile, k walked superblock by
 // superblock by all eight wavefronts; four consumers own 64 rows each (a 64 x 128 tile per wavefront), four producers
 // 32 columns each, whose blocks they unpack once for all 256 rows into LDS (per k-step and column block the two
-// parts of the split scale as two fragments), a chunk of 64 elements ahead, two buffers, one bare barrier per chunk.
-// The consumers take the two parts one after the other (the same activation fragment, eight matrix instructions
-// each) and read the next half-step's four fragments from LDS while the current eight instructions run.
-// Accumulators in units of 16 d as in gemm_q6k_pc_kernel.
+// parts of the split scale as two fragments), two phases (chunks of 64 elements) ahead, three buffers, one bare
+// barrier per phase.  The consumers take the two parts one after the other (the same activation fragment, eight
+// matrix instructions each) and read the next half-step's four fragments from LDS, across the barrier too, while the
+// current eight instructions run.  Accumulators in units of 16 d as in gemm_q6k_pc_kernel, the change of unit spread
+// between the matrix instructions on both sides of a superblock's end.
 constexpr int kQ6TlStage = 4 * 8 * 1024;          // a phase: four k-steps x (four column blocks x two parts) x 1 KiB
-constexpr int kQ6TlLds = 2 * kQ6TlStage + 2 * 128 * 4 + 128 * 4 + 256 * 4;
+constexpr int kQ6TlLds = 3 * kQ6TlStage + 2 * 128 * 4 + 128 * 4 + 256 * 4;
 
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __restrict__ w, const float* __restrict__ inv_scale,
@@ -1604,7 +1661,7 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
     const int mt = blockIdx.x % m_tiles, tn = blockIdx.x / m_tiles;  // (the row tiles of a column tile run side by side)
     const int n0 = tn * 128;
     uint8_t* stage = lds;
-    float* ratios = reinterpret_cast<float*>(lds + 2 * kQ6TlStage);  // [superblock parity][128 columns]
+    float* ratios = reinterpret_cast<float*>(lds + 3 * kQ6TlStage);  // [superblock parity][128 columns]
     float* fin = ratios + 2 * 128;                                   // the last unit of the 128 columns
     float* isc_lds = fin + 128;                                      // the scales of the tile's 256 rows
     if (tid < 256) isc_lds[tid] = inv_scale[mt * 256 + tid];
@@ -1613,6 +1670,13 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
     using C1 = std::integral_constant<int, 1>;
     using C2 = std::integral_constant<int, 2>;
     using C3 = std::integral_constant<int, 3>;
+    // the three buffers in turn: phase p is multiplied from b_cur, phase p + 1 lies complete in b_nxt, phase p + 2 is
+    // being written to b_nx2 (byte offsets, uniform)
+    int b_cur = 0, b_nxt = kQ6TlStage, b_nx2 = 2 * kQ6TlStage;
+    auto turn = [&]() __attribute__((always_inline)) {
+        const int t = b_cur;
+        b_cur = b_nxt, b_nxt = b_nx2, b_nx2 = t;
+    };
 
     if (producer) {
         const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
@@ -1622,11 +1686,13 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
         u32x4 scl, scl_n;
         uint32_t dh_n = 0;
         auto load_half = [&](int sb, int hf) __attribute__((always_inline)) {
+            sb = min(sb, nb - 1);  // (past the end: a repeat, unused)
             qa[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 64 * hf, 0));
             qb[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 64 * hf + 32, 0));
             qh[hf] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow + 16 * h, sb * 210 + 128 + 32 * hf, 0));
         };
         auto load_head = [&](int sb) __attribute__((always_inline)) {
+            sb = min(sb, nb - 1);
             scl_n = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(wrsrc, wrow, sb * 210 + 192, 0));
             dh_n = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(wrsrc, wrow, sb * 210 + 208, 0);
         };
@@ -1643,11 +1709,11 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
             cs = cs_new;
             if (h == 0) ratios[(sb & 1) * 128 + col] = ratio;
         };
-        // chunk cc of the current superblock -> four k-steps x two parts of this producer's column block into `buf`
+        // chunk cc of the current superblock -> four k-steps x two parts of this producer's column block into the buffer at `buf`
         auto unpack = [&](auto cc_const, int buf) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
             constexpr int par = cc & 1, hf = cc >> 1;
-            uint8_t* dst = stage + buf * kQ6TlStage + me * 2048 + lane * 16;
+            uint8_t* dst = stage + buf + me * 2048 + lane * 16;
             asm volatile("" : "+v"(qa[hf]), "+v"(qb[hf]), "+v"(qh[hf]));  // (as for the head)
             const u32x4 xa = par ? qa[hf] >> 4u : qa[hf], xb = par ? qb[hf] >> 4u : qb[hf], xh = par ? qh[hf] >> 4u : qh[hf];
             half2_t s0v[2], c0v[2], s1v[2], c1v[2];  // [low 32 / high 32 of the chunk]
@@ -1680,34 +1746,36 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
                 *reinterpret_cast<u32x4*>(dst + s4 * 8192 + 1024) = o0;   // part 0: (q - 32) s0 / 16
             }
         };
-        // While the consumers multiply phase (sb, cc) the producer unpacks the phase after it.  Requests, two phases
+        // While the consumers multiply phase (sb, cc) the producer unpacks the phase two after it -- chunks 2 and 3 of
+        // the superblock, then chunks 0 and 1 of the next, whose head it takes up with chunk 0.  Requests, two phases
         // before their use: head and first half of the next superblock with chunk 2, its second half with its chunk 0.
+        // (After the last superblock it unpacks a repeat into buffers that nobody reads any more -- no branch, so
+        // that the requests are not moved down into one -- and keeps the unit.)
         auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
-            const int sbn = min(sb + 1, nb - 1);  // (past the end: a repeat, unused)
-            if (cc == 0) unpack(C1{}, 1);
-            if (cc == 1) {
-                load_head(sbn);
-                load_half(sbn, 0);
-                unpack(C2{}, 0);
+            if (cc == 0) {
+                load_head(sb + 1);
+                load_half(sb + 1, 0);
+                unpack(C2{}, b_nx2);
             }
-            if (cc == 2) unpack(C3{}, 1);
-            if (cc == 3) {
-                // (after the last superblock this unpacks its repeat into a buffer that nobody reads any more -- no
-                // branch, so that the requests above are not moved down into one -- and the unit is kept)
+            if (cc == 1) unpack(C3{}, b_nx2);
+            if (cc == 2) {
                 const float keep = cs;
                 enter(sb + 1);
-                load_half(sbn, 1);
-                unpack(C0{}, 0);
                 if (sb + 1 >= nb) cs = keep;
+                load_half(sb + 1, 1);
+                unpack(C0{}, b_nx2);
             }
+            if (cc == 3) unpack(C1{}, b_nx2);
             barrier();
+            turn();
         };
         load_head(0);
         load_half(0, 0);
         load_half(0, 1);
         enter(0);
-        unpack(C0{}, 0);
+        unpack(C0{}, b_cur);
+        unpack(C1{}, b_nxt);
         barrier();
         for (int sb = 0; sb < nb; sb++) {
             phase(sb, C0{});
@@ -1738,50 +1806,77 @@ void gemm_q6k_tall_kernel(const u32x4* __restrict__ afrag, const uint8_t* __rest
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int x = 0; x < 16; x++) acc[i][j][x] = 0.f;
+        // half-step hs = 2 s4 + (part 1 first, then part 0): fragment (s4, j, part) of a phase at (s4 * 8 + j * 2 + p) KiB
+        // with p = 0 for part 1; the four fragments of half-step hs + 1 are read while those of hs are multiplied,
+        // half-step 0 of a phase in fb[0]
+        half8_t fb[2][4];
+        float ratio[4] = {1.f, 1.f, 1.f, 1.f};  // of the superblock being entered, by column block
+        // tile t = 4 i + j changes its unit: half `part` of its sixteen registers
+        auto rescale = [&](int t, int part) __attribute__((always_inline)) {
+#pragma unroll
+            for (int x = 0; x < 8; x++) acc[t >> 2][t & 3][8 * part + x] *= ratio[t & 3];
+        };
+        auto fence = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
         auto phase = [&](int sb, auto cc_const) __attribute__((always_inline)) {
             constexpr int cc = decltype(cc_const)::value;
-            float ratio[4];
-            if (cc == 0) {
+            const uint8_t* src = stage + b_cur + lane * 16;
+            const uint8_t* srcn = stage + b_nxt + lane * 16;
+            float rnext[4];
+            if (cc == 3) {  // (the ratios of the next superblock, left by the producers a phase ago: used at the end of this phase)
 #pragma unroll
-                for (int j = 0; j < 4; j++) ratio[j] = ratios[(sb & 1) * 128 + j * 32 + r];
+                for (int j = 0; j < 4; j++) rnext[j] = ratios[((sb + 1) & 1) * 128 + j * 32 + r];
             }
-            const uint8_t* src = stage + (cc & 1) * kQ6TlStage + lane * 16;
-            // half-step hs = 2 s4 + (part 1 first, then part 0): fragment (s4, j, pt) at (s4 * 8 + j * 2 + pt') KiB with
-            // pt' = 0 for part 1; the four fragments of half-step hs + 1 are read while those of hs are multiplied
-            half8_t fb[2][4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(src + j * 2048);
 #pragma unroll
             for (int hs = 0; hs < 8; hs++) {
                 const int s4 = hs >> 1, step = 4 * cc + s4, slot = step & 7;
-                if (hs + 1 < 8) {
+                if (hs < 7) {
                     const int s4n = (hs + 1) >> 1, ptn = (hs + 1) & 1;
 #pragma unroll
                     for (int j = 0; j < 4; j++) fb[(hs + 1) & 1][j] = *reinterpret_cast<const half8_t*>(src + s4n * 8192 + j * 2048 + ptn * 1024);
+                } else {  // the next phase's first half-step: complete since the barrier before this phase
+#pragma unroll
+                    for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(srcn + j * 2048);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+                if (cc == 3 && hs == 7) {
 #pragma unroll
-                for (int i = 0; i < MT; i++) {
-                    const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+                    for (int j = 0; j < 4; j++) ratio[j] = sb + 1 < nb ? rnext[j] : 1.0f;  // (none after the last superblock)
+                }
+                fence();
+                if ((cc == 0 && hs == 0) || (cc == 3 && hs == 7)) {
+                    // the two sides of a superblock's end: tiles 0 .. 2 change their unit between the last matrix
+                    // instructions of the superblock, tiles 3 .. 7 between the first of the next
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        if (cc == 0 && hs == 0) {
-                            // entering a superblock: the accumulators change their unit, tile by tile between the
-                            // matrix instructions of the first half-step
-#pragma unroll
-                            for (int x = 0; x < 16; x++) acc[i][j][x] *= ratio[j];
+                    for (int t = 0; t < 8; t++) {
+                        acc[t >> 2][t & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a[slot][t >> 2]), fb[hs & 1][t & 3],
+                                                                                    acc[t >> 2][t & 3], 0, 0, 0);
+                        fence();
+                        if (cc == 3) {
+                            if (t >= 2) rescale((t - 2) >> 1, t & 1);
+                        } else {
+                            if (t < 4) rescale(3 + (t >> 1), t & 1);
+                            if (t >= 4 && t < 7) rescale(t + 1, 0), rescale(t + 1, 1);
                         }
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[hs & 1][j], acc[i][j], 0, 0, 0);
+                        fence();
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < MT; i++) {
+                        const half8_t fa = __builtin_bit_cast(half8_t, a[slot][i]);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb[hs & 1][j], acc[i][j], 0, 0, 0);
                     }
                 }
                 if (hs & 1) afetch(16 * sb + step + 7, (step + 7) & 7);
-                __builtin_amdgcn_sched_barrier(0);
+                fence();
             }
             barrier();
+            turn();
         };
 #pragma unroll
         for (int s = 0; s < 7; s++) afetch(s, s);
         barrier();
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[0][j] = *reinterpret_cast<const half8_t*>(stage + b_cur + lane * 16 + j * 2048);
         for (int sb = 0; sb < nb; sb++) {
             phase(sb, C0{});
             phase(sb, C1{});

@@ -192,7 +192,8 @@ def test_gemm_q4k_wide_tile_kernel_on_small_and_ragged_shapes(hip, m, n, k):
 def test_gemm_q6k_full_range_of_the_block_fields(hip, m, n, k):
     """Q6_K blocks as real files hold them: int8 scales over all of -128..127 (the benchmark's generator stops at
     +-32), d of either sign, zero and subnormal d, superblock counts that do not divide by the four wavefronts that
-    share a tile's k; with the three forms of the kernel that unpacks the blocks itself and without it."""
+    share a tile's k; with every form of the kernels that unpack the blocks themselves (128 x 64 or 256 x 128 tiles,
+    specialised wavefronts or not) and without them."""
     rng = np.random.default_rng(1000 + k)
     raw = synth.weight(Q6_K, n, k, seed=31).reshape(-1, 210).copy()
     nblk = raw.shape[0]
