@@ -711,10 +711,12 @@ constexpr int kTlStage = 4 * 4 * 1024;           // a phase: four k-steps x four
 constexpr int kTlAux = 128 * 32 + 128 * 4;       // a superblock's min operands (128 columns x (hi, lo) x 16 B) and ratios
 constexpr int kTlLds = 3 * kTlStage + 2 * kTlAux + 128 * 4 + 256 * 4;
 
+// One to three matrices per launch as in gemm_q4k_frag_kernel (tile0 counts 128-column tiles here); pair: a tile holds
+// the same 64 columns of the gate and the up matrix -- producers 0 and 1 unpack the gate's, 2 and 3 the up's, so a
+// consumer's column blocks 0, 1 and 2, 3 meet lane by lane in the store -- and stores silu(gate) * up into c[0].
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const uint8_t* __restrict__ w,
-                          float* __restrict__ c, const float* __restrict__ inv_scale, int m, int n, int k, int m_tiles,
-                          int accumulate, uint32_t a_bytes, uint32_t w_bytes) {
+void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restrict__ sfrag, const Q4kFragSegs segs,
+                          const float* __restrict__ inv_scale, int m, int k, int m_tiles, uint32_t a_bytes) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -723,7 +725,11 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     const int h = lane >> 5, r = lane & 31;
     const int nb = k >> 8, nch = k >> 6;
     const int mt = blockIdx.x % m_tiles, tn = blockIdx.x / m_tiles;  // (the row tiles of a column tile run side by side)
-    const int n0 = tn * 128;
+    const bool pair = segs.pair != 0;
+    const int seg = pair ? 0 : (tn >= segs.tile0[2] ? 2 : (tn >= segs.tile0[1] ? 1 : 0));
+    const int n = segs.n[seg];
+    const int n0 = pair ? tn * 64 : (tn - segs.tile0[seg]) * 128;  // first column of the tile in its matrix (pair: in both)
+    float* __restrict__ c = segs.c[seg];
     uint8_t* stage = lds;
     uint8_t* aux = lds + 3 * kTlStage;
     uint8_t* fin = aux + 2 * kTlAux;
@@ -743,9 +749,10 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
     };
 
     if (producer) {
-        const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)w_bytes, 0x00020000);
+        const uint8_t* w = segs.w[pair ? me >> 1 : seg];
+        const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, n * nb * 144, 0x00020000);  // (checked by the caller to fit)
         const int col = 32 * me + r;  // column of the tile
-        const int wrow = min(n0 + col, n - 1) * nb * 144;
+        const int wrow = min(n0 + (pair ? 32 * (me & 1) + r : col), n - 1) * nb * 144;
         // One set of registers for the header and the four nibble pieces; each is requested again, for the next
         // superblock, right after it is unpacked: four phases before its next use.
         u32x4 hd, q[4];
@@ -995,12 +1002,30 @@ void gemm_q4k_tall_kernel(const u32x4* __restrict__ afrag, const u32x4* __restri
             float sc[16];
 #pragma unroll
             for (int x = 0; x < 16; x++) sc[x] = isc_lds[(me * MT + i) * 32 + 8 * (x >> 2) + 4 * h + (x & 3)];
+            if (pair) {
+#pragma unroll
+                for (int jj = 0; jj < 2; jj++) {
+                    const float ug = *reinterpret_cast<const float*>(fin + (jj * 32 + r) * 4);
+                    const float uu = *reinterpret_cast<const float*>(fin + ((jj + 2) * 32 + r) * 4);
+                    const int col = n0 + 32 * jj + r;
+#pragma unroll
+                    for (int x = 0; x < 16; x++) {
+                        // register x of lane l: row 8 (x / 4) + 4 (l / 32) + x % 4 of the 32 x 32 tile
+                        const int row = (mb0 + i) * 32 + 8 * (x >> 2) + 4 * h + (x & 3);
+                        if (row < m && col < n) {
+                            const float g = acc[i][jj][x] * ug * sc[x], u = acc[i][jj + 2][x] * uu * sc[x];
+                            c[(size_t)row * n + col] = g / (1.0f + expf(-g)) * u;  // silu(gate) * up
+                        }
+                    }
+                }
+                continue;
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const float unit = *reinterpret_cast<const float*>(fin + (j * 32 + r) * 4);
 #pragma unroll
                 for (int x = 0; x < 16; x++) acc[i][j][x] *= unit;
-                store_tile_scaled(acc[i][j], c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, sc, lane, accumulate != 0);
+                store_tile_scaled(acc[i][j], c, n, (mb0 + i) * 32, n0 + 32 * j, m, n, sc, lane, segs.accumulate[seg] != 0);
             }
         }
     }
@@ -1997,11 +2022,21 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     // staging per product, but the two wavefronts of a SIMD no longer meet at the same barriers (measured 4-11 %
     // faster on grids of several rounds, 3 % slower on single-round grids).
     const int n_tiles_all = fs.n_tiles;
-    // one matrix, wide enough that 256 x 128 tiles fill the machine: the kernel that unpacks the weights once per tile
-    const int tall_tiles = ((m + 255) / 256) * ((segs[0].n + 127) / 128);
-    const bool tall = nseg == 1 && !swiglu_pair && (size_t)segs[0].n * (k / 256) * 144 < ((size_t)1 << 31) &&
-                      (ctx->opt_gemm_tile == 3 || (ctx->opt_gemm_tile == 0 && m > 128 && 4 * tall_tiles >= 3 * ctx->compute_units &&
-                                                   tall_tiles <= ctx->compute_units));
+    // 256 x 128 tiles (the kernel that unpacks the weights once per tile) where they keep at least two thirds of the
+    // compute units busy over their rounds: the 14336-column matrices, a q,k,v group and a gate / up pair at 512 rows
+    int tall_cols = 0, tall_tile0[3] = {0, 0, 0};
+    bool tall_fits = true;
+    for (int i = 0; i < nseg; i++) {
+        tall_tile0[i] = tall_cols;
+        tall_cols += (segs[i].n + 127) / 128;
+        tall_fits = tall_fits && (size_t)segs[i].n * (k / 256) * 144 < ((size_t)1 << 31);
+    }
+    for (int i = nseg; i < 3; i++) tall_tile0[i] = tall_cols;
+    if (swiglu_pair) tall_cols = (segs[0].n + 63) / 64;
+    const int tall_tiles = ((m + 255) / 256) * tall_cols;
+    const int tall_rounds = (tall_tiles + ctx->compute_units - 1) / ctx->compute_units;
+    const bool tall = tall_fits && (ctx->opt_gemm_tile == 3 ||
+                                    (ctx->opt_gemm_tile == 0 && m > 128 && 3 * tall_tiles >= 2 * tall_rounds * ctx->compute_units));
     const bool small_tiles = !tall && (ctx->opt_gemm_tile == 1 ||
                              (ctx->opt_gemm_tile == 0 && (m <= 128 || ((m + 127) / 128) * n_tiles_all > ctx->compute_units)));
     const int mt_rows = tall ? 256 : small_tiles ? 64 : 128;
@@ -2024,10 +2059,10 @@ int skn_gemm_q4k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, 
     }
     SKN_LAUNCH_CHECK(ctx);
     if (tall) {
-        const int n_tiles = (fs.n[0] + 127) / 128;
-        skn_launch(ctx, gemm_q4k_tall_kernel, dim3(m_tiles * n_tiles), dim3(512), kTlLds, (const u32x4*)afrag, (const u32x4*)sfrag, fs.w[0],
-                   fs.c[0], isc, m, fs.n[0], k, m_tiles, fs.accumulate[0], (uint32_t)((size_t)m_pad * k * 2),
-                   (uint32_t)((size_t)fs.n[0] * (k / 256) * 144));
+        for (int i = 0; i < 3; i++) fs.tile0[i] = tall_tile0[i];
+        fs.n_tiles = tall_cols;
+        skn_launch(ctx, gemm_q4k_tall_kernel, dim3(m_tiles * tall_cols), dim3(512), kTlLds, (const u32x4*)afrag, (const u32x4*)sfrag, fs, isc, m,
+                   k, m_tiles, (uint32_t)((size_t)m_pad * k * 2));
         SKN_LAUNCH_CHECK(ctx);
         return SKN_OK;
     }

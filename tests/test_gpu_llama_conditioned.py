@@ -85,6 +85,29 @@ def test_44_decode_steps_across_two_page_boundaries(hip, case, fused, graph):
         model.free()
 
 
+@pytest.mark.parametrize("case", ["q4_k", "q4_k_kv2", "q4_k_kv1", "mixed"])
+def test_prompt_with_the_wide_tile_gemm_forced(hip, case):
+    """The prompt's Q4_K products on 256 x 128 tiles, which the library otherwise picks from 129 rows on where they
+    fill the device: the q, k, v group with one launch over three matrices (of 512, 256 or 128 columns with grouped
+    K/V: tiles that end in another matrix's columns or past the last), the gate / up pair with SwiGLU in the store
+    (768 columns: twelve tiles of 64 + 64), the output and down projections with the residual added."""
+    cfg = CASES[case]
+    prompt, first, toks, want = _oracle_prompt(case, 41, 12)
+    hip.set_option("gemm.tile", 3)
+    try:
+        model = llama.LlamaModel(hip, cfg, weights=llama.conditioned_weights(cfg, SEED))
+        model.prefill(prompt)
+        err = logit_err(model.logits(), first)
+        assert err <= PROMPT_TOL, (case, "prompt", err)
+        for i, t in enumerate(toks[:4]):
+            model.decode(t, 1)
+            err = logit_err(model.logits(), want[i])
+            assert err <= PROMPT_TOL, (case, i, err)
+        model.free()
+    finally:
+        hip.set_option("gemm.tile", 0)
+
+
 @pytest.mark.parametrize("fused,graph", [(1, 1), (0, 0)])
 @pytest.mark.parametrize("case", list(CASES))
 def test_41_token_prompt_then_decode_steps(hip, case, fused, graph):
