@@ -247,6 +247,22 @@ def test_gemm_benchmark_shape_q4k_n14336(hip):
     assert err <= TOL, err
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_gemm_2000_rows_take_the_wide_tile_kernels_by_themselves(hip, t):
+    """M = 2000, N = 4096, K = 2048: eight row tiles x 32 column tiles of 256 x 128 fill the 256 compute units, so the
+    library picks the wide-tile kernels without being told; the last row tile has 208 rows.  Sampled columns."""
+    m, n, k = 2000, 4096, 2048
+    raw = synth.weight(t, n, k, seed=23)
+    a = synth.activation_bf16((m, k), seed=24)
+    got = hip.gemm_q_host(t, raw, n, k, a, m)
+    rows = np.arange(0, n, 61)
+    rb = raw.reshape(n, -1)[rows].reshape(-1)
+    want = oracle_c.gemm_q(t, rb, len(rows), k, a, m)
+    floor = 1e-3 * np.abs(got).max()
+    err = np.max(np.abs(got[:, rows] - want) / np.maximum(np.abs(want), floor))
+    assert err <= TOL, err
+
+
 def test_gemm_full_width_slice(hip):
     """The benchmark shape M=512, K=4096 at N=4096: checked on a strided sample of the oracle's columns."""
     m, n, k = 512, 4096, 4096
