@@ -1,5 +1,5 @@
-"""CPU checks of the arithmetic that the Q6_K GEMM kernels (csrc/gemm.hip: gemm_q6k_frag_kernel, gemm_q6k_pc_kernel)
-rest on: the split of the int8 scale into two parts whose products with a quant are exact fp16 numbers, the way a quant
+"""CPU checks of the arithmetic that the Q6_K GEMM kernels (csrc/gemm.hip: gemm_q6k_frag_kernel, gemm_q6k_pc_kernel,
+gemm_q6k_tall_kernel) rest on: the split of the int8 scale into two parts whose products with a quant are exact fp16 numbers, the way a quant
 is assembled in place as the fp16 number 1024 + q and turned into such a product by one fused multiply-add, and the
 map from (chunk, k-step, lane half, slot) of a matrix-core weight fragment to bytes and bits of a 210-byte block.
 The last is restated here in numpy and compared with the oracle's dequantization of the same block."""
