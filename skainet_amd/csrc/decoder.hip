@@ -6,6 +6,7 @@
 // index) from device memory, so that one captured HIP graph of the ~480 kernel launches of a step can be
 // replayed for every token.  The graph holds kernels only (no memset / memcpy nodes).
 #include "kv.h"
+#include "gemm_q6k.h"
 
 #include <algorithm>
 #include <cmath>
@@ -599,6 +600,45 @@ static int expanded_copy(skn_ctx* ctx, skn_llama* m, int l, int which, int type,
     return SKN_OK;
 }
 
+// Prompt rows times up to three matrices of any formats, one activation source (fp32 rows, with RMSNorm when norm_w
+// is given).  Q4_K and Q6_K matrices go behind the fused activation pass of their GEMMs -- the row-wise work inside
+// the pass, one pass per format, a residual (`accumulate`) in the store --, the others through a norm, a bf16
+// conversion, skn_gemm_q per matrix and an add.
+int project_rows(skn_ctx* ctx, skn_llama* m, const int* types, const void* const* blocks, const int* rows, float* const* outs,
+                 int count, int k, const float* x, const float* norm_w, int T, int accumulate) {
+    const skn_llama_config& c = m->cfg;
+    const skn_gemm_src src = {norm_w ? SKN_SRC_RMSNORM : SKN_SRC_F32, x, norm_w, norm_w ? c.rms_eps : 0.f};
+    skn_gemm_seg q4[3], q6[3];
+    int n4 = 0, n6 = 0;
+    bool plain = false;
+    for (int i = 0; i < count; i++) {
+        if (types[i] == SKN_TYPE_Q4_K && k <= 16384) q4[n4++] = {blocks[i], rows[i], outs[i], accumulate};
+        else if (types[i] == SKN_TYPE_Q6_K && skn_gemm_q6k_direct_ok(ctx, rows[i], k, T)) q6[n6++] = {blocks[i], rows[i], outs[i], accumulate};
+        else plain = true;
+    }
+    if (n4) SKN_TRY(skn_gemm_q4k_multi(ctx, q4, n4, k, src, T));
+    if (n6) SKN_TRY(skn_gemm_q6k_multi(ctx, q6, n6, k, src, T));
+    if (!plain) return SKN_OK;
+    if (norm_w) {
+        skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, x, norm_w, m->pxn, k, c.rms_eps);
+        SKN_LAUNCH_CHECK(ctx);
+    }
+    SKN_TRY(to_bf16(ctx, norm_w ? m->pxn : x, m->pb16, (int64_t)T * k));
+    for (int i = 0; i < count; i++) {
+        const bool fused = (types[i] == SKN_TYPE_Q4_K && k <= 16384) || (types[i] == SKN_TYPE_Q6_K && skn_gemm_q6k_direct_ok(ctx, rows[i], k, T));
+        if (fused) continue;
+        if (accumulate) {
+            SKN_TRY(skn_gemm_q(ctx, types[i], blocks[i], rows[i], k, m->pb16, T, m->pproj));
+            skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * rows[i])), dim3(256), 0, outs[i], (const float*)m->pproj,
+                       (int64_t)T * rows[i]);
+            SKN_LAUNCH_CHECK(ctx);
+        } else {
+            SKN_TRY(skn_gemm_q(ctx, types[i], blocks[i], rows[i], k, m->pb16, T, outs[i]));
+        }
+    }
+    return SKN_OK;
+}
+
 int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, int n_tokens, int32_t* next_token_host) {
     SKN_REQUIRE(nullptr, ctx != nullptr, SKN_ERR_ARG, "skn_llama_prefill: ctx is null");
     SKN_REQUIRE(ctx, m && tokens_host, SKN_ERR_ARG, "skn_llama_prefill: null pointer");
@@ -660,12 +700,10 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             if (n4) SKN_TRY(skn_gemm_q4k_multi(ctx, q4, n4, H, src, T));
             if (nx) SKN_TRY(skn_gemm_expanded_multi(ctx, ex, nx, H, src, T));
         } else {
-            skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.attn_norm, m->pxn, H, c.rms_eps);
-            SKN_LAUNCH_CHECK(ctx);
-            SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_q, L.wq, H, H, m->pb16, T, m->pq));
-            SKN_TRY(skn_gemm_q(ctx, L.type_k, L.wk, KVD, H, m->pb16, T, m->pk));
-            SKN_TRY(skn_gemm_q(ctx, L.type_v, L.wv, KVD, H, m->pb16, T, m->pv));
+            const int types[3] = {L.type_q, L.type_k, L.type_v}, rows[3] = {H, KVD, KVD};
+            const void* blocks[3] = {L.wq, L.wk, L.wv};
+            float* outs[3] = {m->pq, m->pk, m->pv};
+            SKN_TRY(project_rows(ctx, m, types, blocks, rows, outs, 3, H, m->px, L.attn_norm, T, 0));
         }
         skn_launch(ctx, rope_store_kernel, dim3(T, NH), dim3(D / 2), 0, m->pq, (const float*)m->pk, (const float*)m->pv,
                    kv->k_pool, kv->v_pool, (const int32_t*)kv->page_table_dev, (const int32_t*)(m->state + 1), NH, KVH, D,
@@ -686,11 +724,9 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             const skn_gemm_src src = {SKN_SRC_F32, m->patt, nullptr, 0.f};
             SKN_TRY(skn_gemm_expanded_multi(ctx, &wo, 1, H, src, T));
         } else {
-            SKN_TRY(to_bf16(ctx, m->patt, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_o, L.wo, H, H, m->pb16, T, m->pproj));
-            skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
-                       (int64_t)T * H);
-            SKN_LAUNCH_CHECK(ctx);
+            const void* blocks[1] = {L.wo};
+            float* outs[1] = {m->px};
+            SKN_TRY(project_rows(ctx, m, &L.type_o, blocks, &H, outs, 1, H, m->patt, nullptr, T, 1));
         }
         if (q4k_gu) {  // RMSNorm inside the activation pass, SwiGLU inside the store: gate and up never reach memory
             const skn_gemm_seg gu[2] = {{L.w_gate, F, m->pmid, 0}, {L.w_up, F, m->pmid, 0}};
@@ -714,11 +750,10 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
                        (const float*)m->pup, m->pmid, (int64_t)T * F);
             SKN_LAUNCH_CHECK(ctx);
         } else {
-            skn_launch(ctx, rmsnorm_rows_kernel, dim3(T), dim3(256), 0, (const float*)m->px, L.ffn_norm, m->pxn, H, c.rms_eps);
-            SKN_LAUNCH_CHECK(ctx);
-            SKN_TRY(to_bf16(ctx, m->pxn, m->pb16, (int64_t)T * H));
-            SKN_TRY(skn_gemm_q(ctx, L.type_gate, L.w_gate, F, H, m->pb16, T, m->pgate));
-            SKN_TRY(skn_gemm_q(ctx, L.type_up, L.w_up, F, H, m->pb16, T, m->pup));
+            const int types[2] = {L.type_gate, L.type_up}, rows[2] = {F, F};
+            const void* blocks[2] = {L.w_gate, L.w_up};
+            float* outs[2] = {m->pgate, m->pup};
+            SKN_TRY(project_rows(ctx, m, types, blocks, rows, outs, 2, H, m->px, L.ffn_norm, T, 0));
             skn_launch(ctx, swiglu_rows_kernel, dim3(nblk((int64_t)T * F)), dim3(256), 0, (const float*)m->pgate,
                        (const float*)m->pup, m->pmid, (int64_t)T * F);
             SKN_LAUNCH_CHECK(ctx);
@@ -733,11 +768,9 @@ int skn_llama_prefill(skn_ctx* ctx, skn_llama* m, const int32_t* tokens_host, in
             const skn_gemm_src mid = {SKN_SRC_F32, m->pmid, nullptr, 0.f};
             SKN_TRY(skn_gemm_expanded_multi(ctx, &down, 1, F, mid, T));
         } else {
-            SKN_TRY(to_bf16(ctx, m->pmid, m->pb16, (int64_t)T * F));
-            SKN_TRY(skn_gemm_q(ctx, L.type_down, L.w_down, H, F, m->pb16, T, m->pproj));
-            skn_launch(ctx, add_rows_kernel, dim3(nblk((int64_t)T * H)), dim3(256), 0, m->px, (const float*)m->pproj,
-                       (int64_t)T * H);
-            SKN_LAUNCH_CHECK(ctx);
+            const void* blocks[1] = {L.w_down};
+            float* outs[1] = {m->px};
+            SKN_TRY(project_rows(ctx, m, &L.type_down, blocks, &H, outs, 1, F, m->pmid, nullptr, T, 1));
         }
         // the cache of this layer now holds pos0 + T tokens
         kv->len[0] = pos0 + T;

@@ -17,6 +17,7 @@
 //     integers below 2^10, exact in fp16, so one MFMA per k-step suffices; the f16 superblock scale d is the
 //     unit in which a column's accumulators are kept.
 #include "common.h"
+#include "gemm_q6k.h"
 
 #include <type_traits>
 
@@ -2096,39 +2097,89 @@ extern "C" int skn_gemm_q(skn_ctx* ctx, int ggml_type, const void* w_dev, int n,
     // general path.  Workspace: activations in fragment order (rows padded to whole tiles) + row scales, then
     // the weights as an fp16 pair in fragment order (rows padded to whole 64-column tiles)
     SKN_REQUIRE(ctx, ((uintptr_t)a_bf16_dev & 7) == 0, SKN_ERR_ARG, "skn_gemm_q: activations must be 8-byte aligned");
+    const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
+    // Q6_K with whole superblocks: the kernels that unpack the blocks themselves (no weight pass, no expanded copy)
+    if (ggml_type == SKN_TYPE_Q6_K && skn_gemm_q6k_direct_ok(ctx, n, k, m)) {
+        const skn_gemm_seg seg = {w_dev, n, c_dev, 0};
+        return skn_gemm_q6k_multi(ctx, &seg, 1, k, src, m);
+    }
     const int mt = hilo_mt(m);
-    // Q6_K with whole superblocks: the kernels that unpack the blocks themselves (no weight pass, no expanded copy);
-    // 256 x 128 tiles where they fill three quarters of the compute units or more in one round (or by option)
-    const int tall_tiles = ((m + 255) / 256) * ((n + 127) / 128);
-    const bool q6k_tall = ggml_type == SKN_TYPE_Q6_K && k % 256 == 0 && k <= 16384 && ctx->opt_gemm_q6k_fused == 1 &&
-                          (ctx->opt_gemm_tile == 3 || (ctx->opt_gemm_tile == 0 && m > 128 && 4 * tall_tiles >= 3 * ctx->compute_units &&
-                                                       tall_tiles <= ctx->compute_units));
-    const int m_rows = q6k_tall ? 256 : 32 * mt;
-    const int m_pad = (m + m_rows - 1) / m_rows * m_rows, n_pad = (n + kBN - 1) / kBN * kBN;
+    const int m_pad = (m + 32 * mt - 1) / (32 * mt) * (32 * mt), n_pad = (n + kBN - 1) / kBN * kBN;
     const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
-    const bool q6k_fused = ggml_type == SKN_TYPE_Q6_K && k % 256 == 0 && ctx->opt_gemm_q6k_fused != 0 && af_bytes < ((size_t)1 << 31) &&
-                           (size_t)n * (k / 256) * 210 < ((size_t)1 << 31);
     uint8_t* ws;
-    int rc = gemm_workspace(ctx, af_bytes + is_bytes + (q6k_fused ? 0 : (size_t)n_pad * k * 4), &ws);
+    int rc = gemm_workspace(ctx, af_bytes + is_bytes + (size_t)n_pad * k * 4, &ws);
     if (rc != SKN_OK) return rc;
     _Float16* afrag = (_Float16*)ws;
     float* isc = (float*)(ws + af_bytes);
     uint8_t* bfrag = ws + af_bytes + is_bytes;
-    const skn_gemm_src src = {SKN_SRC_BF16, a_bf16_dev, nullptr, 0.f};
     _Float16* no_sums = nullptr;
     launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k);
     SKN_LAUNCH_CHECK(ctx);
-    if (q6k_fused && q6k_tall) {
-        const int m_tiles = m_pad / 256;
-        skn_launch(ctx, gemm_q6k_tall_kernel, dim3((unsigned)tall_tiles), dim3(512), kQ6TlLds, (const u32x4*)afrag, (const uint8_t*)w_dev,
-                   (const float*)isc, c_dev, m, n, k, m_tiles, 0, (uint32_t)((size_t)m_pad * k * 2), (uint32_t)((size_t)n * (k / 256) * 210));
-        SKN_LAUNCH_CHECK(ctx);
-        return SKN_OK;
-    }
-    if (q6k_fused) return launch_q6k_gemm_mt(ctx, mt, (const u32x4*)afrag, (const uint8_t*)w_dev, isc, c_dev, m, n, k, 0);
     rc = skn_weights_hilo_frag(ctx, ggml_type, (const uint8_t*)w_dev, n, k, bfrag);
     if (rc != SKN_OK) return rc;
     return launch_hilo_gemm_mt(ctx, mt, (const u32x4*)afrag, (const u32x4*)bfrag, isc, c_dev, m, n, k, 0);
+}
+
+namespace {
+// 256 x 128 tiles for a Q6_K matrix: where they fill three quarters of the compute units or more in one round (or by option)
+bool q6k_wide_tiles(const skn_ctx* ctx, int n, int k, int m) {
+    const int tiles = ((m + 255) / 256) * ((n + 127) / 128);
+    return k <= 16384 && ctx->opt_gemm_q6k_fused == 1 &&
+           (ctx->opt_gemm_tile == 3 ||
+            (ctx->opt_gemm_tile == 0 && m > 128 && 4 * tiles >= 3 * ctx->compute_units && tiles <= ctx->compute_units));
+}
+}  // namespace
+
+bool skn_gemm_q6k_direct_ok(const skn_ctx* ctx, int n, int k, int m) {
+    const size_t m_pad = ((size_t)m + 255) / 256 * 256;
+    return ctx->opt_gemm_q6k_fused != 0 && n > 0 && m > 0 && k > 0 && k % 256 == 0 && m_pad * k * 2 + 256 < ((size_t)1 << 31) &&
+           (size_t)n * (k / 256) * 210 < ((size_t)1 << 31);
+}
+
+int skn_gemm_q6k_multi(skn_ctx* ctx, const skn_gemm_seg* segs, int nseg, int k, const skn_gemm_src& src, int m) {
+    SKN_REQUIRE(ctx, nseg >= 1 && nseg <= 3 && m > 0, SKN_ERR_ARG, "Q6_K GEMM: bad segment count or shape");
+    SKN_REQUIRE(ctx, src.a && ((uintptr_t)src.a & (src.kind == SKN_SRC_BF16 ? 7 : 15)) == 0, SKN_ERR_ARG,
+                "Q6_K GEMM: activations are null or misaligned");
+    SKN_REQUIRE(ctx, src.kind == SKN_SRC_BF16 || src.kind == SKN_SRC_F32 || (src.b && ((uintptr_t)src.b & 15) == 0),
+                SKN_ERR_ARG, "Q6_K GEMM: second activation operand is null or misaligned");
+    bool any_wide = false;
+    for (int i = 0; i < nseg; i++) {
+        SKN_REQUIRE(ctx, segs[i].w && segs[i].c && skn_gemm_q6k_direct_ok(ctx, segs[i].n, k, m), SKN_ERR_ARG,
+                    "Q6_K GEMM: a matrix is null or not one this path takes");
+        any_wide = any_wide || q6k_wide_tiles(ctx, segs[i].n, k, m);
+    }
+    // (rows padded to the tallest tile in use: the kernels with shorter tiles address their own row blocks inside it)
+    const int mt = hilo_mt(m);
+    const int m_rows = any_wide ? 256 : 32 * mt;
+    const int m_pad = (m + m_rows - 1) / m_rows * m_rows;
+    const size_t af_bytes = align_up((size_t)m_pad * k * 2), is_bytes = align_up((size_t)m_pad * 4);
+    uint8_t* ws;
+    int rc = gemm_workspace(ctx, af_bytes + is_bytes, &ws);
+    if (rc != SKN_OK) return rc;
+    _Float16* afrag = (_Float16*)ws;
+    float* isc = (float*)(ws + af_bytes);
+    _Float16* no_sums = nullptr;
+    switch (src.kind) {
+        case SKN_SRC_BF16: launch_prep<SKN_SRC_BF16, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        case SKN_SRC_F32: launch_prep<SKN_SRC_F32, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        case SKN_SRC_RMSNORM: launch_prep<SKN_SRC_RMSNORM, false>(ctx, src, afrag, isc, no_sums, m, m_pad, k); break;
+        default: return skn_fail(ctx, SKN_ERR_ARG, "Q6_K GEMM: unknown activation source %d", src.kind);
+    }
+    SKN_LAUNCH_CHECK(ctx);
+    for (int i = 0; i < nseg; i++) {
+        const int n = segs[i].n;
+        if (q6k_wide_tiles(ctx, n, k, m)) {
+            const int m_tiles = m_pad / 256, tiles = m_tiles * ((n + 127) / 128);
+            skn_launch(ctx, gemm_q6k_tall_kernel, dim3((unsigned)tiles), dim3(512), kQ6TlLds, (const u32x4*)afrag, (const uint8_t*)segs[i].w,
+                       (const float*)isc, segs[i].c, m, n, k, m_tiles, segs[i].accumulate, (uint32_t)((size_t)m_pad * k * 2),
+                       (uint32_t)((size_t)n * (k / 256) * 210));
+            SKN_LAUNCH_CHECK(ctx);
+        } else {
+            rc = launch_q6k_gemm_mt(ctx, mt, (const u32x4*)afrag, (const uint8_t*)segs[i].w, isc, segs[i].c, m, n, k, segs[i].accumulate);
+            if (rc != SKN_OK) return rc;
+        }
+    }
+    return SKN_OK;
 }
 
 // ---- expanded weights: the general path with its weight pass done once ------------------------------------
